@@ -1,0 +1,74 @@
+"""ctypes binding of libbitlinear_hip.so (the C ABI in include/bitlinear_hip.h).
+
+The library is the only compute path: if it has not been built, loading
+raises -- there is no fallback.
+"""
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "lib", "libbitlinear_hip.so")
+
+_c_int = ctypes.c_int
+_c_ptr = ctypes.c_void_p
+
+# name -> (restype, argtypes); mirrors include/bitlinear_hip.h one to one
+SIGNATURES = {
+    "bitlinear_int8xint2": (None, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
+    "bitlinear_last_status": (_c_int, []),
+    "bitlinear_status_string": (ctypes.c_char_p, [_c_int]),
+    "bitlinear_ws_num": (_c_int, [_c_int, _c_int]),
+    "bitlinear_int8xint2_acc_i32": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    ),
+    "bitlinear_int8xint2_seg": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.POINTER(_c_int), _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
+    "bitlinear_quant_absmax": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
+    "bitlinear_forward_bf16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
+    "bitlinear_set_tuning": (_c_int, [_c_int, _c_int]),
+}
+
+_lib = None
+
+
+class BitLinearLibraryError(RuntimeError):
+    pass
+
+
+def load_library(path: str = None) -> ctypes.CDLL:
+    """Open the shared library and type its entry points.  Raises
+    BitLinearLibraryError when the .so is missing or lacks a symbol."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or os.environ.get("BITLINEAR_HIP_LIB", LIB_PATH)
+    if not os.path.exists(p):
+        raise BitLinearLibraryError(
+            f"{p} not found: build it with `python -m bitnet_amd.build` (hipcc, gfx950); there is no fallback path"
+        )
+    try:
+        lib = ctypes.CDLL(p)
+    except OSError as e:  # missing ROCm runtime, wrong arch, ...
+        raise BitLinearLibraryError(f"cannot load {p}: {e}") from e
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as e:
+            raise BitLinearLibraryError(f"{p} does not export {name}") from e
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load_library().bitlinear_status_string(status).decode()
+        raise BitLinearLibraryError(f"{what}: status {status} ({msg})")

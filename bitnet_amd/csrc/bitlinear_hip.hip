@@ -1,0 +1,391 @@
+// Ternary BitLinear for MI355X (gfx950 / CDNA4): hand-written HIP kernels and
+// the C ABI declared in include/bitlinear_hip.h.
+//
+// Data layout consumed in place (what gpu/pack_weight.py:76-98 of the reference
+// writes): 16 weight rows x 32 k form a 128-byte tile of 32 little-endian
+// int32 words; tiles of one 16-row block are contiguous over k (K words per
+// block).  Word t of a tile holds 16 consecutive k of row (t/16)*8 + t%8,
+// k-half (t/8)%2; element e of the word sits at bit (e%4)*8 + (e/4)*2, so
+// (word >> 2i) & 0x03030303 is elements 4i..4i+3 as four bytes.  Stored code
+// = w + 2.
+//
+// Decode GEMV (M <= 16 per workgroup): one workgroup owns one 16-row block and
+// one group of 16 tokens.  Its waves split K in steps of 64.  For one step a
+// lane loads ONE packed word (row lane%16, 16 k chosen by lane/16) -- the 64
+// lanes of a wave cover 256 contiguous bytes -- expands it to 16 int8 with 3
+// shifts + 4 ands, and that is exactly the A operand of
+// v_mfma_i32_16x16x64_i8.  The B operand is 16 int8 of token lane%16 for the
+// same 16 k.  The +2 bias of the stored codes is removed exactly by a second
+// MFMA whose A operand is the constant -2: sum((q-2)*a) = sum(q*a) + sum(-2*a).
+// Partial 16x16 tiles of the waves are summed through LDS and the reference's
+// epilogue (gpu/bitnet_kernels/bitnet_kernels.h:79-82) is applied.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "bitlinear_hip.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kMaxSeg = 8;
+constexpr int kMaxWaves = 16;
+
+struct ScaleMap {
+    int nseg;
+    int ends[kMaxSeg];
+};
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// ---------------------------------------------------------------------------
+// GEMV / small-M kernel
+// ---------------------------------------------------------------------------
+template <int UPW>
+__global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
+    int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
+    ScaleMap smap, int M, int N, int K) {
+    __shared__ int red[kMaxWaves * 256];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const int g = lane >> 4;  // which 16 of the step's 64 k
+    const int p = lane & 15;  // weight row (A operand) / token (B operand)
+    const int nb = blockIdx.x;
+    const int m0 = blockIdx.y * 16;
+    const int units = K >> 6;
+
+    // word of (row p, k-chunk g) inside a 64-k step: two tiles of 32 words
+    const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
+    const uint32_t* wrow = wq + (size_t)nb * K + lane_word;
+    const bool tok_ok = (m0 + p) < M;
+    const int8_t* arow = act + (size_t)(tok_ok ? (m0 + p) : 0) * K + g * 16;
+
+    v4i acc_q = {0, 0, 0, 0};
+    v4i acc_b = {0, 0, 0, 0};
+    const int neg2w = (int)0xFEFEFEFEu;
+    const v4i neg2 = {neg2w, neg2w, neg2w, neg2w};
+
+    for (int base = wave * UPW; base < units; base += nwaves * UPW) {
+        uint32_t w[UPW];
+        v4i b[UPW];
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            const int u = base + j;
+            const bool live = u < units;
+            w[j] = live ? __builtin_nontemporal_load(wrow + (size_t)u * 64) : 0u;
+            b[j] = (live && tok_ok) ? *(const v4i*)(arow + (size_t)u * 64) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            v4i a;
+            a.x = (int)(w[j] & 0x03030303u);
+            a.y = (int)((w[j] >> 2) & 0x03030303u);
+            a.z = (int)((w[j] >> 4) & 0x03030303u);
+            a.w = (int)((w[j] >> 6) & 0x03030303u);
+            acc_q = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[j], acc_q, 0, 0, 0);
+            acc_b = __builtin_amdgcn_mfma_i32_16x16x64_i8(neg2, b[j], acc_b, 0, 0, 0);
+        }
+    }
+
+    // lane holds token p, rows 4g + i in register i
+    int* my = red + wave * 256 + lane;
+    my[0] = acc_q.x + acc_b.x;
+    my[64] = acc_q.y + acc_b.y;
+    my[128] = acc_q.z + acc_b.z;
+    my[192] = acc_q.w + acc_b.w;
+    __syncthreads();
+
+    for (int t = threadIdx.x; t < 256; t += blockDim.x) {
+        const int l = t & 63;
+        const int m = m0 + (l & 15);
+        if (m >= M) continue;
+        int sum = 0;
+        for (int wv = 0; wv < nwaves; ++wv) sum += red[wv * 256 + t];
+        const int n = nb * 16 + 4 * (l >> 4) + (t >> 6);
+        if (acc_out) acc_out[(size_t)m * N + n] = sum;
+        if (out) {
+            int slot = 0;  // ends[] ascend, so the slot is the count of boundaries at or below n
+#pragma unroll
+            for (int j = 0; j < kMaxSeg - 1; ++j) slot += (j < smap.nseg - 1 && n >= smap.ends[j]) ? 1 : 0;
+            const float v = (float)sum / bf16_to_f32(s[m]) * bf16_to_f32(ws[slot]);
+            out[(size_t)m * N + n] = f32_to_bf16_rne(v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Per-token absmax quantizer: one workgroup per token row
+// ---------------------------------------------------------------------------
+constexpr int kQuantThreads = 256;
+constexpr int kQuantRegVecs = 4;  // 16-byte vectors (8 bf16) kept in registers per thread
+
+__device__ __forceinline__ uint32_t absmax_bits8(const uint4& v, uint32_t cur) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        cur = max(cur, d[i] & 0x7fffu);
+        cur = max(cur, (d[i] >> 16) & 0x7fffu);
+    }
+    return cur;
+}
+
+template <int MODE>
+__device__ __forceinline__ int quant_one(uint32_t bits16, float s32) {
+    const float x = __uint_as_float(bits16 << 16);
+    float pr = x * s32;
+    if (MODE == 1) pr = bf16_to_f32(f32_to_bf16_rne(pr));
+    const float r = fminf(fmaxf(rintf(pr), -128.0f), 127.0f);
+    return ((int)r) & 0xff;
+}
+
+template <int MODE>
+__device__ __forceinline__ uint2 quant_vec8(const uint4& v, float s32) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = (uint32_t)quant_one<MODE>(d[i] & 0xffffu, s32);
+        const uint32_t hi = (uint32_t)quant_one<MODE>(d[i] >> 16, s32);
+        o[i >> 1] |= (lo | (hi << 8)) << ((i & 1) * 16);
+    }
+    return make_uint2(o[0], o[1]);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint16_t* __restrict__ x,
+                                                                     int8_t* __restrict__ q,
+                                                                     uint16_t* __restrict__ s, int K) {
+    __shared__ uint32_t wmax[kQuantThreads / 64];
+    const int row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int nvec = K >> 3;
+    const uint4* xr = (const uint4*)(x + (size_t)row * K);
+    uint2* qr = (uint2*)(q + (size_t)row * K);
+
+    uint4 v[kQuantRegVecs];
+    uint32_t am = 0;
+#pragma unroll
+    for (int r = 0; r < kQuantRegVecs; ++r) {
+        const int idx = tid + r * kQuantThreads;
+        if (idx < nvec) {
+            v[r] = xr[idx];
+            am = absmax_bits8(v[r], am);
+        } else {
+            v[r] = make_uint4(0, 0, 0, 0);
+        }
+    }
+    for (int idx = tid + kQuantRegVecs * kQuantThreads; idx < nvec; idx += kQuantThreads)
+        am = absmax_bits8(xr[idx], am);
+
+    // |x| as bf16 bit patterns orders like the values, so the max is an integer max
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) am = max(am, (uint32_t)__shfl_xor((int)am, off));
+    if ((tid & 63) == 0) wmax[tid >> 6] = am;
+    __syncthreads();
+    am = wmax[0];
+#pragma unroll
+    for (int i = 1; i < kQuantThreads / 64; ++i) am = max(am, wmax[i]);
+
+    // torch evaluates 127 / t as t.reciprocal() * 127: a reciprocal, then a multiply
+    float amax = __uint_as_float(am << 16);
+    float s32;
+    if (MODE == 0) {
+        const float r = 1.0f / fmaxf(amax, 1e-5f);
+        s32 = bf16_to_f32(f32_to_bf16_rne(r * 127.0f));
+    } else {
+        amax = fmaxf(amax, bf16_to_f32(f32_to_bf16_rne(1e-5f)));
+        const float r = bf16_to_f32(f32_to_bf16_rne(1.0f / amax));
+        s32 = bf16_to_f32(f32_to_bf16_rne(r * 127.0f));
+    }
+    if (tid == 0) s[row] = f32_to_bf16_rne(s32);
+
+#pragma unroll
+    for (int r = 0; r < kQuantRegVecs; ++r) {
+        const int idx = tid + r * kQuantThreads;
+        if (idx < nvec) qr[idx] = quant_vec8<MODE>(v[r], s32);
+    }
+    for (int idx = tid + kQuantRegVecs * kQuantThreads; idx < nvec; idx += kQuantThreads)
+        qr[idx] = quant_vec8<MODE>(xr[idx], s32);
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+thread_local int g_status = BITLINEAR_OK;
+int g_tune_waves = 0;
+int g_tune_upw = 0;
+
+int set_status(int st) {
+    g_status = st;
+    return st;
+}
+
+struct ShapeWs {
+    int n, k, ws_num;
+};
+// (N, K) -> ws_num of the reference's template instances (bitnet_kernels.cu:4-33)
+const ShapeWs kShapeTable[] = {
+    {3840, 2560, 3},  {2560, 2560, 1},  {13824, 2560, 2}, {2560, 6912, 1},  {4800, 3200, 6},
+    {3200, 3200, 1},  {20480, 3200, 2}, {3200, 10240, 1}, {5120, 27648, 1}, {55296, 5120, 1},
+};
+
+bool shape_ok(int M, int N, int K) { return M >= 1 && N >= 16 && K >= 64 && (N % 16) == 0 && (K % 64) == 0; }
+
+void pick_launch(int K, int* waves, int* upw) {
+    const int units = K / 64;
+    int u = 1;
+    while (u < 16 && (units + u - 1) / u > kMaxWaves) u *= 2;
+    if (u < 4 && units >= 4 * 4) u = 4;  // keep a few loads in flight per wave
+    int w = (units + u - 1) / u;
+    if (w > kMaxWaves) w = kMaxWaves;
+    if (g_tune_waves > 0) {
+        w = g_tune_waves;
+        u = g_tune_upw;
+    }
+    *waves = w;
+    *upw = u;
+}
+
+int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
+                const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+    int waves, upw;
+    pick_launch(K, &waves, &upw);
+    const dim3 grid(N / 16, (M + 15) / 16, 1);
+    const dim3 block(waves * 64, 1, 1);
+    const uint32_t* wq = (const uint32_t*)packed;
+#define BITLINEAR_LAUNCH(U)                                                                                  \
+    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, M, N, K)
+    switch (upw) {
+        case 1: BITLINEAR_LAUNCH(1); break;
+        case 2: BITLINEAR_LAUNCH(2); break;
+        case 4: BITLINEAR_LAUNCH(4); break;
+        case 8: BITLINEAR_LAUNCH(8); break;
+        default: BITLINEAR_LAUNCH(16); break;
+    }
+#undef BITLINEAR_LAUNCH
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+ScaleMap equal_slots(int N, int ws_num) {
+    ScaleMap sm;
+    sm.nseg = ws_num;
+    for (int j = 0; j < kMaxSeg; ++j) sm.ends[j] = (j < ws_num) ? (j + 1) * (N / ws_num) : N;
+    sm.ends[ws_num - 1] = N;
+    return sm;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bitlinear_last_status(void) { return g_status; }
+
+const char* bitlinear_status_string(int status) {
+    switch (status) {
+        case BITLINEAR_OK: return "ok";
+        case BITLINEAR_ERR_SHAPE: return "unsupported shape (need M >= 1, N % 16 == 0, K % 64 == 0)";
+        case BITLINEAR_ERR_NULL: return "null pointer";
+        case BITLINEAR_ERR_LAUNCH: return "kernel launch failed";
+        case BITLINEAR_ERR_ARG: return "invalid argument";
+        default: return "unknown status";
+    }
+}
+
+int bitlinear_ws_num(int N, int K) {
+    for (const ShapeWs& e : kShapeTable)
+        if (e.n == N && e.k == K) return e.ws_num;
+    return 1;
+}
+
+int bitlinear_set_tuning(int waves_per_group, int ksteps_in_flight) {
+    if (waves_per_group == 0 && ksteps_in_flight == 0) {
+        g_tune_waves = g_tune_upw = 0;
+        return set_status(BITLINEAR_OK);
+    }
+    const int u = ksteps_in_flight;
+    if (waves_per_group < 1 || waves_per_group > kMaxWaves || !(u == 1 || u == 2 || u == 4 || u == 8 || u == 16))
+        return set_status(BITLINEAR_ERR_ARG);
+    g_tune_waves = waves_per_group;
+    g_tune_upw = u;
+    return set_status(BITLINEAR_OK);
+}
+
+int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1, int32_t* acc_out, uint16_t* output0,
+                                const uint16_t* s, const uint16_t* ws, int M, int N, int K, void* stream) {
+    if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
+    if (!input0 || !input1 || (!acc_out && !output0) || (output0 && (!s || !ws))) return set_status(BITLINEAR_ERR_NULL);
+    return set_status(launch_gemv(input0, input1, output0, acc_out, s, ws, equal_slots(N, bitlinear_ws_num(N, K)), M,
+                                  N, K, (hipStream_t)stream));
+}
+
+void bitlinear_int8xint2(int8_t* input0, int8_t* input1, uint16_t* output0, uint16_t* s, uint16_t* ws, int M, int N,
+                         int K, void* stream) {
+    if (!shape_ok(M, N, K)) {
+        // same line the reference prints for a shape it has no kernel for (bitnet_kernels.cu:35)
+        printf("required ladder gemm kernel: M %d, N %d, K %d\n", M, N, K);
+        fflush(stdout);
+        set_status(BITLINEAR_ERR_SHAPE);
+        return;
+    }
+    if (!input0 || !input1 || !output0 || !s || !ws) {
+        set_status(BITLINEAR_ERR_NULL);
+        return;
+    }
+    set_status(launch_gemv(input0, input1, output0, nullptr, s, ws, equal_slots(N, bitlinear_ws_num(N, K)), M, N, K,
+                           (hipStream_t)stream));
+}
+
+int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1, uint16_t* output0, const uint16_t* s,
+                            const uint16_t* ws, const int* seg_ends, int nseg, int M, int N, int K, void* stream) {
+    if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
+    if (!input0 || !input1 || !output0 || !s || !ws || !seg_ends) return set_status(BITLINEAR_ERR_NULL);
+    if (nseg < 1 || nseg > kMaxSeg) return set_status(BITLINEAR_ERR_ARG);
+    ScaleMap sm;
+    sm.nseg = nseg;
+    int prev = 0;
+    for (int j = 0; j < kMaxSeg; ++j) {
+        if (j < nseg) {
+            if (seg_ends[j] <= prev || seg_ends[j] > N) return set_status(BITLINEAR_ERR_ARG);
+            prev = seg_ends[j];
+        }
+        sm.ends[j] = (j < nseg) ? seg_ends[j] : N;
+    }
+    if (prev != N) return set_status(BITLINEAR_ERR_ARG);
+    return set_status(launch_gemv(input0, input1, output0, nullptr, s, ws, sm, M, N, K, (hipStream_t)stream));
+}
+
+int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s, int M, int K, int mode, void* stream) {
+    if (M < 1 || K < 8 || (K % 8) != 0) return set_status(BITLINEAR_ERR_SHAPE);
+    if (!x || !q || !s) return set_status(BITLINEAR_ERR_NULL);
+    if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
+    const dim3 grid(M, 1, 1), block(kQuantThreads, 1, 1);
+    if (mode == 0)
+        hipLaunchKernelGGL(quant_absmax_kernel<0>, grid, block, 0, (hipStream_t)stream, x, q, s, K);
+    else
+        hipLaunchKernelGGL(quant_absmax_kernel<1>, grid, block, 0, (hipStream_t)stream, x, q, s, K);
+    return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
+}
+
+int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
+                           int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+    if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
+    if (!x || !packed || !output0 || !ws || !q_ws || !s_ws) return set_status(BITLINEAR_ERR_NULL);
+    const int st = bitlinear_quant_absmax(x, q_ws, s_ws, M, K, mode, stream);
+    if (st != BITLINEAR_OK) return st;
+    return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, equal_slots(N, bitlinear_ws_num(N, K)), M,
+                                  N, K, (hipStream_t)stream));
+}
+
+}  // extern "C"

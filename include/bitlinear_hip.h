@@ -1,0 +1,126 @@
+/*
+ * libbitlinear_hip.so -- C ABI of the MI355X (gfx950) ternary BitLinear library.
+ *
+ * Plain C: pointers and sizes only.  Every pointer is a DEVICE pointer owned
+ * by the caller; the library neither allocates nor frees device memory in any
+ * entry point below, never synchronises, and launches only on the stream it is
+ * given (a hipStream_t passed as void*; NULL = the default stream).  All entry
+ * points are therefore legal on a stream that is being captured into a graph.
+ *
+ * bf16 values are passed as raw 16-bit patterns (uint16_t).
+ *
+ * Weight operand ("packed"): int8 [N, K/4] exactly as the reference packer
+ * writes it (gpu/pack_weight.py:76-98): stored 2-bit code = w + 2, 16x32 tiles
+ * of 128 bytes, 16 codes interleaved per little-endian int32.  It is consumed
+ * in place; no repack is needed.
+ */
+#ifndef BITLINEAR_HIP_H
+#define BITLINEAR_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes, returned by the int entry points and kept per host thread */
+#define BITLINEAR_OK 0
+#define BITLINEAR_ERR_SHAPE 1   /* N % 16 != 0, K % 64 != 0, or a size <= 0 */
+#define BITLINEAR_ERR_NULL 2    /* a required pointer is NULL               */
+#define BITLINEAR_ERR_LAUNCH 3  /* the HIP runtime refused the launch       */
+#define BITLINEAR_ERR_ARG 4     /* bad mode / segment list / tuning value   */
+
+/*
+ * Drop-in replacement for the reference's only exported symbol
+ *   extern "C" void bitlinear_int8xint2(int8_t*, int8_t*, __nv_bfloat16*,
+ *        __nv_bfloat16*, __nv_bfloat16*, int, int, int, cudaStream_t)
+ * (gpu/bitnet_kernels/bitnet_kernels.cu:3), bound by ctypes in
+ * gpu/model.py:18-37 and gpu/test.py:13-29.
+ *
+ *   input0  int8 [M, K] row-major activations
+ *   input1  packed ternary weight [N, K/4]
+ *   output0 bf16 [M, N]; every element is written
+ *   s       bf16 [M] activation scales (127/absmax); row m uses s[m]
+ *   ws      bf16 weight scales, at least ws_num(N, K) entries
+ * out[m, n] = bf16( float(acc[m, n]) / float(s[m]) * float(ws[n / (N / ws_num)]) )
+ * with acc the exact int32 dot product (bitnet_kernels.h:79-82).  ws_num is
+ * looked up from (N, K) with the reference's table (bitnet_kernels.cu:4-33)
+ * and is 1 for shapes the reference has no instance for.  Unlike the
+ * reference, any M >= 1, N % 16 == 0, K % 64 == 0 is computed; an unsupported
+ * shape prints the reference's "required ladder gemm kernel" line, launches
+ * nothing and sets the thread's status to BITLINEAR_ERR_SHAPE.
+ */
+void bitlinear_int8xint2(int8_t* input0, int8_t* input1, uint16_t* output0,
+                         uint16_t* s, uint16_t* ws, int M, int N, int K,
+                         void* stream);
+
+/* Status of the calling host thread's most recent library call (the
+ * reference's entry point returns void and reports nothing,
+ * bitnet_kernels.cu:34-36). */
+int bitlinear_last_status(void);
+const char* bitlinear_status_string(int status);
+
+/* The (N, K) -> ws_num table of bitnet_kernels.cu:4-33; 1 for other shapes. */
+int bitlinear_ws_num(int N, int K);
+
+/*
+ * Same computation, also storing the raw int32 accumulators
+ * (in_thread_C_local after the reduction, bitnet_kernels.h:74-78) to
+ * acc_out [M, N].  output0 may be NULL (then s and ws may be NULL too).
+ * Exists so tests can prove the accumulators bit-exact.
+ */
+int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1,
+                                int32_t* acc_out, uint16_t* output0,
+                                const uint16_t* s, const uint16_t* ws,
+                                int M, int N, int K, void* stream);
+
+/*
+ * Variant with explicit weight-scale segments: row n uses ws[j] for the first
+ * j with n < seg_ends[j]  (seg_ends ascending, seg_ends[nseg-1] == N,
+ * 1 <= nseg <= 8, host array).  This is the scale layout
+ * gpu/convert_checkpoint.py:42-77 writes for fused tensors (q/k/v rows
+ * 2560/640/640), which the reference kernel's equal-slot indexing
+ * (bitnet_kernels.h:80) does not follow for wqkv.
+ */
+int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1,
+                            uint16_t* output0, const uint16_t* s,
+                            const uint16_t* ws, const int* seg_ends, int nseg,
+                            int M, int N, int K, void* stream);
+
+/*
+ * Per-token absmax activation quantizer, BitLinearKernel.quant_input
+ * (gpu/model.py:68-71):  s = 127 / max|x|.clamp(min=1e-5),
+ * q = round_half_even(x * s).clamp(-128, 127).
+ *   x bf16 [M, K] row-major, K % 8 == 0;  q int8 [M, K];  s bf16 [M].
+ * torch evaluates 127 / t as t.reciprocal() * 127, and so do both modes:
+ *   mode 0: r = 1/amax and r*127 in fp32, s = bf16(r*127), q from the exact
+ *           fp32 product x * s (bit-identical to what torch.compile's
+ *           Inductor CPU backend makes of the expression)
+ *   mode 1: amax, r, s and the product x * s are each rounded to bf16
+ *           (bit-identical to torch eager on bf16 tensors)
+ */
+int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s,
+                           int M, int K, int mode, void* stream);
+
+/*
+ * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer
+ * (mode as above) then bitlinear_int8xint2.  q_ws (int8 [M, K]) and s_ws
+ * (bf16 [M]) are caller-provided workspaces that receive the quantized
+ * activations and scales.
+ */
+int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
+                           uint16_t* output0, const uint16_t* ws,
+                           int8_t* q_ws, uint16_t* s_ws,
+                           int M, int N, int K, int mode, void* stream);
+
+/*
+ * Launch-shape override for tuning runs: waves per workgroup (1..16) and
+ * 64-wide k-steps each wave keeps in flight (1, 2, 4, 8 or 16); 0, 0 restores
+ * the built-in choice.  Process-wide; results never depend on it.
+ */
+int bitlinear_set_tuning(int waves_per_group, int ksteps_in_flight);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITLINEAR_HIP_H */

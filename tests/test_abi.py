@@ -1,0 +1,72 @@
+"""The C-ABI library loads without a GPU and exports every function the
+header declares; host-only entry points behave as documented."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from bitnet_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "bitlinear_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(bitlinear_[a-z0-9_]+)\s*\(", text)
+
+
+def test_header_declares_the_drop_in_symbol():
+    names = _declared_functions()
+    assert "bitlinear_int8xint2" in names
+    assert len(names) == len(set(names)) >= 9
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built (run python -m bitnet_amd.build)")
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared_functions():
+        assert hasattr(raw, name), name
+    # and the binding table covers exactly the header
+    assert set(_lib.SIGNATURES) == set(_declared_functions())
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(_lib.BitLinearLibraryError):
+        _lib.load_library(str(tmp_path / "nope.so"))
+
+
+def test_host_only_entry_points():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built")
+    lib = _lib.load_library()
+    # shape table of the reference dispatcher (gpu/bitnet_kernels/bitnet_kernels.cu:4-33)
+    table = {(3840, 2560): 3, (2560, 2560): 1, (13824, 2560): 2, (2560, 6912): 1, (4800, 3200): 6,
+             (3200, 3200): 1, (20480, 3200): 2, (3200, 10240): 1, (5120, 27648): 1, (55296, 5120): 1}
+    for (n, k), v in table.items():
+        assert lib.bitlinear_ws_num(n, k) == v
+    assert lib.bitlinear_ws_num(1024, 4096) == 1
+    assert lib.bitlinear_status_string(0) == b"ok"
+    assert b"shape" in lib.bitlinear_status_string(1)
+    assert lib.bitlinear_set_tuning(8, 4) == 0
+    assert lib.bitlinear_set_tuning(17, 4) != 0
+    assert lib.bitlinear_set_tuning(8, 3) != 0
+    assert lib.bitlinear_set_tuning(0, 0) == 0
+
+
+def test_argument_checks_need_no_gpu(capfd):
+    """Shape and NULL checks run before any HIP call."""
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built")
+    lib = _lib.load_library()
+    # N not a multiple of 16: the reference's message, nothing launched
+    lib.bitlinear_int8xint2(None, None, None, None, None, 1, 100, 2560, None)
+    assert lib.bitlinear_last_status() == 1
+    assert "required ladder gemm kernel: M 1, N 100, K 2560" in capfd.readouterr().out
+    lib.bitlinear_int8xint2(None, None, None, None, None, 1, 2560, 2560, None)
+    assert lib.bitlinear_last_status() == 2
+    assert lib.bitlinear_quant_absmax(None, None, None, 1, 2560, 0, None) == 2
+    assert lib.bitlinear_quant_absmax(None, None, None, 1, 2563, 0, None) == 1
+    assert lib.bitlinear_int8xint2_acc_i32(None, None, None, None, None, None, 1, 2560, 100, None) == 1

@@ -1,0 +1,231 @@
+"""GPU parity tests: every call goes through the C ABI of libbitlinear_hip.so
+(via the ctypes host mirror) and is compared with the CPU oracle.
+
+Bars: int32 accumulators bit-exact; bf16 outputs bit-exact against the
+oracle's IEEE fp32 divide + multiply + RNE cast (the north star allows
+1 bf16 ulp / rel 1e-3; the tests assert the tighter bound and would report
+the ulp distance if it ever failed); quantizer outputs bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from bitnet_amd import _lib, bitlinear, pack_weight, workload
+from oracle import bitlinear_oracle as o
+from tests.gpu_util import bf16_ulp_distance, dev_bf16, dev_i8, host_bits
+
+pytestmark = pytest.mark.gpu
+
+SHAPES_2B = [(3840, 2560), (2560, 2560), (13824, 2560), (2560, 6912)]  # (N, K)
+SHAPES_3B = [(3200, 3200), (4800, 3200), (3200, 10240), (20480, 3200)]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu_and_lib():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    _lib.load_library()  # raises if the HIP library is missing: no fallback
+    yield
+    _lib.load_library().bitlinear_set_tuning(0, 0)
+
+
+def _rand_case(n, k, m, seed, full_range=True):
+    rng = np.random.default_rng(seed)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    lo, hi = (-128, 128) if full_range else (-128, 127)  # gpu/test.py:48 draws from [-128, 127)
+    a = rng.integers(lo, hi, size=(m, k), dtype=np.int8)
+    return w, a
+
+
+def _packed_dev(w):
+    return pack_weight.convert_weight_int8_to_int2(torch.from_numpy(w)).cuda()
+
+
+def _assert_bits_equal(got_bits, want_bits, what):
+    if not np.array_equal(got_bits, want_bits):
+        d = bf16_ulp_distance(got_bits, want_bits)
+        raise AssertionError(f"{what}: {int((d > 0).sum())} of {d.size} differ, max {int(d.max())} bf16 ulp")
+
+
+@pytest.mark.parametrize("n,k", SHAPES_2B + SHAPES_3B + [(16, 64), (48, 192), (5120, 27648)])
+def test_acc_bit_exact_m1(n, k):
+    w, a = _rand_case(n, k, 1, seed=n * 7 + k)
+    acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+    assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
+
+
+@pytest.mark.parametrize("n,k", SHAPES_2B + SHAPES_3B)
+def test_reference_known_answer_unit_scales(n, k):
+    """The reference's own check (gpu/test.py:42-61): s = ws = 1, output must
+    equal the bf16 cast of the integer matmul exactly."""
+    w, a = _rand_case(n, k, 1, seed=42 + n + k, full_range=False)
+    s = torch.ones(1, dtype=torch.bfloat16, device="cuda")
+    ws = torch.ones(6, dtype=torch.bfloat16, device="cuda")
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(a), _packed_dev(w), s, ws)
+    want = torch.from_numpy(a.astype(np.int32) @ w.astype(np.int32).T).to(torch.bfloat16)
+    assert out.shape == (1, n) and out.dtype == torch.bfloat16
+    assert torch.equal(out.cpu(), want)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 15, 16, 17, 33])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (2560, 6912), (3840, 2560)])
+def test_acc_bit_exact_small_m(n, k, m):
+    w, a = _rand_case(n, k, m, seed=1000 + m)
+    acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+    assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
+
+
+def test_acc_extreme_values():
+    n, k = 64, 6912
+    for wv, av in [(1, -128), (-1, -128), (1, 127), (0, -128)]:
+        w = np.full((n, k), wv, dtype=np.int8)
+        a = np.full((2, k), av, dtype=np.int8)
+        acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+        assert np.array_equal(acc.cpu().numpy(), np.full((2, n), wv * av * k, dtype=np.int32))
+
+
+def test_acc_single_nonzero_weight_picks_the_activation():
+    n, k = 32, 256
+    rng = np.random.default_rng(5)
+    a = rng.integers(-128, 128, size=(1, k), dtype=np.int8)
+    for r, c, v in [(0, 0, 1), (5, 17, -1), (15, 31, 1), (16, 32, -1), (31, 255, 1), (9, 77, -1), (12, 200, 1)]:
+        w = np.zeros((n, k), dtype=np.int8)
+        w[r, c] = v
+        acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w)).cpu().numpy()
+        want = np.zeros((1, n), dtype=np.int32)
+        want[0, r] = v * int(a[0, c])
+        assert np.array_equal(acc, want), (r, c, v)
+
+
+@pytest.mark.parametrize("shape_id", [0, 1, 2, 3])
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_scaled_output_at_2b_shapes(shape_id, m):
+    """Configs 0-2: seeded N(0,1) activations, quantized per token, real
+    weight scales in the slots this shape uses."""
+    sh = workload.shapes_2b()[shape_id]
+    w = workload.ternary_weight(sh.K, sh.N, shape_id)
+    ws_bits = workload.weight_scales(sh.K, sh.N, shape_id, sh.parts)
+    xb = workload.activations_bf16(m, sh.K, shape_id)
+    q, s_bits = o.quant_input(xb, o.QUANT_COMPILED)
+    acc, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(q), _packed_dev(w), dev_bf16(s_bits), dev_bf16(ws_bits))
+    _assert_bits_equal(host_bits(out), want, f"{sh.name} M={m}")
+    # and the whole BitLinearKernel.forward (quantizer + product) in one go
+    mod = bitlinear.BitLinearKernel(sh.K, sh.N).cuda()
+    mod.weight.data = _packed_dev(w)
+    mod.weight_scale.data = dev_bf16(ws_bits)
+    out2 = mod(dev_bf16(xb))
+    _assert_bits_equal(host_bits(out2), want, f"{sh.name} forward M={m}")
+
+
+def test_qkv_scale_slots_follow_the_reference_rule_and_seg_variant():
+    n, k = 3840, 2560
+    w, a = _rand_case(n, k, 2, seed=77)
+    s_bits = o.f32_to_bf16_bits(np.array([3.25, 17.5], dtype=np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.011, 0.023, 0.037, 0.0], dtype=np.float32))
+    pk = _packed_dev(w)
+    _, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)  # equal thirds
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(a), pk, dev_bf16(s_bits), dev_bf16(ws_bits))
+    _assert_bits_equal(host_bits(out), want, "equal-slot rule")
+    _, want_seg = o.bitlinear_int8xint2_seg(a, w, s_bits, ws_bits, [2560, 3200, 3840])
+    out_seg = bitlinear.bitnet_int8xint2_linear_seg(dev_i8(a), pk, dev_bf16(s_bits), dev_bf16(ws_bits), [2560, 3200, 3840])
+    _assert_bits_equal(host_bits(out_seg), want_seg, "segment rule")
+    assert not np.array_equal(want, want_seg)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("m,k", [(1, 2560), (1, 6912), (16, 2560), (5, 27648), (3, 8), (2, 10240)])
+def test_quantizer_bit_exact(mode, m, k):
+    rng = np.random.default_rng(k + m + mode)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    if m > 1:
+        x[1] *= 1e-7  # below the clamp
+    if m > 2:
+        x[2, ::7] *= 20.0
+    xb = o.f32_to_bf16_bits(x)
+    q, s = bitlinear.quant_input(dev_bf16(xb), mode)
+    wq, wsb = o.quant_input(xb, mode)
+    assert q.shape == (m, k) and s.shape == (m, 1)
+    assert np.array_equal(host_bits(s).reshape(-1), wsb)
+    assert np.array_equal(q.cpu().numpy(), wq)
+
+
+def test_quantizer_matches_committed_torch_vectors():
+    import os
+
+    fx = np.load(os.path.join(os.path.dirname(__file__), "golden", "quant_compiled_fixture.npz"))
+    for K in (256, 2560):
+        for mode, tag in ((0, "compiled"), (1, "eager")):
+            q, s = bitlinear.quant_input(dev_bf16(fx[f"x_{K}"]), mode)
+            assert np.array_equal(host_bits(s).reshape(-1), fx[f"s_{tag}_{K}"]), (K, tag)
+            assert np.array_equal(q.cpu().numpy(), fx[f"q_{tag}_{K}"]), (K, tag)
+
+
+def test_result_independent_of_launch_shape():
+    lib = _lib.load_library()
+    n, k, m = 2560, 6912, 3
+    w, a = _rand_case(n, k, m, seed=9)
+    pk, ad = _packed_dev(w), dev_i8(a)
+    want = o.acc_int32(a, w)
+    try:
+        for waves, upw in [(1, 1), (2, 16), (3, 4), (7, 8), (16, 2), (16, 16), (5, 1)]:
+            assert lib.bitlinear_set_tuning(waves, upw) == 0
+            acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
+            assert np.array_equal(acc.cpu().numpy(), want), (waves, upw)
+    finally:
+        lib.bitlinear_set_tuning(0, 0)
+
+
+def test_3d_input_and_out_argument():
+    n, k = 2560, 2560
+    w, a = _rand_case(n, k, 6, seed=3)
+    a3 = a.reshape(2, 3, k)
+    s_bits = o.f32_to_bf16_bits(np.linspace(1.0, 40.0, 6).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.016, 0, 0, 0], dtype=np.float32))
+    out = torch.full((2, 3, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ret = bitlinear.bitnet_int8xint2_linear(dev_i8(a3), _packed_dev(w), dev_bf16(s_bits).reshape(2, 3, 1), dev_bf16(ws_bits), out=out)
+    assert ret is out and out.shape == (2, 3, n)
+    _, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    _assert_bits_equal(host_bits(out).reshape(6, n), want, "3d")
+
+
+def test_unsupported_shape_reports_status_and_launches_nothing():
+    lib = _lib.load_library()
+    a = torch.zeros(1, 2560, dtype=torch.int8, device="cuda")
+    wbad = torch.zeros(100, 640, dtype=torch.int8, device="cuda")  # N = 100
+    s = torch.ones(1, dtype=torch.bfloat16, device="cuda")
+    ws = torch.ones(4, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.BitLinearLibraryError):
+        bitlinear.bitnet_int8xint2_linear(a, wbad, s, ws)
+    assert lib.bitlinear_last_status() == 1
+    with pytest.raises(ValueError):
+        bitlinear.bitnet_int8xint2_linear(a.cpu(), wbad, s, ws)
+
+
+def test_runs_on_a_side_stream_and_in_a_graph():
+    """The reference call sits inside a captured graph (gpu/generate.py:181-203):
+    no allocation, no sync, launches on the given stream only."""
+    n, k = 2560, 2560
+    w, a = _rand_case(n, k, 1, seed=21)
+    pk, ad = _packed_dev(w), dev_i8(a)
+    s = dev_bf16(o.f32_to_bf16_bits(np.array([7.0], dtype=np.float32)))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.02, 0, 0, 0], dtype=np.float32))
+    wsd = dev_bf16(ws_bits)
+    _, want = o.bitlinear_int8xint2(a, w, o.f32_to_bf16_bits(np.array([7.0], dtype=np.float32)), ws_bits)
+    out = torch.zeros(1, n, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        bitlinear.bitnet_int8xint2_linear(ad, pk, s, wsd, out=out)
+    side.synchronize()
+    _assert_bits_equal(host_bits(out), want, "side stream")
+    out.zero_()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        bitlinear.bitnet_int8xint2_linear(ad, pk, s, wsd, out=out)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        _assert_bits_equal(host_bits(out), want, "graph replay")
