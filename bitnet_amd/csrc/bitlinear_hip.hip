@@ -27,6 +27,7 @@
 #include "bitlinear_hip.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -47,8 +48,139 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// Scale slot of output row n: ends[] ascend, so it is the number of segment
+// boundaries at or below n.
+__device__ __forceinline__ int scale_slot(const ScaleMap& smap, int n) {
+    int slot = 0;
+#pragma unroll
+    for (int j = 0; j < kMaxSeg - 1; ++j) slot += (j < smap.nseg - 1 && n >= smap.ends[j]) ? 1 : 0;
+    return slot;
+}
+
 // ---------------------------------------------------------------------------
-// GEMV / small-M kernel
+// Decode kernel, M <= 4 tokens: one wave owns a 16-row block over all of K
+// ---------------------------------------------------------------------------
+// A lane loads 16 bytes (dwordx4): four packed words = rows 4q..4q+3 of one
+// 16-k chunk; the wave's 64 lanes cover 1 KB contiguous = 16 rows x 256 k.
+// Word i of every lane is the A operand of MFMA i (i = 0..3), which therefore
+// sees row 4q+i at A-row index p = 4*sigma + q with k-chunk 4g + sigma
+// (g = lane / 16).  The B operand puts token m's chunk 4g + sigma' at column
+// p' = 4*sigma' + m.  Entry (p, p') of the 16x16 result is a true partial dot
+// product exactly when sigma == sigma'; those entries sit in lanes 20*G + m
+// (G = sigma), register q, and the four G parts are added at the end.  The
+// off-diagonal entries are never read.  No cross-wave reduction, no workgroup
+// barrier after the weight stream.
+constexpr int kDecodeMaxTokens = 4;
+constexpr int kDecodeMaxWaves = 4;
+constexpr int kDecodeMaxLdsBytes = 48 * 1024;
+
+template <int R>
+__global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
+    const int8_t* __restrict__ act, const v4u* __restrict__ wq, uint16_t* __restrict__ out,
+    int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
+    ScaleMap smap, int M, int N, int K) {
+    __shared__ int red[kDecodeMaxWaves * 256];
+    extern __shared__ __attribute__((aligned(16))) int8_t lds_act[];  // [M][K]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const int rb = blockIdx.x * nwaves + wave;  // 16-row block of this wave
+    const bool rows_ok = rb < (N >> 4);
+    const int g = lane >> 4;
+    const int sg = (lane >> 2) & 3;  // sigma (A side) / sigma' (B side)
+    const int q = lane & 3;          // row quad (A side) / token (B side)
+    const int chunk = 4 * g + sg;    // 16-k chunk inside a 256-k step
+    const int steps = (K + 255) >> 8;
+
+    // 16-byte group of (row quad q, chunk): tile chunk/2, half chunk&1
+    const int grp = (chunk >> 1) * 8 + (q >> 1) * 4 + (chunk & 1) * 2 + (q & 1);
+    const v4u* wp = wq + (size_t)(rows_ok ? rb : 0) * (K >> 2) + grp;
+
+    // epilogue operands, fetched early as raw bits (see the split-K kernel)
+    const int e_row = lane >> 2;
+    const int e_m = lane & 3;
+    const int e_n = rb * 16 + e_row;
+    uint16_t e_sb = 0, e_wsb = 0;
+    if (out) {
+        e_sb = s[e_m < M ? e_m : M - 1];
+        e_wsb = ws[scale_slot(smap, rows_ok ? e_n : 0)];
+    }
+
+    const int tokB = q < M ? q : M - 1;  // columns of tokens >= M are never read
+    const int8_t* bp = lds_act + (size_t)tokB * K + chunk * 16;
+
+    v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0}, acc3 = {0, 0, 0, 0};
+    v4i accb = {0, 0, 0, 0};
+    const int neg2w = (int)0xFEFEFEFEu;
+    const v4i neg2 = {neg2w, neg2w, neg2w, neg2w};
+
+    for (int base = 0; base < steps; base += R) {
+        v4u w[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const int st = base + j;
+            const bool live = rows_ok && st < steps && (st * 256 + chunk * 16) < K;
+            w[j] = live ? __builtin_nontemporal_load(wp + (size_t)st * 64) : v4u{0u, 0u, 0u, 0u};
+        }
+        if (base == 0) {
+            // activations -> LDS while the weight loads are in flight
+            const int nvec = (M * K) >> 4;
+            for (int i = threadIdx.x; i < nvec; i += blockDim.x)
+                *(v4i*)(lds_act + (size_t)i * 16) = *(const v4i*)(act + (size_t)i * 16);
+            __syncthreads();
+        }
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const int st = base + j;
+            const bool live = st < steps && (st * 256 + chunk * 16) < K;
+            const v4i b = live ? *(const v4i*)(bp + (size_t)st * 256) : v4i{0, 0, 0, 0};
+            const uint32_t wd[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
+            v4i a[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                a[i].x = (int)(wd[i] & 0x03030303u);
+                a[i].y = (int)((wd[i] >> 2) & 0x03030303u);
+                a[i].z = (int)((wd[i] >> 4) & 0x03030303u);
+                a[i].w = (int)((wd[i] >> 6) & 0x03030303u);
+            }
+            acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[1], b, acc1, 0, 0, 0);
+            acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[2], b, acc2, 0, 0, 0);
+            acc3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[3], b, acc3, 0, 0, 0);
+            accb = __builtin_amdgcn_mfma_i32_16x16x64_i8(neg2, b, accb, 0, 0, 0);
+        }
+    }
+
+    // result lane 16G + p' holds A-rows 4G + r (r = register): diagonal <=> sigma' == G
+    int* myred = red + wave * 256;
+    if (sg == g) {
+        int* dst = myred + g * 64 + q;  // [G][row][token], token = q here
+        const int r0[4] = {acc0.x, acc1.x, acc2.x, acc3.x};
+        const int r1[4] = {acc0.y, acc1.y, acc2.y, acc3.y};
+        const int r2[4] = {acc0.z, acc1.z, acc2.z, acc3.z};
+        const int r3[4] = {acc0.w, acc1.w, acc2.w, acc3.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {  // register r of MFMA i is row 4r + i
+            dst[(0 + i) * 4] = r0[i] + accb.x;
+            dst[(4 + i) * 4] = r1[i] + accb.y;
+            dst[(8 + i) * 4] = r2[i] + accb.z;
+            dst[(12 + i) * 4] = r3[i] + accb.w;
+        }
+    }
+    // same wave wrote and reads: LDS operations of a wave complete in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (rows_ok && e_m < M) {
+        const int sum = myred[lane] + myred[64 + lane] + myred[128 + lane] + myred[192 + lane];
+        if (acc_out) acc_out[(size_t)e_m * N + e_n] = sum;
+        if (out) out[(size_t)e_m * N + e_n] = f32_to_bf16_rne((float)sum / bf16_to_f32(e_sb) * bf16_to_f32(e_wsb));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Small-batch kernel (M <= 16 per workgroup), K split across the waves
 // ---------------------------------------------------------------------------
 template <int UPW>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
@@ -71,6 +203,19 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     const uint32_t* wrow = wq + (size_t)nb * K + lane_word;
     const bool tok_ok = (m0 + p) < M;
     const int8_t* arow = act + (size_t)(tok_ok ? (m0 + p) : 0) * K + g * 16;
+
+    // The thread that will finish output (row, token) fetches its two scales
+    // now, as raw bits with nothing depending on them until the epilogue, so
+    // their latency overlaps the weight stream instead of preceding or
+    // following it.  Indices are clamped so every thread may load.
+    const int e_lane = threadIdx.x & 63;
+    const int e_m = m0 + (e_lane & 15);
+    const int e_n = nb * 16 + 4 * (e_lane >> 4) + ((threadIdx.x >> 6) & 3);
+    uint16_t e_sb = 0, e_wsb = 0;
+    if (out) {
+        e_sb = s[e_m < M ? e_m : M - 1];
+        e_wsb = ws[scale_slot(smap, e_n)];
+    }
 
     v4i acc_q = {0, 0, 0, 0};
     v4i acc_b = {0, 0, 0, 0};
@@ -107,6 +252,20 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     my[192] = acc_q.w + acc_b.w;
     __syncthreads();
 
+    if (blockDim.x >= 256) {
+        if (threadIdx.x < 256 && e_m < M) {
+            int part[kMaxWaves];  // independent LDS reads, one wait
+#pragma unroll
+            for (int wv = 0; wv < kMaxWaves; ++wv) part[wv] = (wv < nwaves) ? red[wv * 256 + threadIdx.x] : 0;
+            int sum = 0;
+#pragma unroll
+            for (int wv = 0; wv < kMaxWaves; ++wv) sum += part[wv];
+            if (acc_out) acc_out[(size_t)e_m * N + e_n] = sum;
+            if (out) out[(size_t)e_m * N + e_n] = f32_to_bf16_rne((float)sum / bf16_to_f32(e_sb) * bf16_to_f32(e_wsb));
+        }
+        return;
+    }
+    // fewer than four waves: every thread finishes several outputs
     for (int t = threadIdx.x; t < 256; t += blockDim.x) {
         const int l = t & 63;
         const int m = m0 + (l & 15);
@@ -116,10 +275,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
         const int n = nb * 16 + 4 * (l >> 4) + (t >> 6);
         if (acc_out) acc_out[(size_t)m * N + n] = sum;
         if (out) {
-            int slot = 0;  // ends[] ascend, so the slot is the count of boundaries at or below n
-#pragma unroll
-            for (int j = 0; j < kMaxSeg - 1; ++j) slot += (j < smap.nseg - 1 && n >= smap.ends[j]) ? 1 : 0;
-            const float v = (float)sum / bf16_to_f32(s[m]) * bf16_to_f32(ws[slot]);
+            const float v = (float)sum / bf16_to_f32(s[m]) * bf16_to_f32(ws[scale_slot(smap, n)]);
             out[(size_t)m * N + n] = f32_to_bf16_rne(v);
         }
     }
@@ -226,6 +382,8 @@ __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint1
 thread_local int g_status = BITLINEAR_OK;
 int g_tune_waves = 0;
 int g_tune_upw = 0;
+int g_tune_decode_waves = 0;
+int g_tune_path = 0;  // 0 = built-in choice, 2 = always the split-K kernel
 
 int set_status(int st) {
     g_status = st;
@@ -258,8 +416,8 @@ void pick_launch(int K, int* waves, int* upw) {
     *upw = u;
 }
 
-int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
-                const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
+                  const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     int waves, upw;
     pick_launch(K, &waves, &upw);
     const dim3 grid(N / 16, (M + 15) / 16, 1);
@@ -276,6 +434,36 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     }
 #undef BITLINEAR_LAUNCH
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
+                  const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+    const int steps = (K + 255) / 256;
+    int waves = 1;
+    if (g_tune_decode_waves > 0) waves = g_tune_decode_waves;
+    const int blocks16 = N / 16;
+    const dim3 grid((blocks16 + waves - 1) / waves, 1, 1);
+    const dim3 block(waves * 64, 1, 1);
+    const size_t lds = (size_t)M * K;
+    const v4u* wq = (const v4u*)packed;
+#define BITLINEAR_LAUNCH(R)                                                                                     \
+    hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, out, acc_out, s, ws, smap, M, N, K)
+    if (steps <= 4) BITLINEAR_LAUNCH(4);
+    else if (steps <= 10) BITLINEAR_LAUNCH(10);
+    else if (steps <= 16) BITLINEAR_LAUNCH(16);
+    else if (steps <= 27) BITLINEAR_LAUNCH(27);
+    else BITLINEAR_LAUNCH(32);
+#undef BITLINEAR_LAUNCH
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
+                const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+    // vector loads: 16-byte groups of both operands must be 16-byte aligned
+    if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
+    const bool decode_fits = M <= kDecodeMaxTokens && (size_t)M * K <= (size_t)kDecodeMaxLdsBytes;
+    if (decode_fits && g_tune_path != 2) return launch_decode(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+    return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
 }
 
 ScaleMap equal_slots(int N, int ws_num) {
@@ -309,17 +497,27 @@ int bitlinear_ws_num(int N, int K) {
     return 1;
 }
 
-int bitlinear_set_tuning(int waves_per_group, int ksteps_in_flight) {
-    if (waves_per_group == 0 && ksteps_in_flight == 0) {
-        g_tune_waves = g_tune_upw = 0;
+int bitlinear_set_tuning(int kernel, int waves_per_group, int ksteps_in_flight) {
+    if (kernel == 0) {
+        g_tune_path = g_tune_waves = g_tune_upw = g_tune_decode_waves = 0;
         return set_status(BITLINEAR_OK);
     }
-    const int u = ksteps_in_flight;
-    if (waves_per_group < 1 || waves_per_group > kMaxWaves || !(u == 1 || u == 2 || u == 4 || u == 8 || u == 16))
-        return set_status(BITLINEAR_ERR_ARG);
-    g_tune_waves = waves_per_group;
-    g_tune_upw = u;
-    return set_status(BITLINEAR_OK);
+    if (kernel == 1) {
+        if (waves_per_group < 1 || waves_per_group > kDecodeMaxWaves) return set_status(BITLINEAR_ERR_ARG);
+        g_tune_path = 1;
+        g_tune_decode_waves = waves_per_group;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 2) {
+        const int u = ksteps_in_flight;
+        if (waves_per_group < 1 || waves_per_group > kMaxWaves || !(u == 1 || u == 2 || u == 4 || u == 8 || u == 16))
+            return set_status(BITLINEAR_ERR_ARG);
+        g_tune_path = 2;
+        g_tune_waves = waves_per_group;
+        g_tune_upw = u;
+        return set_status(BITLINEAR_OK);
+    }
+    return set_status(BITLINEAR_ERR_ARG);
 }
 
 int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1, int32_t* acc_out, uint16_t* output0,

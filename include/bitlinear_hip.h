@@ -28,7 +28,8 @@ extern "C" {
 #define BITLINEAR_ERR_SHAPE 1   /* N % 16 != 0, K % 64 != 0, or a size <= 0 */
 #define BITLINEAR_ERR_NULL 2    /* a required pointer is NULL               */
 #define BITLINEAR_ERR_LAUNCH 3  /* the HIP runtime refused the launch       */
-#define BITLINEAR_ERR_ARG 4     /* bad mode / segment list / tuning value   */
+#define BITLINEAR_ERR_ARG 4     /* bad mode / segment list / tuning value, or
+                                   an operand not 16-byte aligned           */
 
 /*
  * Drop-in replacement for the reference's only exported symbol
@@ -114,11 +115,16 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
                            int M, int N, int K, int mode, void* stream);
 
 /*
- * Launch-shape override for tuning runs: waves per workgroup (1..16) and
- * 64-wide k-steps each wave keeps in flight (1, 2, 4, 8 or 16); 0, 0 restores
- * the built-in choice.  Process-wide; results never depend on it.
+ * Kernel / launch-shape override for tuning runs and tests.  Process-wide;
+ * results never depend on it.
+ *   kernel 0: built-in choice (other arguments ignored)
+ *   kernel 1: decode kernel where it applies (M <= 4, M*K <= 48 KiB) with
+ *             waves_per_group (1..4) 16-row blocks per workgroup
+ *   kernel 2: split-K kernel always, waves_per_group (1..16) waves per
+ *             workgroup each keeping ksteps_in_flight (1, 2, 4, 8 or 16)
+ *             64-wide k-steps in flight
  */
-int bitlinear_set_tuning(int waves_per_group, int ksteps_in_flight);
+int bitlinear_set_tuning(int kernel, int waves_per_group, int ksteps_in_flight);
 
 #ifdef __cplusplus
 }

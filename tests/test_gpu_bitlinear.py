@@ -25,7 +25,7 @@ def _need_gpu_and_lib():
     assert torch.cuda.is_available(), "these tests need the MI355X"
     _lib.load_library()  # raises if the HIP library is missing: no fallback
     yield
-    _lib.load_library().bitlinear_set_tuning(0, 0)
+    _lib.load_library().bitlinear_set_tuning(0, 0, 0)
 
 
 def _rand_case(n, k, m, seed, full_range=True):
@@ -160,19 +160,39 @@ def test_quantizer_matches_committed_torch_vectors():
             assert np.array_equal(q.cpu().numpy(), fx[f"q_{tag}_{K}"]), (K, tag)
 
 
-def test_result_independent_of_launch_shape():
+def test_result_independent_of_kernel_and_launch_shape():
     lib = _lib.load_library()
-    n, k, m = 2560, 6912, 3
-    w, a = _rand_case(n, k, m, seed=9)
-    pk, ad = _packed_dev(w), dev_i8(a)
+    n, k = 2560, 6912
+    try:
+        for m in (1, 3, 4):
+            w, a = _rand_case(n, k, m, seed=9 + m)
+            pk, ad = _packed_dev(w), dev_i8(a)
+            want = o.acc_int32(a, w)
+            settings = [(2, wv, u) for wv, u in [(1, 1), (2, 16), (3, 4), (7, 8), (16, 2), (16, 16), (5, 1)]]
+            settings += [(1, 1, 0), (1, 2, 0), (1, 3, 0), (1, 4, 0), (0, 0, 0)]
+            for setting in settings:
+                assert lib.bitlinear_set_tuning(*setting) == 0
+                acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
+                assert np.array_equal(acc.cpu().numpy(), want), (m, setting)
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0)
+
+
+@pytest.mark.parametrize("n,k", [(16, 64), (16, 128), (48, 192), (80, 320), (32, 3200), (1040, 256)])
+@pytest.mark.parametrize("m", [1, 2, 4])
+def test_decode_kernel_ragged_shapes(n, k, m):
+    """K not a multiple of 256 (partial last step) and row-block counts that
+    do not fill the last workgroup."""
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=n + k + m)
     want = o.acc_int32(a, w)
     try:
-        for waves, upw in [(1, 1), (2, 16), (3, 4), (7, 8), (16, 2), (16, 16), (5, 1)]:
-            assert lib.bitlinear_set_tuning(waves, upw) == 0
-            acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
-            assert np.array_equal(acc.cpu().numpy(), want), (waves, upw)
+        for waves in (1, 3, 4):
+            assert lib.bitlinear_set_tuning(1, waves, 0) == 0
+            acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+            assert np.array_equal(acc.cpu().numpy(), want), waves
     finally:
-        lib.bitlinear_set_tuning(0, 0)
+        lib.bitlinear_set_tuning(0, 0, 0)
 
 
 def test_3d_input_and_out_argument():
