@@ -144,7 +144,7 @@ def cpu_baseline(shapes, M, budget_s=12.0):
             one_layer(nt)
             n += 1
             el = time.perf_counter() - t0
-            if el > budget_s * share or n >= 2000:
+            if el > budget_s * share:
                 break
         out[tag] = (layer_bytes * n / el / 1e9, n, el)
     return {
@@ -154,7 +154,7 @@ def cpu_baseline(shapes, M, budget_s=12.0):
         "kind": "port",
         "sample": (
             f"one decoder layer (wqkv, wo, w13, w2; {layer_bytes} packed-weight bytes) at M={M}, "
-            f"{out['threads'][1]} passes in {out['threads'][2]:.1f} s on {threads} threads; "
+            f"{out['threads'][1]} passes in {out['threads'][2]:.1f} s on {threads} threads (weights stay cache-resident); "
             f"C/AVX2 restatement of ggml_vec_dot_i2_i8_s + explicit -sum(y) correction"
         ),
         "single_thread_GBps": round(out["single"][0], 3),

@@ -439,7 +439,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
 int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                   const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     const int steps = (K + 255) / 256;
-    int waves = 1;
+    int waves = 4;
     if (g_tune_decode_waves > 0) waves = g_tune_decode_waves;
     const int blocks16 = N / 16;
     const dim3 grid((blocks16 + waves - 1) / waves, 1, 1);
@@ -462,7 +462,10 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // vector loads: 16-byte groups of both operands must be 16-byte aligned
     if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
     const bool decode_fits = M <= kDecodeMaxTokens && (size_t)M * K <= (size_t)kDecodeMaxLdsBytes;
-    if (decode_fits && g_tune_path != 2) return launch_decode(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+    // The one-wave-per-row-block kernel pays off once there are enough row
+    // blocks to fill every SIMD; below that, splitting K across waves wins.
+    const bool many_rows = (N / 16) >= 512;
+    if (decode_fits && g_tune_path != 2 && (many_rows || g_tune_path == 1)) return launch_decode(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
     return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
 }
 

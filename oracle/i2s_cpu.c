@@ -29,7 +29,6 @@
  * |y| <= 127 and codes <= 2 with up to 32 blocks: 32*4*2*2*127 = 65024 can
  * exceed 32767 only for adversarial same-sign data).
  */
-#include <pthread.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -220,48 +219,37 @@ void i2s_gemm(int n, float* s, size_t bs, const void* vx, const void* vy, int nr
 
 /* ---- BitLinear on top of the dot kernels ----------------------------------*/
 
-typedef struct {
-    int K, N, M, c_begin, c_end;
-    const uint8_t* x;
-    const int8_t* y;
-    int32_t* acc; /* [M, N] */
-    float* tmp;   /* [M, N] */
-} job_t;
-
-static void* job_main(void* arg) {
-    job_t* j = (job_t*)arg;
-    const int nr4 = j->M == 1 ? 1 : j->M - j->M % I2S_ROW_TILE;
-    gemm_cols(j->K, j->tmp, (size_t)j->N, j->x, j->y, nr4, j->c_begin, j->c_end);
-    for (int r = nr4; r < j->M; ++r)
-        gemm_cols(j->K, j->tmp + (size_t)r * j->N, (size_t)j->N, j->x, j->y + (size_t)r * j->K, 1, j->c_begin, j->c_end);
-    for (int m = 0; m < j->M; ++m) {
+/* Weight rows [c_begin, c_end) of the product for all M activation rows. */
+static void bitlinear_cols(const uint8_t* x, const int8_t* y, int32_t* acc, float* tmp, int M, int N, int K,
+                           int c_begin, int c_end) {
+    const int nr4 = M == 1 ? 1 : M - M % I2S_ROW_TILE;
+    gemm_cols(K, tmp, (size_t)N, x, y, nr4, c_begin, c_end);
+    for (int r = nr4; r < M; ++r) gemm_cols(K, tmp + (size_t)r * N, (size_t)N, x, y + (size_t)r * K, 1, c_begin, c_end);
+    for (int m = 0; m < M; ++m) {
         int ysum = 0;
-        for (int k = 0; k < j->K; ++k) ysum += j->y[(size_t)m * j->K + k];
-        for (int c = j->c_begin; c < j->c_end; ++c)
-            j->acc[(size_t)m * j->N + c] = (int32_t)j->tmp[(size_t)m * j->N + c] - ysum; /* q = w + 1 */
+        for (int k = 0; k < K; ++k) ysum += y[(size_t)m * K + k];
+        for (int c = c_begin; c < c_end; ++c)
+            acc[(size_t)m * N + c] = (int32_t)tmp[(size_t)m * N + c] - ysum; /* q = w + 1 */
     }
-    return NULL;
 }
 
 /* acc[m, n] = sum_k w[n, k] * y[m, k] from I2_S-packed weights, weight rows
- * split contiguously over nthreads (ggml splits the rows of the weight
- * matrix across its thread pool in the same way).  tmp is float [M, N]. */
+ * split contiguously over nthreads OpenMP threads (ggml splits the rows of
+ * the weight matrix across its thread pool in the same way; the reference's
+ * own harness is built with -fopenmp, utils/test_gemm_kernel.sh:392-397).
+ * tmp is float [M, N]. */
 void i2s_bitlinear_acc(const void* packed, const int8_t* y, int32_t* acc, float* tmp, int M, int N, int K, int nthreads) {
     if (nthreads < 1) nthreads = 1;
-    if (nthreads > 256) nthreads = 256;
-    pthread_t th[256];
-    job_t jobs[256];
     const int per = (N + nthreads - 1) / nthreads;
-    int used = 0;
+    if (nthreads == 1) {
+        bitlinear_cols((const uint8_t*)packed, y, acc, tmp, M, N, K, 0, N);
+        return;
+    }
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
     for (int t = 0; t < nthreads; ++t) {
         const int b = t * per, e = b + per < N ? b + per : N;
-        if (b >= e) break;
-        jobs[t] = (job_t){K, N, M, b, e, (const uint8_t*)packed, y, acc, tmp};
-        ++used;
+        if (b < e) bitlinear_cols((const uint8_t*)packed, y, acc, tmp, M, N, K, b, e);
     }
-    for (int t = 1; t < used; ++t) pthread_create(&th[t], NULL, job_main, &jobs[t]);
-    job_main(&jobs[0]);
-    for (int t = 1; t < used; ++t) pthread_join(th[t], NULL);
 }
 
 int i2s_has_avx2(void) {
