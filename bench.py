@@ -5,18 +5,20 @@
 
 One "step" is one pass of the hot path over the BitLinear stack of a
 BitNet-b1.58-2B decoder at M tokens (default 1): 30 layers x (wqkv, wo, w13,
-w2), each call = fused absmax quantizer kernel + int8 x int2 GEMV kernel
-(BitLinearKernel.forward of the reference, gpu/model.py:73-75), every layer
-with its own weights (521 MB of packed weights per step, so the stream comes
-from HBM, not from cache).  The 240 launches of a step are replayed from a
-HIP graph, as the reference replays its decode step from a CUDA graph
-(gpu/generate.py:198-211).  Inputs are resident in HBM before timing starts.
+w2), each call = BitLinearKernel.forward of the reference (gpu/model.py:73-75:
+absmax quantizer, int8 x int2 product, scale epilogue), which the library runs
+as ONE kernel per call at decode sizes.  Every layer has its own weights
+(521 MB of packed weights per step, so the stream comes from HBM, not from
+cache).  The 120 launches of a step are replayed from a HIP graph, as the
+reference replays its decode step from a CUDA graph (gpu/generate.py:198-211).
+Inputs are resident in HBM before timing starts.
 
-Prints ONE JSON line.  `value` is packed-weight bytes (K*N/4 per GEMV) per
-second over the whole step.  `roofline` is for the GEMV kernel alone: a graph
-of only the 120 GEMV launches of a step is timed with HIP events on its
-stream; `cpu_baseline` is the C restatement of the reference's CPU I2_S
-kernel timed on this host on a bounded sample of the same workload.
+Prints ONE JSON line.  `value` is packed-weight bytes (K*N/4 per product) per
+second over the whole step.  `roofline` is for the kernel those launches run
+(bitlinear_fused_kernel): the same timed region, measured with HIP events on
+the stream the graph is replayed on, divided by the 120 launches of a step.
+`cpu_baseline` is the C restatement of the reference's CPU I2_S kernel timed
+on this host on a bounded sample of the same workload.
 """
 import argparse
 import ctypes
@@ -122,17 +124,19 @@ def cpu_baseline(shapes, M, budget_s=12.0):
     except AttributeError:
         cores = os.cpu_count() or 1
     threads = max(1, min(cores, 16))
+    n_layers = 8  # distinct weights per layer: 139 MB of packed weights, streamed from DRAM like the GPU's from HBM
     cases = []
-    for sh in shapes:
-        w = workload.ternary_weight(sh.K, sh.N, sh.shape_id)
-        q, _ = o.quant_input(workload.activations_bf16(M, sh.K, sh.shape_id))
-        packed = i2s_cpu.pack(w)
-        acc = np.empty((M, sh.N), dtype=np.int32)
-        tmp = np.empty((M, sh.N), dtype=np.float32)
-        cases.append((packed, q, acc, tmp))
-    layer_bytes = sum(sh.weight_bytes for sh in shapes)
+    for layer in range(n_layers):
+        for sh in shapes:
+            w = workload.ternary_weight(sh.K, sh.N, sh.shape_id, layer)
+            q, _ = o.quant_input(workload.activations_bf16(M, sh.K, sh.shape_id))
+            packed = i2s_cpu.pack(w)
+            acc = np.empty((M, sh.N), dtype=np.int32)
+            tmp = np.empty((M, sh.N), dtype=np.float32)
+            cases.append((packed, q, acc, tmp))
+    layer_bytes = sum(sh.weight_bytes for sh in shapes) * n_layers
 
-    def one_layer(nt):
+    def one_layer(nt):  # one pass over the n_layers sample
         for packed, q, acc, tmp in cases:
             i2s_cpu.bitlinear_acc(packed, q, nt, tmp=tmp, acc=acc)
 
@@ -153,12 +157,12 @@ def cpu_baseline(shapes, M, budget_s=12.0):
         "cores": threads,
         "kind": "port",
         "sample": (
-            f"one decoder layer (wqkv, wo, w13, w2; {layer_bytes} packed-weight bytes) at M={M}, "
-            f"{out['threads'][1]} passes in {out['threads'][2]:.1f} s on {threads} threads (weights stay cache-resident); "
+            f"{n_layers} decoder layers with distinct weights (wqkv, wo, w13, w2 each; {layer_bytes} packed-weight "
+            f"bytes per pass) at M={M}, {out['threads'][1]} passes in {out['threads'][2]:.1f} s on {threads} threads; "
             f"C/AVX2 restatement of ggml_vec_dot_i2_i8_s + explicit -sum(y) correction"
         ),
         "single_thread_GBps": round(out["single"][0], 3),
-        "tokens_per_s_bitlinear_only": round(out["threads"][0] * 1e9 / (layer_bytes * 30), 2),
+        "tokens_per_s_bitlinear_only": round(out["threads"][0] * 1e9 / (layer_bytes / n_layers * 30), 2),
     }
 
 
@@ -170,6 +174,12 @@ def main():
     ap.add_argument("--m", type=int, default=1, help="tokens per step (decode batch), 1..16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument(
+        "--pmc-probe",
+        action="store_true",
+        help="counter run for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: three plain 256 MiB device copies "
+        "(calibration) and one eager pass of the 120 GEMV launches, then exit",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         print(
@@ -203,8 +213,8 @@ def main():
                 )
                 assert st == 0, lib.bitlinear_status_string(st)
 
-    def launch_gemv_only(sp, only=None):
-        for row in layers:
+    def launch_gemv_only(sp, only=None, passes=1):
+        for row in layers * passes:
             for i, sh in enumerate(shapes):
                 if only is not None and i != only:
                     continue
@@ -216,6 +226,19 @@ def main():
             for i, sh in enumerate(shapes):
                 lib.bitlinear_quant_absmax(_p(acts[i]), _p(q_buf[i]), _p(s_buf[i]), M, sh.K, 0, sp)
 
+    if args.pmc_probe:
+        launch_quant_only(None)  # fills q_buf / s_buf
+        src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        launch_path(None)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": "3 copies of 268435456 B (read 256 MiB + write 256 MiB each), then the 120 launches of one step"}))
+        return
+
     step_bytes = sum(sh.weight_bytes for sh in shapes) * len(layers)
     n_gemv = len(shapes) * len(layers)
 
@@ -226,25 +249,29 @@ def main():
     ms_per_step = wall_s * 1e3 / args.steps
     value = step_bytes / (wall_s / args.steps) / 1e9
 
-    # ---- dominant kernel: GEMV launches only, HIP events on their stream ----
+    # ---- the drop-in product entry alone (int8 activations already quantized) ----
     gemv = GraphRun(launch_gemv_only)
     gemv.replay(args.warmup)
     _, gemv_ms = gemv.timed(args.steps)
     gemv_us = gemv_ms * 1e3 / (args.steps * n_gemv)
-    achieved = (step_bytes / n_gemv) / (gemv_us * 1e-6) / 1e9
+    # the timed region holds nothing but the 120 launches of the fused kernel
+    fused_us = ev_ms * 1e3 / (args.steps * n_gemv)
+    achieved = (step_bytes / n_gemv) / (fused_us * 1e-6) / 1e9
 
     per_shape = {}
     for i, sh in enumerate(shapes):
-        g = GraphRun(lambda sp, i=i: launch_gemv_only(sp, only=i))
+        passes = 8  # 240 launches per graph, so the cost of starting a replay does not weigh on the figure
+        g = GraphRun(lambda sp, i=i: launch_gemv_only(sp, only=i, passes=passes))
         g.replay(max(2, args.warmup // 4))
-        _, ms = g.timed(args.steps)
-        us = ms * 1e3 / (args.steps * len(layers))
+        nrep = max(1, args.steps // 4)
+        _, ms = g.timed(nrep)
+        us = ms * 1e3 / (nrep * len(layers) * passes)
         per_shape[sh.name] = {
             "K": sh.K,
             "N": sh.N,
             "us_per_launch": round(us, 3),
             "GBps": round(sh.weight_bytes / (us * 1e-6) / 1e9, 1),
-            "note": "30 weight copies of this shape replayed in a loop: fits the 256 MB last-level cache, not HBM-cold",
+            "note": "30 weight copies of this shape in a loop (49-265 MB): partly served by the 256 MB last-level cache",
         }
         del g
     quant = GraphRun(launch_quant_only)
@@ -253,12 +280,12 @@ def main():
     quant_us = q_ms * 1e3 / (args.steps * n_gemv)
 
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "gemv_hbm_traffic.json")
+    # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs, kept with their commands in profiles/
+    tpath = os.path.join(ROOT, "profiles", "bitlinear_fused_m1_bitnet2b_hbm_traffic.txt")
     if M == 1 and os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
-        except (ValueError, OSError):
-            traffic = None
+        for line in open(tpath):
+            if line.startswith("traffic_bytes_per_launch:"):
+                traffic = int(float(line.split(":", 1)[1]))
 
     result = {
         "metric": METRIC,
@@ -277,8 +304,8 @@ def main():
         "config": {
             "workload": (
                 f"BitNet-2B BitLinear stack, M={M}: 30 layers x (K,N) in (2560,3840) (2560,2560) (2560,13824) "
-                "(6912,2560), quantizer + GEMV per call, 240 launches per step from a HIP graph, distinct weights "
-                "per layer"
+                "(6912,2560), BitLinearKernel.forward (quantizer + product + epilogue, one kernel) per call, 120 "
+                "launches per step from a HIP graph, distinct weights per layer"
             ),
             "tokens_per_step": M,
             "packed_weight_bytes_per_step": step_bytes,
@@ -293,11 +320,13 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "kernel": "gemv_i2 (int8 x int2 GEMV), mean over the 120 launches of a step",
+            "kernel": "bitlinear_fused_kernel (quantizer + int8 x int2 product + epilogue), mean over the 120 "
+            "launches of a step, HIP events on the replay stream over the timed region",
             "bytes_per_launch": step_bytes // n_gemv,
-            "us_per_launch": round(gemv_us, 3),
+            "us_per_launch": round(fused_us, 3),
         },
-        "per_shape_gemv": per_shape,
+        "product_only_us_per_launch": round(gemv_us, 3),
+        "per_shape_product_only": per_shape,
         "quantizer_us_per_launch": round(quant_us, 3),
     }
     if not args.no_cpu_baseline:

@@ -31,7 +31,7 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
-    "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int]),
+    "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
 }
 
 _lib = None

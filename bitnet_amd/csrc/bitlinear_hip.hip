@@ -48,6 +48,40 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
+// for every outstanding global load of the wave, which would serialise the
+// weight stream behind the barrier; here the weight words stay in flight.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Wave-wide reductions with DPP lane permutes (no LDS): two quad permutes and
+// two mirrors leave every lane of a 16-lane row with the row's result; the
+// four row results are then combined through scalar registers.
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, (uint32_t)dpp_move<0xB1>((int)v));   // quad_perm [1,0,3,2]
+    v = max(v, (uint32_t)dpp_move<0x4E>((int)v));   // quad_perm [2,3,0,1]
+    v = max(v, (uint32_t)dpp_move<0x141>((int)v));  // row_half_mirror
+    v = max(v, (uint32_t)dpp_move<0x140>((int)v));  // row_mirror
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ int wave_sum_i32(int v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);
+    return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+           __builtin_amdgcn_readlane(v, 48);
+}
+
 // Scale slot of output row n: ends[] ascend, so it is the number of segment
 // boundaries at or below n.
 __device__ __forceinline__ int scale_slot(const ScaleMap& smap, int n) {
@@ -319,6 +353,21 @@ __device__ __forceinline__ uint2 quant_vec8(const uint4& v, float s32) {
     return make_uint2(o[0], o[1]);
 }
 
+// Activation scale from the row's |x| maximum (as bf16 bits).  torch evaluates
+// 127 / t as t.reciprocal() * 127: a reciprocal, then a multiply.  The value
+// returned is exactly representable in bf16.
+template <int MODE>
+__device__ __forceinline__ float quant_scale(uint32_t amax_bits) {
+    float amax = __uint_as_float(amax_bits << 16);
+    if (MODE == 0) {
+        const float r = 1.0f / fmaxf(amax, 1e-5f);
+        return bf16_to_f32(f32_to_bf16_rne(r * 127.0f));
+    }
+    amax = fmaxf(amax, bf16_to_f32(f32_to_bf16_rne(1e-5f)));
+    const float r = bf16_to_f32(f32_to_bf16_rne(1.0f / amax));
+    return bf16_to_f32(f32_to_bf16_rne(r * 127.0f));
+}
+
 template <int MODE>
 __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint16_t* __restrict__ x,
                                                                      int8_t* __restrict__ q,
@@ -354,17 +403,7 @@ __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint1
 #pragma unroll
     for (int i = 1; i < kQuantThreads / 64; ++i) am = max(am, wmax[i]);
 
-    // torch evaluates 127 / t as t.reciprocal() * 127: a reciprocal, then a multiply
-    float amax = __uint_as_float(am << 16);
-    float s32;
-    if (MODE == 0) {
-        const float r = 1.0f / fmaxf(amax, 1e-5f);
-        s32 = bf16_to_f32(f32_to_bf16_rne(r * 127.0f));
-    } else {
-        amax = fmaxf(amax, bf16_to_f32(f32_to_bf16_rne(1e-5f)));
-        const float r = bf16_to_f32(f32_to_bf16_rne(1.0f / amax));
-        s32 = bf16_to_f32(f32_to_bf16_rne(r * 127.0f));
-    }
+    const float s32 = quant_scale<MODE>(am);
     if (tid == 0) s[row] = f32_to_bf16_rne(s32);
 
 #pragma unroll
@@ -377,13 +416,191 @@ __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint1
 }
 
 // ---------------------------------------------------------------------------
+// BitLinearKernel.forward in one kernel: absmax quantizer + product + epilogue
+// ---------------------------------------------------------------------------
+// Every workgroup quantizes the (small) activation block itself -- it is a few
+// KB read from L2 while the weight words are already in flight -- keeps the
+// int8 rows in LDS, and feeds the B operand of the MFMAs from there.  The
+// +2 bias of the stored codes is removed with sum(q) per token, collected
+// while quantizing: sum((c - 2) * q) = sum(c * q) - 2 * sum(q).
+// A workgroup owns RB consecutive 16-row blocks; S waves split K for each.
+constexpr int kFusedMaxRB = 4;
+constexpr int kFusedMaxTokens = 16;
+constexpr int kFusedRowPad = 64;  // bytes between token rows in LDS beyond K
+
+template <int UPW, int VMAX>
+__global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
+    const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
+    int M, int N, int K, int RB, int S, int mode) {
+    extern __shared__ __attribute__((aligned(16))) int8_t lds_q[];  // [M][K + pad]
+    __shared__ int red[kFusedMaxRB * 256];
+    __shared__ uint32_t amax_bits[kFusedMaxTokens];
+    __shared__ int qsum[kFusedMaxTokens];
+    __shared__ float sval[kFusedMaxTokens];  // activation scale per token (a bf16 value)
+
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int rbl = wave / S;  // row block inside the workgroup
+    const int ks = wave - rbl * S;
+    const int rb = blockIdx.x * RB + rbl;
+    const bool rows_ok = rb < (N >> 4);
+    const int g = lane >> 4;
+    const int p = lane & 15;
+    const int units = K >> 6;
+    const int kp = K + kFusedRowPad;
+
+    const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
+    const uint32_t* wrow = wq + (size_t)(rows_ok ? rb : 0) * K + lane_word;
+
+    // Activation block first: 16-byte vectors of 8 bf16, VMAX per thread.  The
+    // memory counter retires loads in issue order, so what is needed first
+    // (x) is requested first and the weight words stay outstanding behind it.
+    const int vec_per_row = K >> 3;
+    const int nvec = M * vec_per_row;
+    // Loads are unconditional (indices clamped into range, surplus results
+    // ignored later): a load under a branch would force a full wait for all
+    // earlier loads at the first use of x.
+    uint4 xv[VMAX];
+#pragma unroll
+    for (int v = 0; v < VMAX; ++v) {
+        const int idx = tid + v * nthreads;
+        xv[v] = *(const uint4*)(x + (size_t)(idx < nvec ? idx : nvec - 1) * 8);
+    }
+    // weight words of the first round
+    uint32_t w[UPW];
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) {
+        const int u = ks * UPW + j;
+        w[j] = __builtin_nontemporal_load(wrow + (size_t)(u < units ? u : units - 1) * 64);
+    }
+    // epilogue weight scale, raw bits, nothing depends on it until the end
+    uint16_t e_wsb[kFusedMaxRB];
+#pragma unroll
+    for (int r = 0; r < kFusedMaxRB; ++r) {
+        const int t = tid + r * nthreads;  // output slot t of the workgroup: [row block][reg][lane]
+        const int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
+        e_wsb[r] = ws[scale_slot(smap, n < N ? n : N - 1)];  // unconditional: no branch, no early wait
+    }
+
+    for (int i = tid; i < RB * 256; i += nthreads) red[i] = 0;
+    if (tid < kFusedMaxTokens) {
+        amax_bits[tid] = 0u;
+        qsum[tid] = 0;
+    }
+    lds_barrier();
+
+    // one LDS atomic per wave and token row where the wave's 64 vectors lie in
+    // one row (always so when K/8 is a multiple of 64); per lane otherwise
+#pragma unroll
+    for (int v = 0; v < VMAX; ++v) {
+        const int idx = tid + v * nthreads;
+        const int row = idx < nvec ? idx / vec_per_row : -1;
+        const uint32_t lm = idx < nvec ? absmax_bits8(xv[v], 0u) : 0u;
+        const int row0 = __builtin_amdgcn_readfirstlane(row);
+        if (__builtin_amdgcn_ballot_w64(row != row0) == 0) {
+            const uint32_t wm = wave_max_u32(lm);
+            if (lane == 0 && row0 >= 0) atomicMax(&amax_bits[row0], wm);
+        } else if (row >= 0) {
+            atomicMax(&amax_bits[row], lm);
+        }
+    }
+    lds_barrier();
+
+#pragma unroll
+    for (int v = 0; v < VMAX; ++v) {
+        const int idx = tid + v * nthreads;
+        const int prow = idx < nvec ? idx / vec_per_row : -1;
+        int part = 0;  // sum of this thread's 8 quantized values
+        if (idx < nvec) {
+            const int row = prow;
+            const int col = idx - row * vec_per_row;
+            const float sf = mode == 0 ? quant_scale<0>(amax_bits[row]) : quant_scale<1>(amax_bits[row]);
+            const uint2 qv = mode == 0 ? quant_vec8<0>(xv[v], sf) : quant_vec8<1>(xv[v], sf);
+            *(uint2*)(lds_q + (size_t)row * kp + col * 8) = qv;
+            const int ones = 0x01010101;
+            part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, 0, false), false);
+            if (col == 0) sval[row] = sf;
+            if (blockIdx.x == 0) {
+                if (q_out) *(uint2*)(q_out + (size_t)idx * 8) = qv;
+                if (s_out && col == 0) s_out[row] = f32_to_bf16_rne(sf);
+            }
+        }
+        const int row0 = __builtin_amdgcn_readfirstlane(prow);
+        if (__builtin_amdgcn_ballot_w64(prow != row0) == 0) {
+            const int wsum = wave_sum_i32(part);
+            if (lane == 0 && row0 >= 0) atomicAdd(&qsum[row0], wsum);
+        } else if (prow >= 0) {
+            atomicAdd(&qsum[prow], part);
+        }
+    }
+    lds_barrier();
+
+    const bool tok_ok = p < M;
+    const int8_t* brow = lds_q + (size_t)(tok_ok ? p : 0) * kp + g * 16;
+    v4i acc = {0, 0, 0, 0};
+    for (int base = ks * UPW; base < units; base += S * UPW) {
+        if (base != ks * UPW) {
+#pragma unroll
+            for (int j = 0; j < UPW; ++j) {
+                const int u = base + j;
+                w[j] = __builtin_nontemporal_load(wrow + (size_t)(u < units ? u : units - 1) * 64);
+            }
+        }
+        // all B operands of the round first (independent LDS reads, one wait);
+        // a k-step past the end contributes nothing because its A operand is zero
+        v4i b[UPW];
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            const int u = base + j;
+            b[j] = *(const v4i*)(brow + (size_t)(u < units ? u : units - 1) * 64);
+        }
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            const uint32_t wj = (base + j < units) ? w[j] : 0u;
+            v4i a;
+            a.x = (int)(wj & 0x03030303u);
+            a.y = (int)((wj >> 2) & 0x03030303u);
+            a.z = (int)((wj >> 4) & 0x03030303u);
+            a.w = (int)((wj >> 6) & 0x03030303u);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[j], acc, 0, 0, 0);
+        }
+    }
+
+    if (tok_ok) {  // lane holds token p, rows 4g + i in register i
+        int* dst = red + rbl * 256 + lane;
+        atomicAdd(dst, acc.x);
+        atomicAdd(dst + 64, acc.y);
+        atomicAdd(dst + 128, acc.z);
+        atomicAdd(dst + 192, acc.w);
+    }
+    lds_barrier();
+
+#pragma unroll
+    for (int r = 0; r < kFusedMaxRB; ++r) {
+        const int t = tid + r * nthreads;
+        if (t >= RB * 256) break;
+        const int l = t & 63;
+        const int m = l & 15;
+        const int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
+        if (m < M && n < N) {
+            const int sum = red[t] - 2 * qsum[m];
+            out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sval[m] * bf16_to_f32(e_wsb[r]));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 thread_local int g_status = BITLINEAR_OK;
 int g_tune_waves = 0;
 int g_tune_upw = 0;
 int g_tune_decode_waves = 0;
-int g_tune_path = 0;  // 0 = built-in choice, 2 = always the split-K kernel
+int g_tune_path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse
+int g_tune_fused[3] = {1, 10, 4};
 
 int set_status(int st) {
     g_status = st;
@@ -457,6 +674,77 @@ int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
+// Launch shape of the fused kernel: RB 16-row blocks per workgroup, S waves
+// splitting K for each, UPW 64-wide k-steps in flight per wave.
+struct FusedPlan {
+    int rb, s, upw, vmax;
+    bool ok;
+};
+
+FusedPlan plan_fused(int M, int N, int K) {
+    FusedPlan pl = {1, 1, 4, 1, false};
+    if (M > kFusedMaxTokens) return pl;
+    if ((size_t)M * (K + kFusedRowPad) > 60u * 1024u) return pl;
+    const int units = K / 64;
+    if (g_tune_path == 3) {
+        pl.rb = g_tune_fused[0];
+        pl.s = g_tune_fused[1];
+        pl.upw = g_tune_fused[2];
+    } else {
+        // enough row blocks per workgroup to keep about 200 workgroups; up to
+        // 8 waves splitting K for each, with the fewest k-steps per wave that fit
+        const int blocks16 = N / 16;
+        pl.rb = blocks16 / 216;
+        pl.rb = pl.rb < 1 ? 1 : (pl.rb > kFusedMaxRB ? kFusedMaxRB : pl.rb);
+        const int max_s = (kMaxWaves / pl.rb) < 8 ? (kMaxWaves / pl.rb) : 8;
+        const int sizes[5] = {4, 5, 8, 10, 16};
+        pl.upw = 16;
+        for (int i = 0; i < 5; ++i)
+            if ((units + sizes[i] - 1) / sizes[i] <= max_s) {
+                pl.upw = sizes[i];
+                break;
+            }
+        pl.s = (units + pl.upw - 1) / pl.upw;
+        if (pl.s > max_s) pl.s = max_s;
+    }
+    const int nthreads = 64 * pl.rb * pl.s;
+    const int nvec = M * (K / 8);
+    const int need = (nvec + nthreads - 1) / nthreads;
+    pl.vmax = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
+    pl.ok = need <= 4;
+    return pl;
+}
+
+int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const uint16_t* ws, const ScaleMap& smap,
+                 int8_t* q_out, uint16_t* s_out, int M, int N, int K, int mode, const FusedPlan& pl,
+                 hipStream_t stream) {
+    const int blocks16 = N / 16;
+    const dim3 grid((blocks16 + pl.rb - 1) / pl.rb, 1, 1);
+    const dim3 block(64 * pl.rb * pl.s, 1, 1);
+    const size_t lds = (size_t)M * (K + kFusedRowPad);
+    const uint32_t* wq = (const uint32_t*)packed;
+#define BITLINEAR_LAUNCH_UV(U, V)                                                                              \
+    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
+                       s_out, M, N, K, pl.rb, pl.s, mode)
+#define BITLINEAR_LAUNCH_U(U)                      \
+    switch (pl.vmax) {                             \
+        case 1: BITLINEAR_LAUNCH_UV(U, 1); break;  \
+        case 2: BITLINEAR_LAUNCH_UV(U, 2); break;  \
+        default: BITLINEAR_LAUNCH_UV(U, 4); break; \
+    }
+    switch (pl.upw) {
+        case 2: BITLINEAR_LAUNCH_U(2); break;
+        case 4: BITLINEAR_LAUNCH_U(4); break;
+        case 5: BITLINEAR_LAUNCH_U(5); break;
+        case 8: BITLINEAR_LAUNCH_U(8); break;
+        case 10: BITLINEAR_LAUNCH_U(10); break;
+        default: BITLINEAR_LAUNCH_U(16); break;
+    }
+#undef BITLINEAR_LAUNCH_U
+#undef BITLINEAR_LAUNCH_UV
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
 int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                 const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     // vector loads: 16-byte groups of both operands must be 16-byte aligned
@@ -500,24 +788,36 @@ int bitlinear_ws_num(int N, int K) {
     return 1;
 }
 
-int bitlinear_set_tuning(int kernel, int waves_per_group, int ksteps_in_flight) {
+int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     if (kernel == 0) {
         g_tune_path = g_tune_waves = g_tune_upw = g_tune_decode_waves = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 1) {
-        if (waves_per_group < 1 || waves_per_group > kDecodeMaxWaves) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 1 || a > kDecodeMaxWaves) return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 1;
-        g_tune_decode_waves = waves_per_group;
+        g_tune_decode_waves = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 2) {
-        const int u = ksteps_in_flight;
-        if (waves_per_group < 1 || waves_per_group > kMaxWaves || !(u == 1 || u == 2 || u == 4 || u == 8 || u == 16))
+        if (a < 1 || a > kMaxWaves || !(b == 1 || b == 2 || b == 4 || b == 8 || b == 16))
             return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 2;
-        g_tune_waves = waves_per_group;
-        g_tune_upw = u;
+        g_tune_waves = a;
+        g_tune_upw = b;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 3) {
+        const bool upw_ok = c == 2 || c == 4 || c == 5 || c == 8 || c == 10 || c == 16;
+        if (a < 1 || a > kFusedMaxRB || b < 1 || a * b > kMaxWaves || !upw_ok) return set_status(BITLINEAR_ERR_ARG);
+        g_tune_path = 3;
+        g_tune_fused[0] = a;
+        g_tune_fused[1] = b;
+        g_tune_fused[2] = c;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 4) {
+        g_tune_path = 4;
         return set_status(BITLINEAR_OK);
     }
     return set_status(BITLINEAR_ERR_ARG);
@@ -582,11 +882,18 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s, int M, int
 int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
                            int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
-    if (!x || !packed || !output0 || !ws || !q_ws || !s_ws) return set_status(BITLINEAR_ERR_NULL);
+    if (!x || !packed || !output0 || !ws) return set_status(BITLINEAR_ERR_NULL);
+    if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
+    if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)q_ws)) & 15u) return set_status(BITLINEAR_ERR_ARG);
+    const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    const FusedPlan pl = plan_fused(M, N, K);
+    if (pl.ok && g_tune_path != 4)
+        return set_status(launch_fused(x, packed, output0, ws, sm, q_ws, s_ws, M, N, K, mode, pl, (hipStream_t)stream));
+    // activation block too large to quantize inside every workgroup: two kernels
+    if (!q_ws || !s_ws) return set_status(BITLINEAR_ERR_NULL);
     const int st = bitlinear_quant_absmax(x, q_ws, s_ws, M, K, mode, stream);
     if (st != BITLINEAR_OK) return st;
-    return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, equal_slots(N, bitlinear_ws_num(N, K)), M,
-                                  N, K, (hipStream_t)stream));
+    return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream));
 }
 
 }  // extern "C"

@@ -104,10 +104,16 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s,
                            int M, int K, int mode, void* stream);
 
 /*
- * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer
- * (mode as above) then bitlinear_int8xint2.  q_ws (int8 [M, K]) and s_ws
- * (bf16 [M]) are caller-provided workspaces that receive the quantized
- * activations and scales.
+ * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer (mode
+ * as above), product and epilogue.  While the activation block is small
+ * (M <= 16, M * (K + 64) <= 60 KiB and at most 4 vectors of 8 values per
+ * thread) this is ONE kernel: every workgroup quantizes x itself, keeps the
+ * int8 rows in LDS and never reads s from memory.  Larger blocks run the
+ * quantizer kernel and then the product kernel.
+ *   q_ws (int8 [M, K]) and s_ws (bf16 [M]) receive the quantized activations
+ *   and scales; they may be NULL when the one-kernel path applies and are
+ *   required otherwise.  Results equal bitlinear_quant_absmax followed by
+ *   bitlinear_int8xint2 bit for bit.
  */
 int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
                            uint16_t* output0, const uint16_t* ws,
@@ -119,12 +125,15 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
  * results never depend on it.
  *   kernel 0: built-in choice (other arguments ignored)
  *   kernel 1: decode kernel where it applies (M <= 4, M*K <= 48 KiB) with
- *             waves_per_group (1..4) 16-row blocks per workgroup
- *   kernel 2: split-K kernel always, waves_per_group (1..16) waves per
- *             workgroup each keeping ksteps_in_flight (1, 2, 4, 8 or 16)
- *             64-wide k-steps in flight
+ *             a (1..4) 16-row blocks per workgroup
+ *   kernel 2: split-K kernel always, a (1..16) waves per workgroup each
+ *             keeping b (1, 2, 4, 8 or 16) 64-wide k-steps in flight
+ *   kernel 3: fused forward kernel with a (1..4) 16-row blocks per workgroup,
+ *             b waves splitting K for each (a*b <= 16), c (2, 4, 5, 8, 10 or
+ *             16) k-steps in flight per wave
+ *   kernel 4: bitlinear_forward_bf16 always as two kernels
  */
-int bitlinear_set_tuning(int kernel, int waves_per_group, int ksteps_in_flight);
+int bitlinear_set_tuning(int kernel, int a, int b, int c);
 
 #ifdef __cplusplus
 }

@@ -50,13 +50,16 @@ def test_host_only_entry_points():
     assert lib.bitlinear_ws_num(1024, 4096) == 1
     assert lib.bitlinear_status_string(0) == b"ok"
     assert b"shape" in lib.bitlinear_status_string(1)
-    assert lib.bitlinear_set_tuning(2, 8, 4) == 0
-    assert lib.bitlinear_set_tuning(2, 17, 4) != 0
-    assert lib.bitlinear_set_tuning(2, 8, 3) != 0
-    assert lib.bitlinear_set_tuning(1, 4, 0) == 0
-    assert lib.bitlinear_set_tuning(1, 5, 0) != 0
-    assert lib.bitlinear_set_tuning(3, 1, 1) != 0
-    assert lib.bitlinear_set_tuning(0, 0, 0) == 0
+    assert lib.bitlinear_set_tuning(2, 8, 4, 0) == 0
+    assert lib.bitlinear_set_tuning(2, 17, 4, 0) != 0
+    assert lib.bitlinear_set_tuning(2, 8, 3, 0) != 0
+    assert lib.bitlinear_set_tuning(1, 4, 0, 0) == 0
+    assert lib.bitlinear_set_tuning(1, 5, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(3, 1, 1, 0) != 0
+    assert lib.bitlinear_set_tuning(3, 2, 8, 5) == 0
+    assert lib.bitlinear_set_tuning(3, 4, 5, 4) != 0
+    assert lib.bitlinear_set_tuning(5, 0, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(0, 0, 0, 0) == 0
 
 
 def test_argument_checks_need_no_gpu(capfd):

@@ -25,7 +25,7 @@ def _need_gpu_and_lib():
     assert torch.cuda.is_available(), "these tests need the MI355X"
     _lib.load_library()  # raises if the HIP library is missing: no fallback
     yield
-    _lib.load_library().bitlinear_set_tuning(0, 0, 0)
+    _lib.load_library().bitlinear_set_tuning(0, 0, 0, 0)
 
 
 def _rand_case(n, k, m, seed, full_range=True):
@@ -171,11 +171,11 @@ def test_result_independent_of_kernel_and_launch_shape():
             settings = [(2, wv, u) for wv, u in [(1, 1), (2, 16), (3, 4), (7, 8), (16, 2), (16, 16), (5, 1)]]
             settings += [(1, 1, 0), (1, 2, 0), (1, 3, 0), (1, 4, 0), (0, 0, 0)]
             for setting in settings:
-                assert lib.bitlinear_set_tuning(*setting) == 0
+                assert lib.bitlinear_set_tuning(*setting, 0) == 0
                 acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
                 assert np.array_equal(acc.cpu().numpy(), want), (m, setting)
     finally:
-        lib.bitlinear_set_tuning(0, 0, 0)
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
 
 
 @pytest.mark.parametrize("n,k", [(16, 64), (16, 128), (48, 192), (80, 320), (32, 3200), (1040, 256)])
@@ -188,11 +188,81 @@ def test_decode_kernel_ragged_shapes(n, k, m):
     want = o.acc_int32(a, w)
     try:
         for waves in (1, 3, 4):
-            assert lib.bitlinear_set_tuning(1, waves, 0) == 0
+            assert lib.bitlinear_set_tuning(1, waves, 0, 0) == 0
             acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
             assert np.array_equal(acc.cpu().numpy(), want), waves
     finally:
-        lib.bitlinear_set_tuning(0, 0, 0)
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+
+
+def _forward_raw(lib, xb, pk, ws_bits, m, n, k, mode, with_ws=True):
+    import ctypes
+
+    x = dev_bf16(xb)
+    wsd = dev_bf16(ws_bits)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    q = torch.full((m, k), 99, dtype=torch.int8, device="cuda") if with_ws else None
+    s = torch.zeros(m, dtype=torch.bfloat16, device="cuda") if with_ws else None
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    st = lib.bitlinear_forward_bf16(P(x), P(pk), P(out), P(wsd), P(q), P(s), m, n, k, mode, None)
+    torch.cuda.synchronize()
+    return st, out, q, s
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (2560, 6912), (3840, 2560), (48, 192), (1040, 3200)])
+def test_fused_forward_equals_oracle_chain(n, k, m, mode):
+    """One-kernel forward (or its two-kernel form when the activation block is
+    too large) == oracle quantizer -> oracle product, bit for bit, including the
+    q / s workspaces it fills."""
+    lib = _lib.load_library()
+    rng = np.random.default_rng(n + k + m)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    if m > 1:
+        x[1, ::5] *= 20.0
+    xb = o.f32_to_bf16_bits(x)
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    q, s_bits = o.quant_input(xb, mode)
+    _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    st, out, qd, sd = _forward_raw(lib, xb, _packed_dev(w), ws_bits, m, n, k, mode)
+    assert st == 0
+    _assert_bits_equal(host_bits(out), want, "forward")
+    assert np.array_equal(qd.cpu().numpy(), q)
+    assert np.array_equal(host_bits(sd), s_bits)
+
+
+def test_fused_forward_launch_shapes_and_null_workspaces():
+    lib = _lib.load_library()
+    n, k = 2560, 2560
+    rng = np.random.default_rng(123)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    pk = _packed_dev(w)
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0, 0, 0], dtype=np.float32))
+    try:
+        for m in (1, 3, 4):
+            xb = o.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+            q, s_bits = o.quant_input(xb, 0)
+            _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+            for setting in [(3, 1, 10, 4), (3, 1, 5, 8), (3, 2, 5, 8), (3, 4, 4, 10), (3, 2, 8, 5), (3, 1, 16, 2),
+                            (3, 4, 1, 16), (3, 1, 3, 4), (4, 0, 0, 0), (0, 0, 0, 0)]:
+                assert lib.bitlinear_set_tuning(*setting) == 0
+                st, out, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
+                assert st == 0, setting
+                _assert_bits_equal(host_bits(out), want, f"forward {setting} M={m}")
+            lib.bitlinear_set_tuning(0, 0, 0, 0)
+            st, out, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0, with_ws=False)
+            assert st == 0
+            _assert_bits_equal(host_bits(out), want, "forward without workspaces")
+        # a block too large for the one-kernel path needs the workspaces
+        m, kk = 16, 6912
+        xb = o.f32_to_bf16_bits(rng.standard_normal((m, kk)).astype(np.float32))
+        wbig = rng.integers(-1, 2, size=(64, kk), dtype=np.int8)
+        st, _, _, _ = _forward_raw(lib, xb, _packed_dev(wbig), ws_bits, m, 64, kk, 0, with_ws=False)
+        assert st == 2
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
 
 
 def test_3d_input_and_out_argument():
