@@ -316,6 +316,170 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Prefill GEMM (M > 16): int8 MFMA 32x32x32, activations tiled through LDS
+// ---------------------------------------------------------------------------
+// out[m, n] = sum_k a[m, k] * w[n, k].  A workgroup of four waves owns a
+// (32*MT) x (128*NT) output tile; the waves sit side by side along n and share
+// the activation rows, which are staged through LDS in 64-k chunks (double
+// buffered, one LDS-only barrier per chunk).  Weights never touch LDS: one
+// packed word is the 16 k of one row that a lane needs as its B operand for a
+// 32-k step (column n = lane % 32, k-half = lane / 32), so each wave reads its
+// own words straight from global memory -- two full 128-byte tiles per step
+// and 32 columns -- expands them once (3 shifts + 4 ands) and reuses the
+// result for all MT row tiles.  The +2 bias of the codes is removed in the
+// epilogue with sum_k a[m, k], collected while the rows pass through staging.
+constexpr int kPfWaves = 4;
+constexpr int kPfChunk = 64;                   // k per LDS chunk = two MFMA k-steps
+constexpr int kPfRowBytes = kPfChunk + 16;     // padded row: conflict-free 16-byte reads
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int MT, int NT>
+__global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
+    int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
+    ScaleMap smap, int M, int N, int K) {
+    constexpr int TM = MT * 32;
+    constexpr int PPT = TM * 4 / (kPfWaves * 64);  // 16-byte pieces of a chunk per thread
+    __shared__ __attribute__((aligned(16))) int8_t lds_a[2][TM * kPfRowBytes];
+    __shared__ int rowsum[TM];
+    __shared__ float sval[TM];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int m0 = blockIdx.y * TM;
+    const int n0 = (blockIdx.x * kPfWaves + wave) * NT * 32;
+    const int nl = lane & 31;
+    const int kc = lane >> 5;
+    const int nchunks = K / kPfChunk;
+
+    // staging map: piece p = tid + i * 256 is 16 bytes of row p / 4, k-quarter p % 4
+    const int8_t* a_src[PPT];
+    int a_dst[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        const int pce = tid + i * kPfWaves * 64;
+        const int row = pce >> 2;
+        const int mrow = (m0 + row) < M ? (m0 + row) : (M - 1);
+        a_src[i] = act + (size_t)mrow * K + (pce & 3) * 16;
+        a_dst[i] = row * kPfRowBytes + (pce & 3) * 16;
+    }
+    // packed word of (column n, 32-k step, k-half kc); columns past N re-read column N-1
+    const uint32_t* w_src[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int n = n0 + nt * 32 + nl;
+        n = n < N ? n : N - 1;
+        w_src[nt] = wq + (size_t)(n >> 4) * K + ((n & 15) >> 3) * 16 + kc * 8 + (n & 7);
+    }
+    if (tid < TM) sval[tid] = bf16_to_f32(out ? s[(m0 + tid) < M ? (m0 + tid) : (M - 1)] : (uint16_t)0x3f80);
+
+    v16i acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0;
+    int rs[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) rs[i] = 0;
+
+    v4i areg[PPT];
+    uint32_t wcur[2][NT], wnext[2][NT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) areg[i] = *(const v4i*)(a_src[i]);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wcur[ks][nt] = w_src[nt][(size_t)ks * 32];
+    const int ones = 0x01010101;
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        *(v4i*)(&lds_a[0][a_dst[i]]) = areg[i];
+        rs[i] += __builtin_amdgcn_sdot4(areg[i].x, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].y, ones, 0, false) +
+                 __builtin_amdgcn_sdot4(areg[i].z, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].w, ones, 0, false);
+    }
+    lds_barrier();
+
+    for (int c = 0; c < nchunks; ++c) {
+        const bool more = (c + 1) < nchunks;
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < PPT; ++i) areg[i] = *(const v4i*)(a_src[i] + (size_t)(c + 1) * kPfChunk);
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) wnext[ks][nt] = w_src[nt][(size_t)((c + 1) * 2 + ks) * 32];
+        }
+        const int8_t* abuf = &lds_a[c & 1][0] + nl * kPfRowBytes + kc * 16;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v4i bop[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint32_t wd = wcur[ks][nt];
+                bop[nt].x = (int)(wd & 0x03030303u);
+                bop[nt].y = (int)((wd >> 2) & 0x03030303u);
+                bop[nt].z = (int)((wd >> 4) & 0x03030303u);
+                bop[nt].w = (int)((wd >> 6) & 0x03030303u);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const v4i aop = *(const v4i*)(abuf + mt * 32 * kPfRowBytes + ks * 32);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop[nt], acc[mt][nt], 0, 0, 0);
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < PPT; ++i) {
+                *(v4i*)(&lds_a[(c + 1) & 1][a_dst[i]]) = areg[i];
+                rs[i] += __builtin_amdgcn_sdot4(areg[i].x, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].y, ones, 0, false) +
+                         __builtin_amdgcn_sdot4(areg[i].z, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].w, ones, 0, false);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) wcur[ks][nt] = wnext[ks][nt];
+        }
+        lds_barrier();
+    }
+
+    // row sums: the four threads of a quad staged the four k-quarters of one row
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        int v = rs[i];
+        v += dpp_move<0xB1>(v);
+        v += dpp_move<0x4E>(v);
+        if ((tid & 3) == 0) rowsum[(tid + i * kPfWaves * 64) >> 2] = v;
+    }
+    lds_barrier();
+
+    // result lane: column n = lane % 32; register r is row (r / 4) * 8 + (lane / 32) * 4 + r % 4
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n = n0 + nt * 32 + nl;
+        if (n >= N) continue;
+        const float wsf = out ? bf16_to_f32(ws[scale_slot(smap, n)]) : 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ml = mt * 32 + (r >> 2) * 8 + kc * 4 + (r & 3);
+                const int m = m0 + ml;
+                if (m < M) {
+                    const int sum = acc[mt][nt][r] - 2 * rowsum[ml];
+                    if (acc_out) acc_out[(size_t)m * N + n] = sum;
+                    if (out) out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sval[ml] * wsf);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Per-token absmax quantizer: one workgroup per token row
 // ---------------------------------------------------------------------------
 constexpr int kQuantThreads = 256;
@@ -601,6 +765,8 @@ int g_tune_upw = 0;
 int g_tune_decode_waves = 0;
 int g_tune_path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse
 int g_tune_fused[3] = {1, 10, 4};
+int g_tune_prefill_big = 0;
+constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 
 int set_status(int st) {
     g_status = st;
@@ -745,10 +911,28 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
+int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
+                   const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+    const uint32_t* wq = (const uint32_t*)packed;
+    const dim3 block(kPfWaves * 64, 1, 1);
+    // large tile (128 x 256) once it still yields a few hundred workgroups, else 64 x 128
+    const long big_groups = (long)((M + 127) / 128) * ((N + 255) / 256);
+    const bool big = g_tune_path == 5 ? g_tune_prefill_big != 0 : big_groups >= 192;
+    if (big) {
+        const dim3 grid((N + 255) / 256, (M + 127) / 128, 1);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+    } else {
+        const dim3 grid((N + 127) / 128, (M + 63) / 64, 1);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+    }
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
 int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                 const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     // vector loads: 16-byte groups of both operands must be 16-byte aligned
     if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
+    if (M > kPrefillMinTokens && g_tune_path != 2) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
     const bool decode_fits = M <= kDecodeMaxTokens && (size_t)M * K <= (size_t)kDecodeMaxLdsBytes;
     // The one-wave-per-row-block kernel pays off once there are enough row
     // blocks to fill every SIMD; below that, splitting K across waves wins.
@@ -818,6 +1002,11 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     }
     if (kernel == 4) {
         g_tune_path = 4;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 5) {
+        g_tune_path = 5;
+        g_tune_prefill_big = a;
         return set_status(BITLINEAR_OK);
     }
     return set_status(BITLINEAR_ERR_ARG);

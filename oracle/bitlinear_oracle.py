@@ -204,7 +204,11 @@ def reference_supports(m: int, n: int, k: int) -> bool:
 def acc_int32(a: np.ndarray, w: np.ndarray) -> np.ndarray:
     """acc[m, n] = sum_k a[m, k] * w[n, k] with a int8 [M, K], w ternary
     int8 [N, K].  Computed in int64 and checked to fit int32."""
-    acc = a.astype(np.int64) @ w.astype(np.int64).T
+    if a.shape[0] * w.shape[0] * w.shape[1] <= (1 << 24):
+        acc = a.astype(np.int64) @ w.astype(np.int64).T
+    else:
+        # float64 BLAS: every product and partial sum is an integer below 2**53, hence exact
+        acc = np.rint(a.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64)
     assert np.all(np.abs(acc) < 2**31)
     return acc.astype(np.int32)
 

@@ -265,6 +265,75 @@ def test_fused_forward_launch_shapes_and_null_workspaces():
         lib.bitlinear_set_tuning(0, 0, 0, 0)
 
 
+@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("m,n,k", [(17, 48, 192), (64, 128, 64), (100, 272, 320), (128, 2560, 2560), (129, 3840, 2560),
+                                   (300, 1040, 3200), (512, 2560, 6912)])
+def test_prefill_gemm_acc_bit_exact(m, n, k, tile):
+    """MFMA GEMM path (M > 16), both tile sizes, ragged M and N."""
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=m + n + k)
+    try:
+        assert lib.bitlinear_set_tuning(5, tile, 0, 0) == 0
+        acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
+
+
+def test_prefill_extreme_values_and_split_k_agreement():
+    lib = _lib.load_library()
+    n, k, m = 256, 6912, 64
+    for wv, av in [(1, -128), (-1, -128), (1, 127)]:
+        w = np.full((n, k), wv, dtype=np.int8)
+        a = np.full((m, k), av, dtype=np.int8)
+        acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+        assert np.array_equal(acc.cpu().numpy(), np.full((m, n), wv * av * k, dtype=np.int32))
+    w, a = _rand_case(512, 1280, 96, seed=4)
+    pk, ad = _packed_dev(w), dev_i8(a)
+    acc_gemm = bitlinear.bitnet_int8xint2_acc(ad, pk).cpu().numpy()
+    try:
+        lib.bitlinear_set_tuning(2, 10, 4, 0)  # the split-K kernel, 16 tokens per workgroup
+        acc_splitk = bitlinear.bitnet_int8xint2_acc(ad, pk).cpu().numpy()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert np.array_equal(acc_gemm, acc_splitk)
+
+
+@pytest.mark.parametrize("shape_id,m", [(0, 128), (1, 2048), (2, 128), (3, 512)])
+def test_prefill_scaled_output_with_outliers(shape_id, m):
+    """Config 3: N(0,1) activations with 1% of entries x20, quantized per token
+    (two-kernel forward: the block is too large for the fused kernel)."""
+    sh = workload.shapes_2b()[shape_id]
+    w = workload.ternary_weight(sh.K, sh.N, shape_id)
+    ws_bits = workload.weight_scales(sh.K, sh.N, shape_id, sh.parts)
+    xb = workload.activations_bf16(m, sh.K, shape_id, outliers=True)
+    q, s_bits = o.quant_input(xb, o.QUANT_COMPILED)
+    _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    mod = bitlinear.BitLinearKernel(sh.K, sh.N).cuda()
+    mod.weight.data = _packed_dev(w)
+    mod.weight_scale.data = dev_bf16(ws_bits)
+    out = mod(dev_bf16(xb))
+    _assert_bits_equal(host_bits(out), want, f"{sh.name} prefill M={m}")
+
+
+def test_prefill_full_size_linearity_property():
+    """M = 2048 at the widest shape, checked without a CPU product: the result
+    for activations a + b equals the sum of the results for a and for b."""
+    n, k, m = 13824, 2560, 2048
+    rng = np.random.default_rng(8)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    a = rng.integers(-64, 64, size=(m, k), dtype=np.int8)
+    b = rng.integers(-63, 64, size=(m, k), dtype=np.int8)
+    pk = _packed_dev(w)
+    ra = bitlinear.bitnet_int8xint2_acc(dev_i8(a), pk)
+    rb = bitlinear.bitnet_int8xint2_acc(dev_i8(b), pk)
+    rab = bitlinear.bitnet_int8xint2_acc(dev_i8((a + b).astype(np.int8)), pk)
+    assert torch.equal(rab, ra + rb)
+    # and a few rows against the oracle
+    rows = [0, 1, 777, 2047]
+    assert np.array_equal(ra[rows].cpu().numpy(), o.acc_int32(a[rows], w))
+
+
 def test_3d_input_and_out_argument():
     n, k = 2560, 2560
     w, a = _rand_case(n, k, 6, seed=3)

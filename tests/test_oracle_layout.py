@@ -100,6 +100,13 @@ def test_acc_invariants():
     assert np.array_equal(o.acc_int32(a, pick), -a[:, np.arange(16) * 3].astype(np.int32))
 
 
+def test_acc_large_path_equals_integer_path():
+    rng = np.random.default_rng(12)
+    w = rng.integers(-1, 2, size=(272, 2560), dtype=np.int8)
+    a = rng.integers(-128, 128, size=(40, 2560), dtype=np.int8)  # 40*272*2560 > 2**24: float64 route
+    assert np.array_equal(o.acc_int32(a, w), (a.astype(np.int64) @ w.astype(np.int64).T).astype(np.int32))
+
+
 def test_ws_num_table_and_slots():
     assert o.ws_num_for_shape(3840, 2560) == 3
     assert o.ws_num_for_shape(2560, 2560) == 1
