@@ -320,17 +320,19 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
 // ---------------------------------------------------------------------------
 // out[m, n] = sum_k a[m, k] * w[n, k].  A workgroup of four waves owns a
 // (32*MT) x (128*NT) output tile; the waves sit side by side along n and share
-// the activation rows, which are staged through LDS in 64-k chunks (double
+// the activation rows, which are staged through LDS in 256-k chunks (double
 // buffered, one LDS-only barrier per chunk).  Weights never touch LDS: one
-// packed word is the 16 k of one row that a lane needs as its B operand for a
-// 32-k step (column n = lane % 32, k-half = lane / 32), so each wave reads its
+// packed word is the 16 k of one weight row that a lane needs as its MFMA row
+// operand for a 32-k step (row n = lane % 32, k-half = lane / 32), so each wave reads its
 // own words straight from global memory -- two full 128-byte tiles per step
 // and 32 columns -- expands them once (3 shifts + 4 ands) and reuses the
 // result for all MT row tiles.  The +2 bias of the codes is removed in the
 // epilogue with sum_k a[m, k], collected while the rows pass through staging.
 constexpr int kPfWaves = 4;
-constexpr int kPfChunk = 64;                   // k per LDS chunk = two MFMA k-steps
-constexpr int kPfRowBytes = kPfChunk + 16;     // padded row: conflict-free 16-byte reads
+constexpr int kPfSteps = 8;                     // 32-k MFMA steps per LDS chunk (256 k)
+constexpr int kPfChunk = kPfSteps * 32;
+constexpr int kPfRowBytes = kPfChunk + 16;      // padded row: 16-byte reads of 32 rows spread over the banks
+constexpr int kPfPieces = kPfChunk / 16;        // 16-byte pieces per row and chunk
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 template <int MT, int NT>
@@ -339,10 +341,12 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
     ScaleMap smap, int M, int N, int K) {
     constexpr int TM = MT * 32;
-    constexpr int PPT = TM * 4 / (kPfWaves * 64);  // 16-byte pieces of a chunk per thread
-    __shared__ __attribute__((aligned(16))) int8_t lds_a[2][TM * kPfRowBytes];
+    constexpr int NTHR = kPfWaves * 64;
+    constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
+    extern __shared__ __attribute__((aligned(16))) int8_t lds_a[];  // [2][TM * kPfRowBytes]
     __shared__ int rowsum[TM];
     __shared__ float sval[TM];
+    __shared__ float rinv[TM];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -351,18 +355,21 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int n0 = (blockIdx.x * kPfWaves + wave) * NT * 32;
     const int nl = lane & 31;
     const int kc = lane >> 5;
-    const int nchunks = K / kPfChunk;
+    const int ksteps = K >> 5;
+    const int nchunks = (ksteps + kPfSteps - 1) / kPfSteps;
 
-    // staging map: piece p = tid + i * 256 is 16 bytes of row p / 4, k-quarter p % 4
+    // staging map: piece p = tid + i * NTHR is 16 bytes of row p / kPfPieces at k-offset (p % kPfPieces) * 16
     const int8_t* a_src[PPT];
     int a_dst[PPT];
+    int a_koff[PPT];
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
-        const int pce = tid + i * kPfWaves * 64;
-        const int row = pce >> 2;
+        const int pce = tid + i * NTHR;
+        const int row = pce / kPfPieces;
         const int mrow = (m0 + row) < M ? (m0 + row) : (M - 1);
-        a_src[i] = act + (size_t)mrow * K + (pce & 3) * 16;
-        a_dst[i] = row * kPfRowBytes + (pce & 3) * 16;
+        a_koff[i] = (pce % kPfPieces) * 16;
+        a_src[i] = act + (size_t)mrow * K;
+        a_dst[i] = row * kPfRowBytes + a_koff[i];
     }
     // packed word of (column n, 32-k step, k-half kc); columns past N re-read column N-1
     const uint32_t* w_src[NT];
@@ -372,7 +379,11 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
         n = n < N ? n : N - 1;
         w_src[nt] = wq + (size_t)(n >> 4) * K + ((n & 15) >> 3) * 16 + kc * 8 + (n & 7);
     }
-    if (tid < TM) sval[tid] = bf16_to_f32(out ? s[(m0 + tid) < M ? (m0 + tid) : (M - 1)] : (uint16_t)0x3f80);
+    if (tid < TM) {
+        const float sv = bf16_to_f32(out ? s[(m0 + tid) < M ? (m0 + tid) : (M - 1)] : (uint16_t)0x3f80);
+        sval[tid] = sv;
+        rinv[tid] = 1.0f / sv;
+    }
 
     v16i acc[MT][NT];
 #pragma unroll
@@ -385,94 +396,164 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < PPT; ++i) rs[i] = 0;
 
+    // Software pipeline, two chunks deep.  While chunk c is multiplied out of
+    // LDS, chunk c+1 moves from registers into the other LDS buffer
+    // (activations) or waits in registers (weight words), and chunk c+2 is in
+    // flight from memory: every load has a whole multiply phase to land.
     v4i areg[PPT];
-    uint32_t wcur[2][NT], wnext[2][NT];
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) areg[i] = *(const v4i*)(a_src[i]);
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wcur[ks][nt] = w_src[nt][(size_t)ks * 32];
+    uint32_t wc[kPfSteps][NT], wn[kPfSteps][NT], wf[kPfSteps][NT];
+    const v4i zero4 = {0, 0, 0, 0};
     const int ones = 0x01010101;
+    auto load_chunk = [&](int c, uint32_t (&wdst)[kPfSteps][NT]) {
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-        *(v4i*)(&lds_a[0][a_dst[i]]) = areg[i];
-        rs[i] += __builtin_amdgcn_sdot4(areg[i].x, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].y, ones, 0, false) +
-                 __builtin_amdgcn_sdot4(areg[i].z, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].w, ones, 0, false);
-    }
+        for (int i = 0; i < PPT; ++i) {
+            const int k = c * kPfChunk + a_koff[i];
+            areg[i] = *(const v4i*)(a_src[i] + (k < K ? k : 0));  // past-the-end pieces are zeroed when staged
+        }
+#pragma unroll
+        for (int ks = 0; ks < kPfSteps; ++ks) {
+            const int st = c * kPfSteps + ks;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) wdst[ks][nt] = w_src[nt][(size_t)(st < ksteps ? st : ksteps - 1) * 32];
+        }
+    };
+    auto stage_chunk = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+            const v4i v = (c * kPfChunk + a_koff[i]) < K ? areg[i] : zero4;
+            *(v4i*)(lds_a + (c & 1) * (TM * kPfRowBytes) + a_dst[i]) = v;
+            rs[i] += __builtin_amdgcn_sdot4(v.x, ones, 0, false) + __builtin_amdgcn_sdot4(v.y, ones, 0, false) +
+                     __builtin_amdgcn_sdot4(v.z, ones, 0, false) + __builtin_amdgcn_sdot4(v.w, ones, 0, false);
+        }
+    };
+
+    load_chunk(0, wc);
+    stage_chunk(0);
+    load_chunk(1, wn);  // clamped if there is no second chunk
     lds_barrier();
 
+    // Per k-step, besides its MFMAs: one slice of the staging of chunk c+1 (LDS
+    // write + row-sum), the reload of that slice's registers for chunk c+2, this
+    // step's weight words for chunk c+2, and the LDS reads of the next step's A
+    // operands.  Spread like this the memory work issues in the shadow of the
+    // MFMAs (the matrix pipe runs a 32x32x32 for 32 cycles after a 4-cycle issue)
+    // instead of stopping all four waves at once.  Nothing is conditional: k past
+    // the end is staged as zeros and multiplies to nothing, surplus loads are clamped.
     for (int c = 0; c < nchunks; ++c) {
-        const bool more = (c + 1) < nchunks;
-        if (more) {
+        const int8_t* abuf = lds_a + (c & 1) * (TM * kPfRowBytes) + nl * kPfRowBytes + kc * 16;
+        int8_t* sbuf = lds_a + ((c + 1) & 1) * (TM * kPfRowBytes);
+        v4i aop[2][MT];
 #pragma unroll
-            for (int i = 0; i < PPT; ++i) areg[i] = *(const v4i*)(a_src[i] + (size_t)(c + 1) * kPfChunk);
+        for (int mt = 0; mt < MT; ++mt) aop[0][mt] = *(const v4i*)(abuf + mt * 32 * kPfRowBytes);
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < kPfSteps; ++ks) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) wnext[ks][nt] = w_src[nt][(size_t)((c + 1) * 2 + ks) * 32];
-        }
-        const int8_t* abuf = &lds_a[c & 1][0] + nl * kPfRowBytes + kc * 16;
+            for (int i = ks * PPT / kPfSteps; i < (ks + 1) * PPT / kPfSteps; ++i) {
+                const v4i v = ((c + 1) * kPfChunk + a_koff[i]) < K ? areg[i] : zero4;
+                *(v4i*)(sbuf + a_dst[i]) = v;
+                rs[i] += __builtin_amdgcn_sdot4(v.x, ones, 0, false) + __builtin_amdgcn_sdot4(v.y, ones, 0, false) +
+                         __builtin_amdgcn_sdot4(v.z, ones, 0, false) + __builtin_amdgcn_sdot4(v.w, ones, 0, false);
+                const int k = (c + 2) * kPfChunk + a_koff[i];
+                areg[i] = *(const v4i*)(a_src[i] + (k < K ? k : 0));
+            }
+            {
+                const int st = (c + 2) * kPfSteps + ks;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+                for (int nt = 0; nt < NT; ++nt) wf[ks][nt] = w_src[nt][(size_t)(st < ksteps ? st : ksteps - 1) * 32];
+            }
+            if (ks + 1 < kPfSteps) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    aop[(ks + 1) & 1][mt] = *(const v4i*)(abuf + mt * 32 * kPfRowBytes + (ks + 1) * 32);
+            }
             v4i bop[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const uint32_t wd = wcur[ks][nt];
+                const uint32_t wd = wc[ks][nt];
                 bop[nt].x = (int)(wd & 0x03030303u);
                 bop[nt].y = (int)((wd >> 2) & 0x03030303u);
                 bop[nt].z = (int)((wd >> 4) & 0x03030303u);
                 bop[nt].w = (int)((wd >> 6) & 0x03030303u);
             }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const v4i aop = *(const v4i*)(abuf + mt * 32 * kPfRowBytes + ks * 32);
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop[nt], acc[mt][nt], 0, 0, 0);
-            }
+                    acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bop[nt], aop[ks & 1][mt], acc[mt][nt], 0, 0, 0);
+            // keep each step's group together: left alone, the scheduler pulls the LDS reads
+            // back in front of their first use and exposes their latency
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (more) {
 #pragma unroll
-            for (int i = 0; i < PPT; ++i) {
-                *(v4i*)(&lds_a[(c + 1) & 1][a_dst[i]]) = areg[i];
-                rs[i] += __builtin_amdgcn_sdot4(areg[i].x, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].y, ones, 0, false) +
-                         __builtin_amdgcn_sdot4(areg[i].z, ones, 0, false) + __builtin_amdgcn_sdot4(areg[i].w, ones, 0, false);
+        for (int ks = 0; ks < kPfSteps; ++ks)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                wc[ks][nt] = wn[ks][nt];
+                wn[ks][nt] = wf[ks][nt];
             }
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) wcur[ks][nt] = wnext[ks][nt];
-        }
         lds_barrier();
     }
 
-    // row sums: the four threads of a quad staged the four k-quarters of one row
+    // row sums: the kPfPieces (= 16) threads of one DPP row staged the pieces of one activation row
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
         int v = rs[i];
         v += dpp_move<0xB1>(v);
         v += dpp_move<0x4E>(v);
-        if ((tid & 3) == 0) rowsum[(tid + i * kPfWaves * 64) >> 2] = v;
+        v += dpp_move<0x141>(v);
+        v += dpp_move<0x140>(v);
+        if ((tid & 15) == 0) rowsum[(tid + i * NTHR) / kPfPieces] = v;
     }
     lds_barrier();
 
-    // result lane: column n = lane % 32; register r is row (r / 4) * 8 + (lane / 32) * 4 + r % 4
+    // The weights are the MFMA's row operand, so a result lane holds one token
+    // (m = lane % 32 of the row tile) and, in register r, output column
+    // (r / 4) * 8 + (lane / 32) * 4 + r % 4 of the 32-column tile: four
+    // consecutive columns per register quad, stored as one 8-byte (bf16) or
+    // 16-byte (int32) piece.  Everything per token (row sum, scale, its
+    // reciprocal) is a single value per lane; the weight scales of the lane's
+    // 16 * NT columns are fetched once.
+    // Division by the token's scale: a correctly rounded reciprocal per token
+    // (one IEEE divide) and, per element, q0 = a * rinv refined by
+    // e = fma(-q0, s, a), q = fma(e, rinv, q0).
+    float wsf[NT][16];
+    if (out) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int n = n0 + nt * 32 + nl;
-        if (n >= N) continue;
-        const float wsf = out ? bf16_to_f32(ws[scale_slot(smap, n)]) : 0.0f;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int ml = mt * 32 + (r >> 2) * 8 + kc * 4 + (r & 3);
-                const int m = m0 + ml;
-                if (m < M) {
-                    const int sum = acc[mt][nt][r] - 2 * rowsum[ml];
-                    if (acc_out) acc_out[(size_t)m * N + n] = sum;
-                    if (out) out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sval[ml] * wsf);
+                const int n = n0 + nt * 32 + (r >> 2) * 8 + kc * 4 + (r & 3);
+                wsf[nt][r] = bf16_to_f32(ws[scale_slot(smap, n < N ? n : N - 1)]);
+            }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int ml = mt * 32 + nl;
+        const int m = m0 + ml;
+        const int rs2 = 2 * rowsum[ml];
+        const float sv = sval[ml], ri = rinv[ml];
+        if (m >= M) continue;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int n = n0 + nt * 32 + g4 * 8 + kc * 4;  // N % 16 == 0: the four columns are in or out together
+                if (n >= N) continue;
+                const size_t o = (size_t)m * N + n;
+                int sum[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sum[j] = acc[mt][nt][g4 * 4 + j] - rs2;
+                if (acc_out) *(v4i*)(acc_out + o) = v4i{sum[0], sum[1], sum[2], sum[3]};
+                if (out) {
+                    uint32_t h[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float a = (float)sum[j];
+                        const float q0 = a * ri;
+                        const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
+                        h[j] = f32_to_bf16_rne(q * wsf[nt][g4 * 4 + j]);
+                    }
+                    *(uint2*)(out + o) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
                 }
             }
         }
@@ -915,15 +996,26 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
                    const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     const uint32_t* wq = (const uint32_t*)packed;
     const dim3 block(kPfWaves * 64, 1, 1);
-    // large tile (128 x 256) once it still yields a few hundred workgroups, else 64 x 128
-    const long big_groups = (long)((M + 127) / 128) * ((N + 255) / 256);
-    const bool big = g_tune_path == 5 ? g_tune_prefill_big != 0 : big_groups >= 192;
-    if (big) {
+    // the large tile double-buffers 2 x 128 rows x 272 bytes = 68 KiB of LDS: above the 64 KiB a
+    // kernel gets without asking (a host-side attribute, set once per process)
+    static bool lds_limit_raised = false;
+    if (!lds_limit_raised) {
+        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<4, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  2 * 128 * kPfRowBytes);
+        lds_limit_raised = true;
+    }
+    // tile (rows x columns of the output per workgroup): 0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256
+    int tile = (N >= 8192 && M >= 512) ? 2 : 0;  // measured: the wide tile pays once there are many column tiles
+    if (g_tune_path == 5) tile = g_tune_prefill_big;
+    if (tile == 1) {
         const dim3 grid((N + 255) / 256, (M + 127) / 128, 1);
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+    } else if (tile == 2) {
+        const dim3 grid((N + 255) / 256, (M + 63) / 64, 1);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
     } else {
         const dim3 grid((N + 127) / 128, (M + 63) / 64, 1);
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
     }
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }

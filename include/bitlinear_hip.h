@@ -132,8 +132,8 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
  *             b waves splitting K for each (a*b <= 16), c (2, 4, 5, 8, 10 or
  *             16) k-steps in flight per wave
  *   kernel 4: bitlinear_forward_bf16 always as two kernels
- *   kernel 5: prefill GEMM (M > 16) with the 128 x 256 tile if a != 0, the
- *             64 x 128 tile if a == 0
+ *   kernel 5: prefill GEMM (M > 16) with output tile a per workgroup:
+ *             0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256 (tokens x columns)
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 
