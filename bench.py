@@ -166,6 +166,54 @@ def cpu_baseline(shapes, M, budget_s=12.0):
     }
 
 
+def end_to_end_decode(batches=(1, 8), prompt_len=512, gen_len=128):
+    """Random-init BitNet-b1.58-2B-shaped decoder (30 layers, dim 2560, ffn 6912,
+    20/5 heads, vocab 128256, tied bf16 embedding / LM head): a seeded 512-token
+    random-id prompt, then greedy decode steps replayed from a HIP graph;
+    tokens/s over the decode phase (as gpu/generate.py:264-288 counts it)."""
+    import torch
+
+    from bitnet_amd import decoder
+
+    dev = torch.device("cuda:0")
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            model = decoder.Transformer(decoder.ModelArgs())
+    finally:
+        torch.set_default_dtype(prev)
+    decoder.random_init_(model, seed=0)
+    out = {}
+    for B in batches:
+        gen = decoder.Generator(model, B, prompt_len + gen_len + 1, use_graph=True)
+        g = torch.Generator(device=dev).manual_seed(1234 + B)
+        prompt = torch.randint(0, model.args.vocab_size, (B, prompt_len), generator=g, device=dev)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        first = gen.prefill(prompt)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        gen.decode(first, prompt_len, 4)  # captures the graph, warms up
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        toks = gen.decode(first, prompt_len, gen_len - 1)
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        out[f"batch{B}"] = {
+            "decode_tokens_per_s": round(B * (gen_len - 1) / (t3 - t2), 1),
+            "ms_per_decode_step": round((t3 - t2) * 1e3 / (gen_len - 1), 4),
+            "prefill_tokens_per_s": round(B * prompt_len / (t1 - t0), 1),
+            "prompt_len": prompt_len,
+            "generated": gen_len,
+            "distinct_tokens_generated": int(torch.unique(toks).numel()),
+        }
+        del gen
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -174,6 +222,7 @@ def main():
     ap.add_argument("--m", type=int, default=1, help="tokens per step (decode batch), 1..16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end 2B decode measurement")
     ap.add_argument(
         "--pmc-probe",
         action="store_true",
@@ -329,6 +378,10 @@ def main():
         "per_shape_product_only": per_shape,
         "quantizer_us_per_launch": round(quant_us, 3),
     }
+    if not args.no_e2e:
+        del path, gemv, quant, layers
+        torch.cuda.empty_cache()
+        result["end_to_end_decode"] = end_to_end_decode()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(shapes, M, args.cpu_seconds)
     print(json.dumps(result))

@@ -673,16 +673,100 @@ constexpr int kFusedMaxRB = 4;
 constexpr int kFusedMaxTokens = 16;
 constexpr int kFusedRowPad = 64;  // bytes between token rows in LDS beyond K
 
-template <int UPW, int VMAX>
+// What the caller wants done to x before the quantizer, and to the result
+// after the epilogue.  All of it is what sits around a BitLinear in the
+// decoder (gpu/model.py:159-160, 195-196, 237-243 of the reference): the
+// sub-layer RMSNorms, the squared-ReLU gate, the residual add.
+struct FusedExtras {
+    const uint16_t* norm_weight;  // bf16 [K]; nullptr = no RMSNorm in front
+    const uint16_t* residual;     // bf16 [M, N]; nullptr = none; out = bf16(residual + bf16(result))
+    float eps;
+    int glu;                      // 1: x is [M, 2K] = (x1 | x3); h = bf16(bf16(relu(x1)^2) * x3) feeds the norm
+};
+
+__device__ __forceinline__ double dpp_sum_f64_row(double v) {
+    // adds v over each 16-lane row with the same four lane permutes as above, on both halves of the double
+#define BITLINEAR_DPP64(CTRL)                                                                      \
+    {                                                                                              \
+        const long long bits = __double_as_longlong(v);                                            \
+        const int lo = dpp_move<CTRL>((int)(bits & 0xffffffffll)), hi = dpp_move<CTRL>((int)(bits >> 32)); \
+        v += __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);                        \
+    }
+    BITLINEAR_DPP64(0xB1)
+    BITLINEAR_DPP64(0x4E)
+    BITLINEAR_DPP64(0x141)
+    BITLINEAR_DPP64(0x140)
+#undef BITLINEAR_DPP64
+    return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v = dpp_sum_f64_row(v);
+    double t = 0.0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const long long bits = __double_as_longlong(v);
+        const int lo = __builtin_amdgcn_readlane((int)(bits & 0xffffffffll), 16 * r);
+        const int hi = __builtin_amdgcn_readlane((int)(bits >> 32), 16 * r);
+        t += __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+    }
+    return t;
+}
+
+// 8 bf16 (as 4 dwords) -> sum of squares; every square of a bf16 is exact in
+// fp32 and the fp64 sum of a few thousand of them is exact for any data whose
+// magnitudes span less than 2^24, so the result does not depend on the order
+// of the additions.
+__device__ __forceinline__ double sumsq8(const uint4& v) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    double acc = 0.0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = __uint_as_float(d[i] << 16), hi = __uint_as_float(d[i] & 0xffff0000u);
+        acc += (double)(lo * lo) + (double)(hi * hi);
+    }
+    return acc;
+}
+
+// y = bf16(x * rstd * g) on 8 packed bf16
+__device__ __forceinline__ uint4 norm8(const uint4& v, const uint4& g, float rstd) {
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t w[4] = {g.x, g.y, g.z, g.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = __uint_as_float(d[i] << 16) * rstd * __uint_as_float(w[i] << 16);
+        const float hi = __uint_as_float(d[i] & 0xffff0000u) * rstd * __uint_as_float(w[i] & 0xffff0000u);
+        o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// h = bf16(bf16(relu(x1)^2) * x3) on 8 packed bf16
+__device__ __forceinline__ uint4 glu8(const uint4& a, const uint4& b) {
+    const uint32_t d[4] = {a.x, a.y, a.z, a.w};
+    const uint32_t e[4] = {b.x, b.y, b.z, b.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float r0 = fmaxf(__uint_as_float(d[i] << 16), 0.0f), r1 = fmaxf(__uint_as_float(d[i] & 0xffff0000u), 0.0f);
+        const float s0 = bf16_to_f32(f32_to_bf16_rne(r0 * r0)), s1 = bf16_to_f32(f32_to_bf16_rne(r1 * r1));
+        const float lo = s0 * __uint_as_float(e[i] << 16), hi = s1 * __uint_as_float(e[i] & 0xffff0000u);
+        o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+template <int UPW, int VMAX, int PRO>  // PRO 0: plain, 1: RMSNorm in front, 2: squared-ReLU gate + RMSNorm in front
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
-    int M, int N, int K, int RB, int S, int mode) {
+    FusedExtras ex, int M, int N, int K, int RB, int S, int mode) {
     extern __shared__ __attribute__((aligned(16))) int8_t lds_q[];  // [M][K + pad]
     __shared__ int red[kFusedMaxRB * 256];
     __shared__ uint32_t amax_bits[kFusedMaxTokens];
     __shared__ int qsum[kFusedMaxTokens];
     __shared__ float sval[kFusedMaxTokens];  // activation scale per token (a bf16 value)
+    __shared__ double sumsq[kFusedMaxTokens];
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -703,16 +787,21 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     // Activation block first: 16-byte vectors of 8 bf16, VMAX per thread.  The
     // memory counter retires loads in issue order, so what is needed first
     // (x) is requested first and the weight words stay outstanding behind it.
-    const int vec_per_row = K >> 3;
-    const int nvec = M * vec_per_row;
     // Loads are unconditional (indices clamped into range, surplus results
     // ignored later): a load under a branch would force a full wait for all
     // earlier loads at the first use of x.
-    uint4 xv[VMAX];
+    const int vec_per_row = K >> 3;
+    const int nvec = M * vec_per_row;
+    const int xstride = PRO == 2 ? 2 * K : K;  // elements between token rows of x
+    uint4 xv[VMAX], x3v[PRO == 2 ? VMAX : 1], gv[PRO != 0 ? VMAX : 1];
 #pragma unroll
     for (int v = 0; v < VMAX; ++v) {
-        const int idx = tid + v * nthreads;
-        xv[v] = *(const uint4*)(x + (size_t)(idx < nvec ? idx : nvec - 1) * 8);
+        const int idx = (tid + v * nthreads) < nvec ? (tid + v * nthreads) : (nvec - 1);
+        const int row = idx / vec_per_row;
+        const int col = idx - row * vec_per_row;
+        xv[v] = *(const uint4*)(x + (size_t)row * xstride + col * 8);
+        if (PRO == 2) x3v[v] = *(const uint4*)(x + (size_t)row * xstride + K + col * 8);
+        if (PRO != 0) gv[v] = *(const uint4*)(ex.norm_weight + col * 8);
     }
     // weight words of the first round
     uint32_t w[UPW];
@@ -721,21 +810,53 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         const int u = ks * UPW + j;
         w[j] = __builtin_nontemporal_load(wrow + (size_t)(u < units ? u : units - 1) * 64);
     }
-    // epilogue weight scale, raw bits, nothing depends on it until the end
-    uint16_t e_wsb[kFusedMaxRB];
+    // epilogue operands, raw bits, nothing depends on them until the end
+    uint16_t e_wsb[kFusedMaxRB], e_res[kFusedMaxRB];
 #pragma unroll
     for (int r = 0; r < kFusedMaxRB; ++r) {
         const int t = tid + r * nthreads;  // output slot t of the workgroup: [row block][reg][lane]
-        const int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
-        e_wsb[r] = ws[scale_slot(smap, n < N ? n : N - 1)];  // unconditional: no branch, no early wait
+        int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
+        n = n < N ? n : N - 1;
+        const int m = (t & 15) < M ? (t & 15) : M - 1;
+        e_wsb[r] = ws[scale_slot(smap, n)];  // unconditional: no branch, no early wait
+        e_res[r] = ex.residual ? ex.residual[(size_t)m * N + n] : (uint16_t)0;
     }
 
     for (int i = tid; i < RB * 256; i += nthreads) red[i] = 0;
     if (tid < kFusedMaxTokens) {
         amax_bits[tid] = 0u;
         qsum[tid] = 0;
+        sumsq[tid] = 0.0;
     }
     lds_barrier();
+
+    if (PRO != 0) {
+        // gate (PRO 2), then sum of squares per token row, then y = bf16(h * rstd * g)
+#pragma unroll
+        for (int v = 0; v < VMAX; ++v) {
+            const int idx = tid + v * nthreads;
+            const int row = idx < nvec ? idx / vec_per_row : -1;
+            if (PRO == 2) xv[v] = glu8(xv[v], x3v[v]);
+            const double sq = idx < nvec ? sumsq8(xv[v]) : 0.0;
+            const int row0 = __builtin_amdgcn_readfirstlane(row);
+            if (__builtin_amdgcn_ballot_w64(row != row0) == 0) {
+                const double wsum = wave_sum_f64(sq);
+                if (lane == 0 && row0 >= 0) atomicAdd(&sumsq[row0], wsum);
+            } else if (row >= 0) {
+                atomicAdd(&sumsq[row], sq);
+            }
+        }
+        lds_barrier();
+#pragma unroll
+        for (int v = 0; v < VMAX; ++v) {
+            const int idx = tid + v * nthreads;
+            if (idx < nvec) {
+                const float mean = (float)(sumsq[idx / vec_per_row] / (double)K);
+                const float rstd = 1.0f / __builtin_sqrtf(mean + ex.eps);
+                xv[v] = norm8(xv[v], gv[v], rstd);
+            }
+        }
+    }
 
     // one LDS atomic per wave and token row where the wave's 64 vectors lie in
     // one row (always so when K/8 is a multiple of 64); per lane otherwise
@@ -832,7 +953,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         const int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
         if (m < M && n < N) {
             const int sum = red[t] - 2 * qsum[m];
-            out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sval[m] * bf16_to_f32(e_wsb[r]));
+            uint16_t o = f32_to_bf16_rne((float)sum / sval[m] * bf16_to_f32(e_wsb[r]));
+            if (ex.residual) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
+            out[(size_t)m * N + n] = o;
         }
     }
 }
@@ -954,33 +1077,53 @@ FusedPlan plan_fused(int M, int N, int K) {
         pl.s = (units + pl.upw - 1) / pl.upw;
         if (pl.s > max_s) pl.s = max_s;
     }
-    const int nthreads = 64 * pl.rb * pl.s;
     const int nvec = M * (K / 8);
-    const int need = (nvec + nthreads - 1) / nthreads;
-    pl.vmax = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
-    pl.ok = need <= 4;
+    int need = (nvec + 64 * pl.rb * pl.s - 1) / (64 * pl.rb * pl.s);
+    if (need > 8 && g_tune_path != 3) {
+        // a large activation block: as many waves as a workgroup may have, so that every
+        // thread quantizes at most 8 vectors
+        pl.s = kMaxWaves / pl.rb;
+        const int per_wave = (units + pl.s - 1) / pl.s;
+        const int sizes[5] = {4, 5, 8, 10, 16};
+        pl.upw = 16;
+        for (int i = 0; i < 5; ++i)
+            if (sizes[i] >= per_wave) {
+                pl.upw = sizes[i];
+                break;
+            }
+        need = (nvec + 64 * pl.rb * pl.s - 1) / (64 * pl.rb * pl.s);
+    }
+    pl.vmax = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : 8));
+    pl.ok = need <= 8;
     return pl;
 }
 
 int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const uint16_t* ws, const ScaleMap& smap,
-                 int8_t* q_out, uint16_t* s_out, int M, int N, int K, int mode, const FusedPlan& pl,
-                 hipStream_t stream) {
+                 int8_t* q_out, uint16_t* s_out, const FusedExtras& ex, int M, int N, int K, int mode,
+                 const FusedPlan& pl, hipStream_t stream) {
     const int blocks16 = N / 16;
     const dim3 grid((blocks16 + pl.rb - 1) / pl.rb, 1, 1);
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
     const size_t lds = (size_t)M * (K + kFusedRowPad);
     const uint32_t* wq = (const uint32_t*)packed;
-#define BITLINEAR_LAUNCH_UV(U, V)                                                                              \
-    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
-                       s_out, M, N, K, pl.rb, pl.s, mode)
+    const int pro = ex.norm_weight ? (ex.glu ? 2 : 1) : 0;
+#define BITLINEAR_LAUNCH_UVP(U, V, P)                                                                             \
+    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
+                       s_out, ex, M, N, K, pl.rb, pl.s, mode)
+#define BITLINEAR_LAUNCH_UV(U, V)                    \
+    switch (pro) {                                   \
+        case 0: BITLINEAR_LAUNCH_UVP(U, V, 0); break; \
+        case 1: BITLINEAR_LAUNCH_UVP(U, V, 1); break; \
+        default: BITLINEAR_LAUNCH_UVP(U, V, 2); break; \
+    }
 #define BITLINEAR_LAUNCH_U(U)                      \
     switch (pl.vmax) {                             \
         case 1: BITLINEAR_LAUNCH_UV(U, 1); break;  \
         case 2: BITLINEAR_LAUNCH_UV(U, 2); break;  \
-        default: BITLINEAR_LAUNCH_UV(U, 4); break; \
+        case 4: BITLINEAR_LAUNCH_UV(U, 4); break;  \
+        default: BITLINEAR_LAUNCH_UV(U, 8); break; \
     }
     switch (pl.upw) {
-        case 2: BITLINEAR_LAUNCH_U(2); break;
         case 4: BITLINEAR_LAUNCH_U(4); break;
         case 5: BITLINEAR_LAUNCH_U(5); break;
         case 8: BITLINEAR_LAUNCH_U(8); break;
@@ -989,6 +1132,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     }
 #undef BITLINEAR_LAUNCH_U
 #undef BITLINEAR_LAUNCH_UV
+#undef BITLINEAR_LAUNCH_UVP
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
@@ -1084,7 +1228,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 3) {
-        const bool upw_ok = c == 2 || c == 4 || c == 5 || c == 8 || c == 10 || c == 16;
+        const bool upw_ok = c == 4 || c == 5 || c == 8 || c == 10 || c == 16;
         if (a < 1 || a > kFusedMaxRB || b < 1 || a * b > kMaxWaves || !upw_ok) return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 3;
         g_tune_fused[0] = a;
@@ -1169,12 +1313,27 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* ou
     const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
     const FusedPlan pl = plan_fused(M, N, K);
     if (pl.ok && g_tune_path != 4)
-        return set_status(launch_fused(x, packed, output0, ws, sm, q_ws, s_ws, M, N, K, mode, pl, (hipStream_t)stream));
+        return set_status(launch_fused(x, packed, output0, ws, sm, q_ws, s_ws, FusedExtras{nullptr, nullptr, 0.0f, 0}, M, N, K,
+                                       mode, pl, (hipStream_t)stream));
     // activation block too large to quantize inside every workgroup: two kernels
     if (!q_ws || !s_ws) return set_status(BITLINEAR_ERR_NULL);
     const int st = bitlinear_quant_absmax(x, q_ws, s_ws, M, K, mode, stream);
     if (st != BITLINEAR_OK) return st;
     return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream));
+}
+
+int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu,
+                                const int8_t* packed, const uint16_t* ws, const uint16_t* residual, uint16_t* output0,
+                                int M, int N, int K, int mode, void* stream) {
+    if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
+    if (!x || !norm_weight || !packed || !ws || !output0) return set_status(BITLINEAR_ERR_NULL);
+    if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
+    if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)norm_weight)) & 15u) return set_status(BITLINEAR_ERR_ARG);
+    const FusedPlan pl = plan_fused(M, N, K);
+    if (!pl.ok) return set_status(BITLINEAR_ERR_SHAPE);  // decode-sized activation blocks only
+    const FusedExtras ex = {norm_weight, residual, eps, glu ? 1 : 0};
+    return set_status(launch_fused(x, packed, output0, ws, equal_slots(N, bitlinear_ws_num(N, K)), nullptr, nullptr, ex, M,
+                                   N, K, mode, pl, (hipStream_t)stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,269 @@
+"""BitNet-b1.58-2B-shaped decoder on top of the BitLinear library: the caller
+of the hot path (gpu/model.py:87-296 and the decode loop of
+gpu/generate.py:159-213, 264-288 of the reference), kept to what a greedy
+decode benchmark needs.
+
+Same module tree and parameter names as the reference (``layers.N.attention.
+{wqkv,wo,attn_sub_norm}``, ``layers.N.feed_forward.{w13,w2,ffn_sub_norm}``,
+``attention_norm``, ``ffn_norm``, ``tok_embeddings``, ``norm``, ``output``), so a
+``model_state_int2.pt`` state dict loads with strict=True.  Where the reference
+leans on xformers (RMSNorm, rope_padded, flash attention on a padded KV cache),
+plain torch ops are used: RMSNorm and RoPE are closed forms, attention is
+softmax(QK^T/sqrt(d))V in fp32 over the cache.  One decode step is captured in
+a HIP graph and replayed per token, as the reference does with CUDA graphs.
+"""
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+from torch import nn
+
+from .bitlinear import BitLinearKernel
+
+
+@dataclass
+class ModelArgs:
+    # gpu/model.py:39-49
+    dim: int = 2560
+    n_layers: int = 30
+    n_heads: int = 20
+    n_kv_heads: int = 5
+    vocab_size: int = 128256
+    ffn_dim: int = 6912
+    norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+
+
+class RMSNorm(nn.Module):
+    """y = x * rsqrt(mean(x^2) + eps) * weight, evaluated in fp32 and rounded
+    to the input dtype once."""
+
+    def __init__(self, dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim), requires_grad=False)
+
+    def forward(self, x):
+        xf = x.float()
+        rstd = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        return (xf * rstd * self.weight.float()).to(x.dtype)
+
+
+def rope_tables(head_dim: int, max_seq: int, theta: float, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos / sin [max_seq, head_dim // 2] in fp32 for rotation of adjacent pairs."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=device, dtype=torch.float32) / head_dim))
+    ang = torch.outer(torch.arange(max_seq, device=device, dtype=torch.float32), inv)
+    return torch.cos(ang), torch.sin(ang)
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [..., n_heads, head_dim]; cos/sin broadcastable to [..., 1, head_dim/2].
+    Pairs (x[2i], x[2i+1]) are rotated by the angle of frequency i, in fp32."""
+    xf = x.float().unflatten(-1, (-1, 2))
+    a, b = xf[..., 0], xf[..., 1]
+    out = torch.stack((a * cos - b * sin, a * sin + b * cos), dim=-1)
+    return out.flatten(-2).to(x.dtype)
+
+
+class Attention(nn.Module):
+    def __init__(self, args: ModelArgs):
+        super().__init__()
+        self.head_dim = args.dim // args.n_heads
+        self.n_heads = args.n_heads
+        self.n_kv_heads = args.n_kv_heads
+        self.wqkv = BitLinearKernel(args.dim, (args.n_heads + 2 * args.n_kv_heads) * self.head_dim)
+        self.wo = BitLinearKernel(args.n_heads * self.head_dim, args.dim)
+        self.attn_sub_norm = RMSNorm(args.dim, args.norm_eps)
+
+    def split_qkv(self, xqkv):
+        nq = self.n_heads * self.head_dim
+        nk = self.n_kv_heads * self.head_dim
+        q = xqkv[..., :nq].unflatten(-1, (self.n_heads, self.head_dim))
+        k = xqkv[..., nq : nq + nk].unflatten(-1, (self.n_kv_heads, self.head_dim))
+        v = xqkv[..., nq + nk :].unflatten(-1, (self.n_kv_heads, self.head_dim))
+        return q, k, v
+
+    def attend(self, q, keys, values, mask):
+        """q [B, T, n_heads, d]; keys/values [B, S, n_kv, d]; mask [B, T, S] bool
+        (True = visible).  fp32 softmax(QK^T / sqrt(d)) V with grouped heads."""
+        B, T = q.shape[0], q.shape[1]
+        g = self.n_heads // self.n_kv_heads
+        qf = q.float().view(B, T, self.n_kv_heads, g, self.head_dim)
+        kf = keys.float()
+        vf = values.float()
+        scores = torch.einsum("btkgd,bskd->bkgts", qf, kf) * (self.head_dim ** -0.5)
+        scores = scores.masked_fill(~mask[:, None, None, :, :], float("-inf"))
+        probs = torch.softmax(scores, dim=-1)
+        out = torch.einsum("bkgts,bskd->btkgd", probs, vf)
+        return out.reshape(B, T, self.n_heads * self.head_dim).to(q.dtype)
+
+
+class FeedForward(nn.Module):
+    def __init__(self, args: ModelArgs):
+        super().__init__()
+        self.w13 = BitLinearKernel(args.dim, 2 * args.ffn_dim)
+        self.w2 = BitLinearKernel(args.ffn_dim, args.dim)
+        self.ffn_sub_norm = RMSNorm(args.ffn_dim, args.norm_eps)
+
+    def forward(self, x):
+        x13 = self.w13(x)
+        x1, x3 = x13.chunk(2, -1)
+        inner = self.ffn_sub_norm(torch.relu(x1) ** 2 * x3)  # squared-ReLU GLU, gpu/model.py:195
+        return self.w2(inner)
+
+
+class TransformerBlock(nn.Module):
+    def __init__(self, args: ModelArgs):
+        super().__init__()
+        self.attention = Attention(args)
+        self.feed_forward = FeedForward(args)
+        self.attention_norm = RMSNorm(args.dim, args.norm_eps)
+        self.ffn_norm = RMSNorm(args.dim, args.norm_eps)
+
+
+class Transformer(nn.Module):
+    """Decoder with an explicit KV cache [n_layers] x (k, v) of shape
+    [batch, max_seq, n_kv_heads, head_dim]."""
+
+    def __init__(self, args: ModelArgs):
+        super().__init__()
+        self.args = args
+        self.tok_embeddings = nn.Embedding(args.vocab_size, args.dim)
+        self.layers = nn.ModuleList([TransformerBlock(args) for _ in range(args.n_layers)])
+        self.norm = RMSNorm(args.dim, args.norm_eps)
+        self.output = nn.Linear(args.dim, args.vocab_size, bias=False)
+
+    def make_cache(self, batch: int, max_seq: int, device, dtype=torch.bfloat16) -> List[Tuple[torch.Tensor, torch.Tensor]]:
+        a = self.args
+        shape = (batch, max_seq, a.n_kv_heads, a.dim // a.n_heads)
+        return [(torch.zeros(shape, device=device, dtype=dtype), torch.zeros(shape, device=device, dtype=dtype))
+                for _ in range(a.n_layers)]
+
+    @torch.no_grad()
+    def forward_tokens(self, tokens, positions, cache, cos, sin):
+        """tokens [B, T] int64; positions [B, T] int64 (absolute position of every
+        token).  Writes k/v of these tokens into the cache at their positions
+        and attends to every cached position <= the token's own.  Works for
+        prefill (T = prompt length) and for decode (T = 1); all shapes are
+        static, so a decode step can be captured in a graph.  Returns logits
+        [B, T, vocab] in fp32."""
+        B, T = tokens.shape
+        S = cache[0][0].shape[1]
+        h = self.tok_embeddings(tokens)
+        c = cos[positions][:, :, None, :]
+        s = sin[positions][:, :, None, :]
+        mask = torch.arange(S, device=tokens.device)[None, None, :] <= positions[:, :, None]
+        bidx = torch.arange(B, device=tokens.device)[:, None].expand(B, T)
+        for layer, (ck, cv) in zip(self.layers, cache):
+            att = layer.attention
+            q, k, v = att.split_qkv(att.wqkv(layer.attention_norm(h)))
+            q = apply_rope(q, c, s)
+            k = apply_rope(k, c, s)
+            ck.index_put_((bidx, positions), k)
+            cv.index_put_((bidx, positions), v)
+            o = att.attend(q, ck, cv, mask)
+            h = h + att.wo(att.attn_sub_norm(o))
+            h = h + layer.feed_forward(layer.ffn_norm(h))
+        return self.output(self.norm(h)).float()
+
+
+def random_init_(model: Transformer, seed: int = 0) -> Transformer:
+    """Random weights of the benchmark configuration: BitLinear weights ternary
+    iid with P(0) = 0.4, P(+-1) = 0.3 packed in the int2 layout, one weight
+    scale per sub-tensor; embedding / LM head bf16 N(0, 0.02^2), tied as the
+    reference's converter ties them (gpu/convert_safetensors.py:88-89)."""
+    from .pack_weight import convert_weight_int8_to_int2
+
+    dev = model.tok_embeddings.weight.device
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    a = model.args
+    hd = a.dim // a.n_heads
+
+    def fill(mod: BitLinearKernel, parts):
+        N, K = mod.out_features, mod.in_features
+        u = torch.rand(N, K, generator=gen, device=dev)
+        w = (u >= 0.7).to(torch.int8) - (u < 0.3).to(torch.int8)
+        mod.weight.data = convert_weight_int8_to_int2(w, keep_device=True)
+        sc = torch.zeros(4, dtype=torch.float32, device=dev)
+        sc[: len(parts)] = 0.016 * (1.0 + 0.1 * torch.arange(len(parts), device=dev))
+        mod.weight_scale.data = sc.to(torch.bfloat16)
+
+    for layer in model.layers:
+        fill(layer.attention.wqkv, (a.n_heads * hd, a.n_kv_heads * hd, a.n_kv_heads * hd))
+        fill(layer.attention.wo, (a.dim,))
+        fill(layer.feed_forward.w13, (a.ffn_dim, a.ffn_dim))
+        fill(layer.feed_forward.w2, (a.dim,))
+    emb = torch.randn(a.vocab_size, a.dim, generator=gen, device=dev) * 0.02
+    model.tok_embeddings.weight.data = emb.to(model.tok_embeddings.weight.dtype)
+    model.output.weight.data = model.tok_embeddings.weight.data  # tied
+    return model
+
+
+class Generator:
+    """Greedy generation: prefill of the whole prompt in one call, then one
+    graph replay per generated token (gpu/generate.py:216-288)."""
+
+    def __init__(self, model: Transformer, batch: int, max_seq: int, use_graph: bool = True):
+        self.model = model
+        self.batch = batch
+        self.max_seq = max_seq
+        dev = model.tok_embeddings.weight.device
+        a = model.args
+        self.cos, self.sin = rope_tables(a.dim // a.n_heads, max_seq, a.rope_theta, dev)
+        self.cache = model.make_cache(batch, max_seq, dev)
+        self.tok = torch.zeros(batch, 1, dtype=torch.int64, device=dev)
+        self.pos = torch.zeros(batch, 1, dtype=torch.int64, device=dev)
+        self.next_tok = torch.zeros(batch, dtype=torch.int64, device=dev)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.use_graph = use_graph
+
+    def _step(self):
+        logits = self.model.forward_tokens(self.tok, self.pos, self.cache, self.cos, self.sin)
+        self.next_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
+
+    def _capture(self):
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self._step()  # warm-up outside the graph
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self._step()
+
+    @torch.no_grad()
+    def prefill(self, prompt: torch.Tensor) -> torch.Tensor:
+        """prompt [B, P] int64 -> first generated token [B]."""
+        B, P = prompt.shape
+        pos = torch.arange(P, device=prompt.device)[None, :].expand(B, P).contiguous()
+        logits = self.model.forward_tokens(prompt, pos, self.cache, self.cos, self.sin)
+        return torch.argmax(logits[:, -1, :], dim=-1)
+
+    @torch.no_grad()
+    def decode(self, first: torch.Tensor, start_pos: int, steps: int) -> torch.Tensor:
+        """Feeds `first` at position start_pos and generates `steps` further
+        tokens greedily.  Returns [steps, B]."""
+        out = torch.empty(steps, self.batch, dtype=torch.int64, device=first.device)
+        self.tok.copy_(first.view(-1, 1))
+        self.pos.fill_(start_pos)
+        if self.use_graph and self.graph is None:
+            # capture with the real inputs in place; the captured step is re-run below
+            saved_k = [ck.clone() for ck, _ in self.cache]
+            saved_v = [cv.clone() for _, cv in self.cache]
+            self._capture()
+            for (ck, cv), sk, sv in zip(self.cache, saved_k, saved_v):
+                ck.copy_(sk)
+                cv.copy_(sv)
+            self.tok.copy_(first.view(-1, 1))
+            self.pos.fill_(start_pos)
+        for i in range(steps):
+            if self.use_graph:
+                self.graph.replay()
+            else:
+                self._step()
+            out[i] = self.next_tok
+            self.tok.copy_(self.next_tok.view(-1, 1))
+            self.pos.add_(1)
+        return out

@@ -106,8 +106,8 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s,
 /*
  * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer (mode
  * as above), product and epilogue.  While the activation block is small
- * (M <= 16, M * (K + 64) <= 60 KiB and at most 4 vectors of 8 values per
- * thread) this is ONE kernel: every workgroup quantizes x itself, keeps the
+ * (M <= 16, M * (K + 64) <= 60 KiB and at most 8 vectors of 8 values per
+ * thread of a 1024-thread workgroup) this is ONE kernel: every workgroup quantizes x itself, keeps the
  * int8 rows in LDS and never reads s from memory.  Larger blocks run the
  * quantizer kernel and then the product kernel.
  *   q_ws (int8 [M, K]) and s_ws (bf16 [M]) receive the quantized activations
@@ -121,6 +121,29 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
                            int M, int N, int K, int mode, void* stream);
 
 /*
+ * bitlinear_forward_bf16 with the operations that surround a BitLinear in the
+ * reference's decoder folded into the same kernel (decode-sized activation
+ * blocks only: the one-kernel conditions of bitlinear_forward_bf16, else
+ * BITLINEAR_ERR_SHAPE):
+ *   in front  y = RMSNorm(h) = bf16(h * rsqrt(mean(h^2) + eps) * norm_weight)
+ *             (attention_norm / ffn_norm / attn_sub_norm / ffn_sub_norm,
+ *             gpu/model.py:159, 195, 228-229); the mean is taken in fp64 and
+ *             rounded to fp32, the two multiplies are fp32, one rounding to
+ *             bf16.  With glu != 0, x is [M, 2K] = (x1 | x3) and
+ *             h = bf16(bf16(relu(x1)^2) * x3) (gpu/model.py:164-166, 195);
+ *             otherwise h = x, [M, K].
+ *   behind    if residual != NULL: out = bf16(residual + bf16(result))
+ *             (gpu/model.py:237-243), residual bf16 [M, N].
+ *   norm_weight bf16 [K].  The reference uses xformers' RMSNorm, which is not
+ *   part of its tree: the rounding points above are this library's definition.
+ */
+int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
+                                float eps, int glu, const int8_t* packed,
+                                const uint16_t* ws, const uint16_t* residual,
+                                uint16_t* output0, int M, int N, int K,
+                                int mode, void* stream);
+
+/*
  * Kernel / launch-shape override for tuning runs and tests.  Process-wide;
  * results never depend on it.
  *   kernel 0: built-in choice (other arguments ignored)
@@ -129,8 +152,8 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
  *   kernel 2: split-K kernel always, a (1..16) waves per workgroup each
  *             keeping b (1, 2, 4, 8 or 16) 64-wide k-steps in flight
  *   kernel 3: fused forward kernel with a (1..4) 16-row blocks per workgroup,
- *             b waves splitting K for each (a*b <= 16), c (2, 4, 5, 8, 10 or
- *             16) k-steps in flight per wave
+ *             b waves splitting K for each (a*b <= 16), c (4, 5, 8, 10 or 16)
+ *             k-steps in flight per wave
  *   kernel 4: bitlinear_forward_bf16 always as two kernels
  *   kernel 5: prefill GEMM (M > 16) with output tile a per workgroup:
  *             0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256 (tokens x columns)

@@ -341,6 +341,52 @@ def fake_quant_input(x_bits: np.ndarray, mode: int = QUANT_COMPILED) -> np.ndarr
 
 
 # --------------------------------------------------------------------------
+# Operations around a BitLinear in the decoder  (gpu/model.py:159-166, 195, 237-243)
+# --------------------------------------------------------------------------
+
+
+def rmsnorm_bf16(h_bits: np.ndarray, g_bits: np.ndarray, eps: float) -> np.ndarray:
+    """y = bf16(h * rsqrt(mean(h^2) + eps) * g), rows of bf16 bit patterns.
+    The reference calls xformers' RMSNorm, which is not in its tree; the
+    rounding points are therefore a definition of this build: mean of squares
+    in float64 rounded to fp32, rsqrt as 1/sqrt in fp32, two fp32 multiplies,
+    one rounding to bf16.  Pinned against torch's fp32 RMSNorm within 1 bf16
+    ulp (it cannot be pinned tighter against a library that is absent)."""
+    h = bf16_bits_to_f32(h_bits)
+    g = bf16_bits_to_f32(g_bits)
+    k = h.shape[-1]
+    mean = (np.sum(h.astype(np.float64) ** 2, axis=-1, keepdims=True) / np.float64(k)).astype(np.float32)
+    rstd = (np.float32(1.0) / np.sqrt((mean + np.float32(eps)).astype(np.float32))).astype(np.float32)
+    return f32_to_bf16_bits(((h * rstd).astype(np.float32) * g).astype(np.float32))
+
+
+def squared_relu_glu_bf16(x13_bits: np.ndarray) -> np.ndarray:
+    """[M, 2K] = (x1 | x3) -> h = bf16(bf16(relu(x1)^2) * x3): the reference's
+    ``squared_relu(x1) * x3`` (gpu/model.py:164-166, 195) with a bf16 rounding
+    after the square and after the product, as torch eager gives."""
+    k = x13_bits.shape[-1] // 2
+    x1 = bf16_bits_to_f32(x13_bits[..., :k])
+    x3 = bf16_bits_to_f32(x13_bits[..., k:])
+    r = np.maximum(x1, np.float32(0.0))
+    sq = bf16_round((r * r).astype(np.float32))
+    return f32_to_bf16_bits((sq * x3).astype(np.float32))
+
+
+def residual_add_bf16(res_bits: np.ndarray, o_bits: np.ndarray) -> np.ndarray:
+    """bf16(res + o) as ``h = x + attention(...)`` does on bf16 tensors."""
+    return f32_to_bf16_bits((bf16_bits_to_f32(res_bits) + bf16_bits_to_f32(o_bits)).astype(np.float32))
+
+
+def norm_bitlinear(x_bits, g_bits, eps, w, ws_bits, glu=False, residual_bits=None, mode=QUANT_COMPILED, ws_num=None):
+    """[gate ->] RMSNorm -> quantizer -> product -> epilogue [-> residual add]."""
+    h = squared_relu_glu_bf16(x_bits) if glu else x_bits
+    y = rmsnorm_bf16(h, g_bits, eps)
+    q, s_bits = quant_input(y, mode)
+    _, out = bitlinear_int8xint2(q, w, s_bits, ws_bits, ws_num)
+    return residual_add_bf16(residual_bits, out) if residual_bits is not None else out
+
+
+# --------------------------------------------------------------------------
 # W: absmean ternarisation  (gpu/convert_checkpoint.py:23-27, 42-77)
 # --------------------------------------------------------------------------
 

@@ -245,7 +245,7 @@ def test_fused_forward_launch_shapes_and_null_workspaces():
             xb = o.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
             q, s_bits = o.quant_input(xb, 0)
             _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
-            for setting in [(3, 1, 10, 4), (3, 1, 5, 8), (3, 2, 5, 8), (3, 4, 4, 10), (3, 2, 8, 5), (3, 1, 16, 2),
+            for setting in [(3, 1, 10, 4), (3, 1, 5, 8), (3, 2, 5, 8), (3, 4, 4, 10), (3, 2, 8, 5), (3, 1, 16, 4),
                             (3, 4, 1, 16), (3, 1, 3, 4), (4, 0, 0, 0), (0, 0, 0, 0)]:
                 assert lib.bitlinear_set_tuning(*setting) == 0
                 st, out, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
@@ -332,6 +332,35 @@ def test_prefill_full_size_linearity_property():
     # and a few rows against the oracle
     rows = [0, 1, 777, 2047]
     assert np.array_equal(ra[rows].cpu().numpy(), o.acc_int32(a[rows], w))
+
+
+@pytest.mark.parametrize("glu,res", [(0, 0), (0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("m", [1, 2, 4, 8])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (3840, 2560), (2560, 6912), (48, 192), (1040, 3200)])
+def test_fused_norm_gate_residual_forward(n, k, m, glu, res):
+    """[gate ->] RMSNorm -> quantizer -> product -> epilogue [-> residual] in one
+    kernel against the oracle chain, bit for bit."""
+    import ctypes
+
+    lib = _lib.load_library()
+    if m * (k + 64) > 60 * 1024:
+        pytest.skip("activation block beyond the one-kernel limit")
+    rng = np.random.default_rng(n + k + m + 7 * glu + res)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    xin = rng.standard_normal((m, 2 * k if glu else k)).astype(np.float32) * 1.7
+    xb = o.f32_to_bf16_bits(xin)
+    gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+    rb = o.f32_to_bf16_bits(rng.standard_normal((m, n)).astype(np.float32)) if res else None
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=bool(glu), residual_bits=rb)
+    x, g, pk, wsd = dev_bf16(xb), dev_bf16(gb), _packed_dev(w), dev_bf16(ws_bits)
+    r = dev_bf16(rb) if res else None
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    st = lib.bitlinear_norm_forward_bf16(P(x), P(g), 1e-5, glu, P(pk), P(wsd), P(r), P(out), m, n, k, 0, None)
+    torch.cuda.synchronize()
+    assert st == 0
+    _assert_bits_equal(host_bits(out), want, f"norm forward glu={glu} res={res}")
 
 
 def test_3d_input_and_out_argument():

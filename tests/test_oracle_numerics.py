@@ -130,3 +130,28 @@ def test_fused_scales_layout():
     assert w.shape == (64, 64) and ws.shape == (4,) and ws[3] == 0
     for j, p in enumerate(parts):
         assert ws[j] == o.quant_weight_int8(p)[1][0]
+
+
+def test_glu_matches_torch_eager_and_norm_is_within_one_ulp_of_torch_fp32():
+    rng = np.random.default_rng(8)
+    x13 = o.f32_to_bf16_bits(rng.standard_normal((4, 512)).astype(np.float32))
+    t = _bf16(x13)
+    x1, x3 = t.chunk(2, -1)
+    ref = torch.relu(x1) ** 2 * x3  # gpu/model.py:164-166, 195 evaluated by torch eager on bf16
+    assert np.array_equal(o.squared_relu_glu_bf16(x13), _bits(ref))
+
+    h = o.f32_to_bf16_bits((rng.standard_normal((5, 2560)) * np.array([[1], [30], [0.01], [1], [1]])).astype(np.float32))
+    g = o.f32_to_bf16_bits((1.0 + 0.1 * rng.standard_normal(2560)).astype(np.float32))
+    got = o.rmsnorm_bf16(h, g, 1e-5)
+    hf = _bf16(h).float()
+    want = (hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + 1e-5) * _bf16(g).float()).to(torch.bfloat16)
+    a, b = got.astype(np.int32), _bits(want).astype(np.int32)
+    assert np.max(np.abs(a - b)) <= 1 and np.mean(a != b) < 0.01
+    # closed form: a constant row normalises to +-g (eps negligible)
+    c = o.f32_to_bf16_bits(np.full((1, 256), -3.0, dtype=np.float32))
+    g1 = o.f32_to_bf16_bits(np.linspace(0.5, 2.0, 256).astype(np.float32))
+    assert np.array_equal(o.rmsnorm_bf16(c, g1, 0.0)[0], o.f32_to_bf16_bits(-o.bf16_bits_to_f32(g1)))
+
+    r = o.f32_to_bf16_bits(rng.standard_normal(64).astype(np.float32))
+    v = o.f32_to_bf16_bits(rng.standard_normal(64).astype(np.float32))
+    assert np.array_equal(o.residual_add_bf16(r, v), _bits(_bf16(r) + _bf16(v)))
