@@ -13,7 +13,7 @@ import sys
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
-SRC = os.path.join(PKG_DIR, "csrc", "bitlinear_hip.hip")
+SOURCES = [os.path.join(PKG_DIR, "csrc", "bitlinear_hip.hip"), os.path.join(PKG_DIR, "csrc", "decoder_ops.hip")]
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libbitlinear_hip.so")
 
@@ -39,7 +39,7 @@ def hipcc_path() -> str:
 
 def build_library(verbose: bool = True) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", os.path.join(REPO_ROOT, "include"), SRC, "-o", LIB_PATH]
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", os.path.join(REPO_ROOT, "include"), *SOURCES, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

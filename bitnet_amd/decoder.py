@@ -18,7 +18,8 @@ from typing import List, Optional, Tuple
 import torch
 from torch import nn
 
-from .bitlinear import BitLinearKernel
+from . import _lib
+from .bitlinear import BitLinearKernel, _ptr, _stream_ptr
 
 
 @dataclass
@@ -63,6 +64,38 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     a, b = xf[..., 0], xf[..., 1]
     out = torch.stack((a * cos - b * sin, a * sin + b * cos), dim=-1)
     return out.flatten(-2).to(x.dtype)
+
+
+def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads):
+    """Rope + KV-cache write + grouped-query attention of one new token per
+    sequence in one HIP kernel (bitnet_attn_decode).  xqkv bf16 [B, (n_heads +
+    2 n_kv) * 128]; positions int64 [B]; returns bf16 [B, n_heads * 128]."""
+    B = xqkv.shape[0]
+    S = cache_k.shape[1]
+    hd = cache_k.shape[-1]
+    out = torch.empty(B, n_heads * hd, dtype=torch.bfloat16, device=xqkv.device)
+    st = _lib.load_library().bitnet_attn_decode(
+        _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out), B, S, n_heads,
+        n_kv_heads, hd, _stream_ptr(),
+    )
+    if st != 0:
+        raise _lib.BitLinearLibraryError(f"bitnet_attn_decode: status {st}")
+    return out
+
+
+def norm_bitlinear(x, norm: "RMSNorm", lin: BitLinearKernel, glu: bool = False, residual=None):
+    """[squared-ReLU gate ->] RMSNorm -> BitLinearKernel.forward [-> + residual]
+    as one kernel (bitlinear_norm_forward_bf16); x bf16 [M, K] (or [M, 2K] with
+    glu), decode-sized M."""
+    M = x.shape[0]
+    out = torch.empty(M, lin.out_features, dtype=torch.bfloat16, device=x.device)
+    st = _lib.load_library().bitlinear_norm_forward_bf16(
+        _ptr(x), _ptr(norm.weight), norm.eps, 1 if glu else 0, _ptr(lin.weight), _ptr(lin.weight_scale),
+        _ptr(residual) if residual is not None else None, _ptr(out), M, lin.out_features, lin.in_features,
+        lin.quant_mode, _stream_ptr(),
+    )
+    _lib.check(st, f"bitlinear_norm_forward_bf16(M={M}, N={lin.out_features}, K={lin.in_features})")
+    return out
 
 
 class Attention(nn.Module):
@@ -139,6 +172,32 @@ class Transformer(nn.Module):
         return [(torch.zeros(shape, device=device, dtype=dtype), torch.zeros(shape, device=device, dtype=dtype))
                 for _ in range(a.n_layers)]
 
+    def fused_decode_ok(self, batch: int) -> bool:
+        """One new token per sequence can take the five-kernels-per-layer path
+        when the library's one-kernel forward accepts the activation blocks."""
+        a = self.args
+        hd = a.dim // a.n_heads
+        return (hd == 128 and self.norm.weight.dtype == torch.bfloat16
+                and batch * (a.ffn_dim + 64) <= 60 * 1024 and batch <= 16)
+
+    @torch.no_grad()
+    def forward_decode_fused(self, tokens, positions, cache, cos, sin):
+        """One decode step, T = 1, five kernels per layer: norm+wqkv, rope+cache+
+        attention, sub-norm+wo+residual, norm+w13, gate+sub-norm+w2+residual.
+        tokens / positions [B, 1].  Returns logits [B, 1, vocab] fp32."""
+        a = self.args
+        B = tokens.shape[0]
+        pos = positions.reshape(B)
+        h = self.tok_embeddings(tokens.reshape(B))
+        for layer, (ck, cv) in zip(self.layers, cache):
+            att, ffn = layer.attention, layer.feed_forward
+            xqkv = norm_bitlinear(h, layer.attention_norm, att.wqkv)
+            o = attn_decode(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads)
+            h = norm_bitlinear(o, att.attn_sub_norm, att.wo, residual=h)
+            x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
+            h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)
+        return self.output(self.norm(h)).float().view(B, 1, -1)
+
     @torch.no_grad()
     def forward_tokens(self, tokens, positions, cache, cos, sin):
         """tokens [B, T] int64; positions [B, T] int64 (absolute position of every
@@ -204,8 +263,9 @@ class Generator:
     """Greedy generation: prefill of the whole prompt in one call, then one
     graph replay per generated token (gpu/generate.py:216-288)."""
 
-    def __init__(self, model: Transformer, batch: int, max_seq: int, use_graph: bool = True):
+    def __init__(self, model: Transformer, batch: int, max_seq: int, use_graph: bool = True, fused: bool = True):
         self.model = model
+        self.fused = fused and model.fused_decode_ok(batch)
         self.batch = batch
         self.max_seq = max_seq
         dev = model.tok_embeddings.weight.device
@@ -219,7 +279,8 @@ class Generator:
         self.use_graph = use_graph
 
     def _step(self):
-        logits = self.model.forward_tokens(self.tok, self.pos, self.cache, self.cos, self.sin)
+        fwd = self.model.forward_decode_fused if self.fused else self.model.forward_tokens
+        logits = fwd(self.tok, self.pos, self.cache, self.cos, self.sin)
         self.next_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
 
     def _capture(self):

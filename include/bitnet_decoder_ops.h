@@ -1,0 +1,43 @@
+/*
+ * Caller-side glue of the BitNet decoder around the BitLinear calls, exported
+ * from the same shared library as include/bitlinear_hip.h.  Plain C; device
+ * pointers owned by the caller; no allocation, no synchronisation, launches on
+ * the given stream (hipStream_t as void*), legal under graph capture.
+ */
+#ifndef BITNET_DECODER_OPS_H
+#define BITNET_DECODER_OPS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * One decode step of the attention block between wqkv and wo
+ * (Attention.forward, gpu/model.py:128-157, which calls xformers' rope_padded
+ * and flash attention on a padded KV cache): for every sequence b
+ *   - rotate q and k of the new token by the angles of position positions[b]
+ *     (adjacent pairs (2i, 2i+1), fp32, results rounded to bf16),
+ *   - write k, v into the cache at that position,
+ *   - out[b, h, :] = softmax(q_h . K[0..pos] / sqrt(head_dim)) V[0..pos] for the
+ *     n_heads query heads, head h using kv head h / (n_heads / n_kv_heads).
+ *   qkv      bf16 [B, (n_heads + 2 n_kv_heads) * head_dim]  (q | k | v)
+ *   cache_k/v bf16 [B, S, n_kv_heads, head_dim]
+ *   positions int64 [B], 0 <= positions[b] < S
+ *   cos/sin  fp32 [S, head_dim / 2]
+ *   out      bf16 [B, n_heads * head_dim]
+ * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8, and
+ * g * (S + 1024) * 4 bytes <= 96 KiB.  Returns 0, or 1 (shape),
+ * 2 (null pointer), 3 (launch failed).  fp32 accumulation; results agree with
+ * an fp32 evaluation of the same formula to about 1e-2 relative on bf16 outputs.
+ */
+int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v,
+                       const int64_t* positions, const float* cos_table,
+                       const float* sin_table, uint16_t* out, int B, int S,
+                       int n_heads, int n_kv_heads, int head_dim, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITNET_DECODER_OPS_H */

@@ -12,9 +12,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_functions():
-    text = open(os.path.join(ROOT, "include", "bitlinear_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return re.findall(r"\b(bitlinear_[a-z0-9_]+)\s*\(", text)
+    names = []
+    for header in ("bitlinear_hip.h", "bitnet_decoder_ops.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"\b(bit(?:linear|net)_[a-z0-9_]+)\s*\(", text)
+    return names
 
 
 def test_header_declares_the_drop_in_symbol():
