@@ -37,8 +37,11 @@ SIGNATURES = {
     ),
     "bitnet_attn_decode": (
         _c_int,
-        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_ptr],
     ),
+    "bitnet_attn_decode_workspace_floats": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
+    "bitnet_attn_decode_set_threads": (_c_int, [_c_int]),
     "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
 }
 

@@ -819,7 +819,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         n = n < N ? n : N - 1;
         const int m = (t & 15) < M ? (t & 15) : M - 1;
         e_wsb[r] = ws[scale_slot(smap, n)];  // unconditional: no branch, no early wait
-        e_res[r] = ex.residual ? ex.residual[(size_t)m * N + n] : (uint16_t)0;
+        // also unconditional: without a residual the load re-reads a weight scale and is ignored
+        const uint16_t* rp = ex.residual ? ex.residual : ws;
+        e_res[r] = rp[ex.residual ? (size_t)m * N + n : 0];
     }
 
     for (int i = tid; i < RB * 256; i += nthreads) red[i] = 0;
@@ -851,7 +853,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         for (int v = 0; v < VMAX; ++v) {
             const int idx = tid + v * nthreads;
             if (idx < nvec) {
-                const float mean = (float)(sumsq[idx / vec_per_row] / (double)K);
+                const float mean = (float)sumsq[idx / vec_per_row] / (float)K;
                 const float rstd = 1.0f / __builtin_sqrtf(mean + ex.eps);
                 xv[v] = norm8(xv[v], gv[v], rstd);
             }
@@ -1061,12 +1063,13 @@ FusedPlan plan_fused(int M, int N, int K) {
         pl.s = g_tune_fused[1];
         pl.upw = g_tune_fused[2];
     } else {
-        // enough row blocks per workgroup to keep about 200 workgroups; up to
-        // 8 waves splitting K for each, with the fewest k-steps per wave that fit
+        // enough row blocks per workgroup to keep about 200 workgroups; up to 8
+        // (16 for K > 4096) waves splitting K for each, with the fewest k-steps per wave that fit
         const int blocks16 = N / 16;
         pl.rb = blocks16 / 216;
         pl.rb = pl.rb < 1 ? 1 : (pl.rb > kFusedMaxRB ? kFusedMaxRB : pl.rb);
-        const int max_s = (kMaxWaves / pl.rb) < 8 ? (kMaxWaves / pl.rb) : 8;
+        const int want_s = units > 64 ? kMaxWaves : 8;  // long rows: more threads share the prologue
+        const int max_s = (kMaxWaves / pl.rb) < want_s ? (kMaxWaves / pl.rb) : want_s;
         const int sizes[5] = {4, 5, 8, 10, 16};
         pl.upw = 16;
         for (int i = 0; i < 5; ++i)

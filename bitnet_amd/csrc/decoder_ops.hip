@@ -5,9 +5,14 @@
 // rope_padded and flash attention there); a floating-point kernel, checked
 // against a torch fp32 restatement within a stated tolerance.
 //
-// One workgroup per (kv head, sequence): the g = n_heads / n_kv_heads query
-// heads that share the kv head are processed together so every cached K / V
-// row is read once.  Phases: (1) rope + cache write, rotated q kept in LDS as
+// One workgroup per (kv head, sequence, split of the cached positions): the
+// g = n_heads / n_kv_heads query heads that share the kv head are processed
+// together so every cached K / V row is read once; splitting the positions
+// over several workgroups spreads the cache read over as many CUs (one CU
+// alone pulls well under 100 GB/s).  With more than one split every workgroup
+// leaves (unnormalised output, max, sum of exponentials) in a workspace and
+// the last one to finish -- an atomic counter per (sequence, kv head), reset
+// by that last workgroup -- merges them.  Phases: (1) rope + cache write, rotated q kept in LDS as
 // bf16; (2) scores with bf16 MFMA, 16 cached positions per wave and step; (3) softmax per head; (4) P.V with the positions split
 // over the waves and combined through LDS.
 
@@ -23,8 +28,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kHeadDim = 128;
 constexpr int kMaxGroup = 8;
-constexpr int kAttnThreads = 1024;
-constexpr int kAttnWaves = kAttnThreads / 64;
+constexpr int kAttnMinThreads = 256;
+constexpr int kAttnMaxThreads = 512;
 
 __device__ __forceinline__ float bf16f(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 __device__ __forceinline__ uint16_t to_bf16(float f) {
@@ -45,49 +50,104 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
     return v;
 }
 
+// Workspace record of one (sequence, kv head, split): G heads x (128 unnormalised outputs,
+// running maximum, sum of exponentials)
+constexpr int kRecFloats = kHeadDim + 2;
+constexpr int kMaxSplits = 8;
+
 template <int G>  // query heads per kv head
-__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
+__global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    uint16_t* __restrict__ out, int S, int n_heads, int n_kv_heads) {
-    extern __shared__ float sc[];  // [g][S] scores, then probabilities; then part[kAttnWaves][g][kHeadDim]
+    uint16_t* __restrict__ out, float* workspace, int* counters, int S, int span, int n_heads, int n_kv_heads) {
+    extern __shared__ float sc[];  // [G][span] scores, then probabilities; then part[nwaves][G][kHeadDim]
     __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
-    __shared__ float inv_sum[G];
+    __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
+    __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
+    __shared__ float red_m[G], red_l[G];
+    __shared__ int is_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int nthreads = blockDim.x;
+    const int nwaves = nthreads >> 6;
     const int kvh = blockIdx.x;
     const int b = blockIdx.y;
-    constexpr int g = G;
-    const int p = (int)positions[b];
+    const int sp = blockIdx.z;
+    const int nsplit = gridDim.z;
     const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
     const uint16_t* row = qkv + (size_t)b * row_elems;
     const size_t cache_row = (size_t)n_kv_heads * kHeadDim;  // elements between positions
     uint16_t* ck = cache_k + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
     uint16_t* cv = cache_v + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
-    float* part = sc + (size_t)g * S;
+    const int c = lane & 15, g4 = lane >> 4;
+    // This split owns positions [lo, lo + span): a fixed slice of the cache, whatever the current
+    // position is, so its rows can be requested before the position is known.  span % 16 == 0.
+    const int lo = sp * span;
+    float* part = sc + (size_t)G * span;
 
-    // (1) rope on adjacent pairs, in fp32, results rounded to bf16; k and v of the new
-    // token go to the cache, from where phases 2 and 4 read them like any other row
-    // (same workgroup, after a barrier)
-    for (int it = tid; it < (g + 2) * (kHeadDim / 2); it += kAttnThreads) {
+    // The kernel is a chain of memory round trips of a microsecond or more each, so everything
+    // that does not depend on anything else is requested first and at once: the position, this
+    // token's q / k / v, and the first round of cached K and V rows of the slice (row indices
+    // clamped to the cache; rows past the current position are ignored later, the row of the new
+    // token itself is patched in from LDS).
+    constexpr int R = 2;   // blocks of 16 positions per wave and round (K)
+    constexpr int U = 16;  // positions per wave and round (V)
+    constexpr int kItems = (G + 2) * (kHeadDim / 2);           // (head, pair) items of phase 1
+    constexpr int kIters = (kItems + kAttnMinThreads - 1) / kAttnMinThreads;
+    uint32_t praw[kIters];
+#pragma unroll
+    for (int u = 0; u < kIters; ++u) {
+        const int it = tid + u * nthreads;
         const int hh = it / (kHeadDim / 2);
         const int i = it - hh * (kHeadDim / 2);
-        if (hh < g + 1) {
-            const int src = hh < g ? (kvh * g + hh) * kHeadDim : (n_heads + kvh) * kHeadDim;
-            const uint32_t pr = *(const uint32_t*)(row + src + 2 * i);
-            const float a = bf16f(pr & 0xffffu), c = bf16f(pr >> 16);
-            const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
-            const uint16_t r0 = to_bf16(a * cs - c * sn), r1 = to_bf16(a * sn + c * cs);
-            if (hh < g) {
-                *(uint32_t*)(&qb[hh][2 * i]) = (uint32_t)r0 | ((uint32_t)r1 << 16);
-            } else {
-                *(uint32_t*)(ck + (size_t)p * cache_row + 2 * i) = (uint32_t)r0 | ((uint32_t)r1 << 16);
+        const int src = hh < G ? (kvh * G + hh) * kHeadDim : (hh == G ? (n_heads + kvh) : (n_heads + n_kv_heads + kvh)) * kHeadDim;
+        praw[u] = *(const uint32_t*)(row + (it < kItems ? src + 2 * i : 0));
+    }
+    uint4 kb[R][4];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int s = lo + wave * 16 + r * nwaves * 16 + c;
+        const uint16_t* kr = ck + (size_t)(s < S ? s : S - 1) * cache_row + g4 * 8;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) kb[r][kk] = *(const uint4*)(kr + kk * 32);
+    }
+    uint32_t vr[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+        const int s = lo + wave + j * nwaves;
+        vr[j] = *(const uint32_t*)(cv + (size_t)(s < S ? s : S - 1) * cache_row + 2 * lane);
+    }
+    const int p = (int)positions[b];
+    const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's positions are [lo, hi)
+    const bool owns_new = p >= lo && p < lo + span;
+
+    // (1) rope on adjacent pairs, in fp32, results rounded to bf16.  Every split needs q; the
+    // split that holds position p also rotates k, keeps k and v of the new token in LDS and
+    // writes them to the cache.
+#pragma unroll
+    for (int u = 0; u < kIters; ++u) {
+        const int it = tid + u * nthreads;
+        const int hh = it / (kHeadDim / 2);
+        const int i = it - hh * (kHeadDim / 2);
+        if (it < kItems) {
+            if (hh <= G) {
+                if (hh < G || owns_new) {
+                    const float a = bf16f(praw[u] & 0xffffu), cc = bf16f(praw[u] >> 16);
+                    const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
+                    const uint32_t rot = (uint32_t)to_bf16(a * cs - cc * sn) | ((uint32_t)to_bf16(a * sn + cc * cs) << 16);
+                    if (hh < G) {
+                        *(uint32_t*)(&qb[hh][2 * i]) = rot;
+                    } else {
+                        *(uint32_t*)(&knew[2 * i]) = rot;
+                        *(uint32_t*)(ck + (size_t)p * cache_row + 2 * i) = rot;
+                    }
+                }
+            } else if (owns_new) {
+                *(uint32_t*)(&vnew[2 * i]) = praw[u];
+                *(uint32_t*)(cv + (size_t)p * cache_row + 2 * i) = praw[u];
             }
-        } else {
-            const uint32_t pr = *(const uint32_t*)(row + (n_heads + n_kv_heads + kvh) * kHeadDim + 2 * i);
-            *(uint32_t*)(cv + (size_t)p * cache_row + 2 * i) = pr;
         }
     }
     __syncthreads();
@@ -98,7 +158,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     // lane % 16, i.e. one 16-byte piece of a K row.  Four steps cover the 128 dims.
     const float scale = 0.08838834764831845f;  // 128^-0.5
     {
-        const int c = lane & 15, g4 = lane >> 4;
         v8bf qa[4];
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
@@ -106,74 +165,79 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             if (c < G) t = *(const uint4*)(&qb[c][kk * 32 + g4 * 8]);
             qa[kk] = __builtin_bit_cast(v8bf, t);
         }
-        // R blocks of 16 positions per wave and round, all their K pieces requested before the first MFMA
-        constexpr int R = 3;
-        for (int s0 = wave * 16; s0 <= p; s0 += kAttnWaves * 16 * R) {
-            uint4 kb[R][4];
+        for (int s0 = lo + wave * 16; s0 < hi; s0 += nwaves * 16 * R) {
+            if (s0 != lo + wave * 16) {  // later rounds of a long slice
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int s = s0 + r * kAttnWaves * 16 + c;
-                const uint16_t* kr = ck + (size_t)(s <= p ? s : p) * cache_row + g4 * 8;
+                for (int r = 0; r < R; ++r) {
+                    const int s = s0 + r * nwaves * 16 + c;
+                    const uint16_t* kr = ck + (size_t)(s < S ? s : S - 1) * cache_row + g4 * 8;
 #pragma unroll
-                for (int kk = 0; kk < 4; ++kk) kb[r][kk] = *(const uint4*)(kr + kk * 32);
+                    for (int kk = 0; kk < 4; ++kk) kb[r][kk] = *(const uint4*)(kr + kk * 32);
+                }
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int s = s0 + r * kAttnWaves * 16 + c;
+                const int s = s0 + r * nwaves * 16 + c;
                 v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int kk = 0; kk < 4; ++kk)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[kk], __builtin_bit_cast(v8bf, kb[r][kk]), acc, 0, 0, 0);
+                for (int kk = 0; kk < 4; ++kk) {
+                    uint4 kv = kb[r][kk];
+                    if (s == p) kv = *(const uint4*)(&knew[kk * 32 + g4 * 8]);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[kk], __builtin_bit_cast(v8bf, kv), acc, 0, 0, 0);
+                }
                 // result lane: position c, heads 4 * g4 + j in register j
-                if (s <= p) {
+                if (s < hi) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        if (4 * g4 + j < G) sc[(size_t)(4 * g4 + j) * S + s] = acc[j] * scale;
+                        if (4 * g4 + j < G) sc[(size_t)(4 * g4 + j) * span + (s - lo)] = acc[j] * scale;
                 }
             }
         }
     }
     __syncthreads();
 
-    // (3) softmax over positions 0..p, one head per wave at a time
-    for (int hh = wave; hh < g; hh += kAttnWaves) {
-        float* srow = sc + (size_t)hh * S;
+    // (3) exp(score - max) over this split's positions, one head per wave at a time
+    for (int hh = wave; hh < G; hh += nwaves) {
+        float* srow = sc + (size_t)hh * span;
         float mx = -INFINITY;
-        for (int s = lane; s <= p; s += 64) mx = fmaxf(mx, srow[s]);
+        for (int s = lane; s < hi - lo; s += 64) mx = fmaxf(mx, srow[s]);
         mx = wave_max_f32(mx);
         float sum = 0.0f;
-        for (int s = lane; s <= p; s += 64) {
+        for (int s = lane; s < hi - lo; s += 64) {
             const float e = __expf(srow[s] - mx);
             srow[s] = e;
             sum += e;
         }
         sum = wave_sum_f32(sum);
-        if (lane == 0) inv_sum[hh] = 1.0f / sum;
+        if (lane == 0) {
+            red_m[hh] = mx;
+            red_l[hh] = sum;
+        }
     }
     __syncthreads();
 
-    // (4) out[hh][d] = sum_s prob[hh][s] * v[s][d]: every wave takes positions wave, wave + 16, ...
-    // for all g heads at once (a V row is read once), a lane owns dims 2*lane, 2*lane+1;
-    // 32 rows are requested per round so their latencies overlap
+    // (4) o[hh][d] = sum_s e[hh][s] * v[s][d]: every wave takes positions lo + wave, + W, ... for all G
+    // heads at once (a V row is read once), a lane owns dims 2*lane, 2*lane+1
     float a0[G], a1[G];
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) a0[hh] = a1[hh] = 0.0f;
-    constexpr int U = 32;
-    for (int s0 = wave; s0 <= p; s0 += kAttnWaves * U) {
-        uint32_t pr[U];
+    for (int s0 = lo + wave; s0 < hi; s0 += nwaves * U) {
+        if (s0 != lo + wave) {
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
-            const int s = s0 + j * kAttnWaves;
-            pr[j] = *(const uint32_t*)(cv + (size_t)(s <= p ? s : p) * cache_row + 2 * lane);
+            for (int j = 0; j < U; ++j) {
+                const int s = s0 + j * nwaves;
+                vr[j] = *(const uint32_t*)(cv + (size_t)(s < S ? s : S - 1) * cache_row + 2 * lane);
+            }
         }
 #pragma unroll
         for (int j = 0; j < U; ++j) {
-            const int s = s0 + j * kAttnWaves;
-            if (s <= p) {
-                const float v0 = bf16f(pr[j] & 0xffffu), v1 = bf16f(pr[j] >> 16);
+            const int s = s0 + j * nwaves;
+            if (s < hi) {
+                const uint32_t pr = s == p ? *(const uint32_t*)(&vnew[2 * lane]) : vr[j];
+                const float v0 = bf16f(pr & 0xffffu), v1 = bf16f(pr >> 16);
 #pragma unroll
                 for (int hh = 0; hh < G; ++hh) {
-                    const float pw = sc[(size_t)hh * S + s];
+                    const float pw = sc[(size_t)hh * span + (s - lo)];
                     a0[hh] += pw * v0;
                     a1[hh] += pw * v1;
                 }
@@ -182,36 +246,109 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     }
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
-        part[((size_t)wave * g + hh) * kHeadDim + 2 * lane] = a0[hh];
-        part[((size_t)wave * g + hh) * kHeadDim + 2 * lane + 1] = a1[hh];
+        part[((size_t)wave * G + hh) * kHeadDim + 2 * lane] = a0[hh];
+        part[((size_t)wave * G + hh) * kHeadDim + 2 * lane + 1] = a1[hh];
     }
     __syncthreads();
-    for (int hh = wave; hh < g; hh += kAttnWaves) {
+
+    uint16_t* orow = out + (size_t)b * n_heads * kHeadDim + (size_t)(kvh * G) * kHeadDim;
+    float* rec = workspace + ((size_t)(b * n_kv_heads + kvh) * nsplit) * G * kRecFloats;
+    for (int hh = wave; hh < G; hh += nwaves) {
         float o0 = 0.0f, o1 = 0.0f;
-#pragma unroll
-        for (int k = 0; k < kAttnWaves; ++k) {
-            o0 += part[((size_t)k * g + hh) * kHeadDim + 2 * lane];
-            o1 += part[((size_t)k * g + hh) * kHeadDim + 2 * lane + 1];
+        for (int k = 0; k < nwaves; ++k) {
+            o0 += part[((size_t)k * G + hh) * kHeadDim + 2 * lane];
+            o1 += part[((size_t)k * G + hh) * kHeadDim + 2 * lane + 1];
         }
-        const float is = inv_sum[hh];
-        const uint32_t pk = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
-        *(uint32_t*)(out + (size_t)b * n_heads * kHeadDim + (size_t)(kvh * g + hh) * kHeadDim + 2 * lane) = pk;
+        if (nsplit == 1) {
+            const float is = 1.0f / red_l[hh];
+            *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
+        } else {
+            float* r = rec + ((size_t)sp * G + hh) * kRecFloats;
+            r[2 * lane] = o0;
+            r[2 * lane + 1] = o1;
+            if (lane == 0) {
+                r[kHeadDim] = red_m[hh];  // -inf for a split with no positions
+                r[kHeadDim + 1] = red_l[hh];
+            }
+        }
+    }
+    if (nsplit == 1) return;
+
+    // the last split of this (sequence, kv head) to finish combines the records
+    __threadfence();  // make this workgroup's record visible device-wide before it is counted
+    __syncthreads();
+    if (tid == 0) {
+        const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = done == nsplit - 1;
+        if (is_last) __hip_atomic_store(&counters[b * n_kv_heads + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    for (int hh = wave; hh < G; hh += nwaves) {
+        // all records' loads first (independent), then the merge
+        float mk[kMaxSplits], lk[kMaxSplits], p0[kMaxSplits], p1[kMaxSplits];
+#pragma unroll
+        for (int k = 0; k < kMaxSplits; ++k) {
+            const float* r = rec + ((size_t)(k < nsplit ? k : 0) * G + hh) * kRecFloats;
+            mk[k] = __hip_atomic_load(r + kHeadDim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lk[k] = __hip_atomic_load(r + kHeadDim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            p0[k] = __hip_atomic_load(r + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            p1[k] = __hip_atomic_load(r + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < kMaxSplits; ++k)
+            if (k < nsplit) mx = fmaxf(mx, mk[k]);
+        float l = 0.0f, o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kMaxSplits; ++k) {
+            if (k < nsplit && lk[k] > 0.0f) {
+                const float w = __expf(mk[k] - mx);
+                l += lk[k] * w;
+                o0 += w * p0[k];
+                o1 += w * p1[k];
+            }
+        }
+        const float is = 1.0f / l;
+        *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
     }
 }
 
 }  // namespace
 
+static int g_attn_threads = 0;
+
+/* tuning override: threads per workgroup of the attention kernel (0 = built-in choice) */
+extern "C" int bitnet_attn_decode_set_threads(int threads) {
+    if (threads != 0 && threads != 256 && threads != 512) return 1;
+    g_attn_threads = threads;
+    return 0;
+}
+
+extern "C" int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits) {
+    if (B < 1 || n_heads < 1 || n_kv_heads < 1 || n_splits < 1 || n_heads % n_kv_heads) return -1;
+    return B * n_kv_heads * n_splits * (n_heads / n_kv_heads) * kRecFloats;
+}
+
 extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
-                                  const float* cos_table, const float* sin_table, uint16_t* out, int B, int S,
-                                  int n_heads, int n_kv_heads, int head_dim, void* stream) {
+                                  const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
+                                  int* counters, int n_splits, int B, int S, int n_heads, int n_kv_heads, int head_dim,
+                                  void* stream) {
     if (B < 1 || S < 1 || n_heads < 1 || n_kv_heads < 1 || head_dim != kHeadDim) return 1;
     if (n_heads % n_kv_heads) return 1;
     const int g = n_heads / n_kv_heads;
     if (g != 1 && g != 2 && g != 4 && g != 8) return 1;
+    if (n_splits < 1 || n_splits > kMaxSplits) return 1;
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
-    const size_t lds = ((size_t)g * S + (size_t)kAttnWaves * g * kHeadDim) * sizeof(float);
+    if (n_splits > 1 && (!workspace || !counters)) return 2;
+    const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // fixed slice of the cache per split
+    // more waves per workgroup keep more cache rows in flight; a slice of 64 rows per 4 waves is plenty
+    int threads = span >= 128 ? 512 : 256;
+    if (g_attn_threads) threads = g_attn_threads;
+    const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * g * kHeadDim) * sizeof(float);
     if (lds > 96u * 1024u) return 1;
-    const dim3 grid(n_kv_heads, B, 1), block(kAttnThreads, 1, 1);
+    const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
 #define BITNET_ATTN_LAUNCH(GG)                                                                                        \
     {                                                                                                                 \
         static bool raised = false; /* more than 64 KiB of dynamic LDS has to be asked for, once per process */     \
@@ -221,14 +358,13 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
             raised = true;                                                                                            \
         }                                                                                                             \
         hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, block, lds, (hipStream_t)stream, qkv, cache_k, cache_v,      \
-                           positions, cos_table, sin_table, out, S, n_heads, n_kv_heads);                            \
+                           positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads);       \
     }
     switch (g) {
         case 1: BITNET_ATTN_LAUNCH(1) break;
         case 2: BITNET_ATTN_LAUNCH(2) break;
         case 4: BITNET_ATTN_LAUNCH(4) break;
-        case 8: BITNET_ATTN_LAUNCH(8) break;
-        default: return 1;
+        default: BITNET_ATTN_LAUNCH(8) break;
     }
 #undef BITNET_ATTN_LAUNCH
     return hipGetLastError() == hipSuccess ? 0 : 3;

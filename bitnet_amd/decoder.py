@@ -66,7 +66,20 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return out.flatten(-2).to(x.dtype)
 
 
-def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads):
+class AttnWorkspace:
+    """Scratch of the split attention kernel: partial results of the splits and
+    one self-resetting arrival counter per (sequence, kv head).  One instance
+    serves all layers of a decoder (their kernels run one after the other)."""
+
+    def __init__(self, batch: int, n_heads: int, n_kv_heads: int, n_splits: int, device):
+        lib = _lib.load_library()
+        self.n_splits = n_splits
+        n = lib.bitnet_attn_decode_workspace_floats(batch, n_heads, n_kv_heads, n_splits)
+        self.partials = torch.empty(max(n, 1), dtype=torch.float32, device=device)
+        self.counters = torch.zeros(batch * n_kv_heads, dtype=torch.int32, device=device)
+
+
+def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads, workspace: "AttnWorkspace" = None):
     """Rope + KV-cache write + grouped-query attention of one new token per
     sequence in one HIP kernel (bitnet_attn_decode).  xqkv bf16 [B, (n_heads +
     2 n_kv) * 128]; positions int64 [B]; returns bf16 [B, n_heads * 128]."""
@@ -74,9 +87,12 @@ def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads
     S = cache_k.shape[1]
     hd = cache_k.shape[-1]
     out = torch.empty(B, n_heads * hd, dtype=torch.bfloat16, device=xqkv.device)
+    ns = workspace.n_splits if workspace is not None else 1
     st = _lib.load_library().bitnet_attn_decode(
-        _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out), B, S, n_heads,
-        n_kv_heads, hd, _stream_ptr(),
+        _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out),
+        _ptr(workspace.partials) if workspace is not None else None,
+        _ptr(workspace.counters) if workspace is not None else None,
+        ns, B, S, n_heads, n_kv_heads, hd, _stream_ptr(),
     )
     if st != 0:
         raise _lib.BitLinearLibraryError(f"bitnet_attn_decode: status {st}")
@@ -181,7 +197,7 @@ class Transformer(nn.Module):
                 and batch * (a.ffn_dim + 64) <= 60 * 1024 and batch <= 16)
 
     @torch.no_grad()
-    def forward_decode_fused(self, tokens, positions, cache, cos, sin):
+    def forward_decode_fused(self, tokens, positions, cache, cos, sin, workspace=None):
         """One decode step, T = 1, five kernels per layer: norm+wqkv, rope+cache+
         attention, sub-norm+wo+residual, norm+w13, gate+sub-norm+w2+residual.
         tokens / positions [B, 1].  Returns logits [B, 1, vocab] fp32."""
@@ -192,7 +208,7 @@ class Transformer(nn.Module):
         for layer, (ck, cv) in zip(self.layers, cache):
             att, ffn = layer.attention, layer.feed_forward
             xqkv = norm_bitlinear(h, layer.attention_norm, att.wqkv)
-            o = attn_decode(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads)
+            o = attn_decode(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads, workspace)
             h = norm_bitlinear(o, att.attn_sub_norm, att.wo, residual=h)
             x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
             h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)
@@ -266,6 +282,10 @@ class Generator:
     def __init__(self, model: Transformer, batch: int, max_seq: int, use_graph: bool = True, fused: bool = True):
         self.model = model
         self.fused = fused and model.fused_decode_ok(batch)
+        a_ = model.args
+        # enough splits of the cached positions that a few dozen CUs share every attention call
+        n_splits = max(1, min(8, 160 // max(1, batch * a_.n_kv_heads)))
+        self.attn_ws = AttnWorkspace(batch, a_.n_heads, a_.n_kv_heads, n_splits, model.tok_embeddings.weight.device)
         self.batch = batch
         self.max_seq = max_seq
         dev = model.tok_embeddings.weight.device
@@ -279,8 +299,10 @@ class Generator:
         self.use_graph = use_graph
 
     def _step(self):
-        fwd = self.model.forward_decode_fused if self.fused else self.model.forward_tokens
-        logits = fwd(self.tok, self.pos, self.cache, self.cos, self.sin)
+        if self.fused:
+            logits = self.model.forward_decode_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)
+        else:
+            logits = self.model.forward_tokens(self.tok, self.pos, self.cache, self.cos, self.sin)
         self.next_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
 
     def _capture(self):

@@ -127,8 +127,8 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
  * BITLINEAR_ERR_SHAPE):
  *   in front  y = RMSNorm(h) = bf16(h * rsqrt(mean(h^2) + eps) * norm_weight)
  *             (attention_norm / ffn_norm / attn_sub_norm / ffn_sub_norm,
- *             gpu/model.py:159, 195, 228-229); the mean is taken in fp64 and
- *             rounded to fp32, the two multiplies are fp32, one rounding to
+ *             gpu/model.py:159, 195, 228-229); the sum of squares is taken in fp64,
+ *             rounded to fp32 and divided by K in fp32; the two multiplies are fp32, one rounding to
  *             bf16.  With glu != 0, x is [M, 2K] = (x1 | x3) and
  *             h = bf16(bf16(relu(x1)^2) * x3) (gpu/model.py:164-166, 195);
  *             otherwise h = x, [M, K].

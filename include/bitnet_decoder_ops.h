@@ -27,15 +27,29 @@ extern "C" {
  *   positions int64 [B], 0 <= positions[b] < S
  *   cos/sin  fp32 [S, head_dim / 2]
  *   out      bf16 [B, n_heads * head_dim]
+ *   workspace float [bitnet_attn_decode_workspace_floats(B, n_heads, n_kv_heads, n_splits)]
+ *   counters  int [B * n_kv_heads], zero before the first call (every call leaves them zero)
+ *   n_splits  1..8 workgroups share the S cache rows of one (sequence, kv head) in fixed slices;
+ *             with 1, workspace and counters may be NULL.  Calls that share a workspace
+ *             must not overlap in time.
  * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8, and
- * g * (S + 1024) * 4 bytes <= 96 KiB.  Returns 0, or 1 (shape),
- * 2 (null pointer), 3 (launch failed).  fp32 accumulation; results agree with
- * an fp32 evaluation of the same formula to about 1e-2 relative on bf16 outputs.
+ * g * (S / n_splits + 16 + 512) * 4 bytes <= 96 KiB.  Returns 0, or 1 (shape), 2 (null
+ * pointer), 3 (launch failed).  fp32 accumulation; results agree with an fp32 evaluation of
+ * the same formula to about 1e-2 relative on bf16 outputs.
  */
 int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v,
                        const int64_t* positions, const float* cos_table,
-                       const float* sin_table, uint16_t* out, int B, int S,
-                       int n_heads, int n_kv_heads, int head_dim, void* stream);
+                       const float* sin_table, uint16_t* out, float* workspace,
+                       int* counters, int n_splits, int B, int S, int n_heads,
+                       int n_kv_heads, int head_dim, void* stream);
+
+/* Tuning override for tests and measurements: threads per workgroup of the attention kernel
+ * (256 or 512; 0 restores the built-in choice).  Results do not depend on it beyond the
+ * order of fp32 additions.  Returns 0, or 1 for another value. */
+int bitnet_attn_decode_set_threads(int threads);
+
+/* Number of floats bitnet_attn_decode needs as workspace; -1 for bad arguments. */
+int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits);
 
 #ifdef __cplusplus
 }

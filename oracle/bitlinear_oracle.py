@@ -348,14 +348,14 @@ def fake_quant_input(x_bits: np.ndarray, mode: int = QUANT_COMPILED) -> np.ndarr
 def rmsnorm_bf16(h_bits: np.ndarray, g_bits: np.ndarray, eps: float) -> np.ndarray:
     """y = bf16(h * rsqrt(mean(h^2) + eps) * g), rows of bf16 bit patterns.
     The reference calls xformers' RMSNorm, which is not in its tree; the
-    rounding points are therefore a definition of this build: mean of squares
-    in float64 rounded to fp32, rsqrt as 1/sqrt in fp32, two fp32 multiplies,
+    rounding points are therefore a definition of this build: sum of squares
+    in float64 rounded to fp32 and divided by K in fp32, rsqrt as 1/sqrt in fp32, two fp32 multiplies,
     one rounding to bf16.  Pinned against torch's fp32 RMSNorm within 1 bf16
     ulp (it cannot be pinned tighter against a library that is absent)."""
     h = bf16_bits_to_f32(h_bits)
     g = bf16_bits_to_f32(g_bits)
     k = h.shape[-1]
-    mean = (np.sum(h.astype(np.float64) ** 2, axis=-1, keepdims=True) / np.float64(k)).astype(np.float32)
+    mean = (np.sum(h.astype(np.float64) ** 2, axis=-1, keepdims=True).astype(np.float32) / np.float32(k)).astype(np.float32)
     rstd = (np.float32(1.0) / np.sqrt((mean + np.float32(eps)).astype(np.float32))).astype(np.float32)
     return f32_to_bf16_bits(((h * rstd).astype(np.float32) * g).astype(np.float32))
 
