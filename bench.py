@@ -166,6 +166,103 @@ def cpu_baseline(shapes, M, budget_s=12.0):
     }
 
 
+INT8_MFMA_PEAK_TOPS = 5000.0
+
+
+def _acts(M, sh, dev, outliers=False):
+    import numpy as np
+    import torch
+
+    from bitnet_amd import workload
+
+    xb = workload.activations_bf16(M, sh.K, sh.shape_id, outliers=outliers)
+    return torch.from_numpy(xb.view(np.int16).copy()).view(torch.bfloat16).to(dev)
+
+
+def batched_and_prefill(lib, shapes, layers, scales, dev, decode_ms=(2, 4, 8, 16), prefill_ms=(128, 512, 2048)):
+    """The other token counts the workload names, on the same 30 layers of
+    weights: batched decode (every row its own absmax scale) through the whole
+    forward call, and prefill with 1 % of the activations scaled x20, as the
+    whole forward call (quantizer kernel + int8 MFMA GEMM) and as the GEMM alone."""
+    import torch
+
+    step_bytes = sum(sh.weight_bytes for sh in shapes) * len(layers)
+    n_calls = len(shapes) * len(layers)
+    out = {"batched_decode": {}, "prefill": {}}
+    for M in decode_ms:
+        acts = [_acts(M, sh, dev) for sh in shapes]
+        o_buf = [torch.empty(M, sh.N, dtype=torch.bfloat16, device=dev) for sh in shapes]
+        q_buf = [torch.empty(M, sh.K, dtype=torch.int8, device=dev) for sh in shapes]
+        s_buf = [torch.empty(M, dtype=torch.bfloat16, device=dev) for sh in shapes]
+
+        def launch(sp):
+            for row in layers:
+                for i, sh in enumerate(shapes):
+                    st = lib.bitlinear_forward_bf16(
+                        _p(acts[i]), _p(row[i]), _p(o_buf[i]), _p(scales[i]), _p(q_buf[i]), _p(s_buf[i]), M, sh.N, sh.K, 0, sp
+                    )
+                    assert st == 0, lib.bitlinear_status_string(st)
+
+        g = GraphRun(launch)
+        g.replay(5)
+        _, ms = g.timed(50)
+        us = ms * 1e3 / (50 * n_calls)
+        out["batched_decode"][f"M{M}"] = {
+            "us_per_call": round(us, 3),
+            "weight_GBps": round(step_bytes / n_calls / (us * 1e-6) / 1e9, 1),
+            "frac_of_hbm_peak": round(step_bytes / n_calls / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "bitlinear_tokens_per_s": round(M / (us * 1e-6 * n_calls), 1),
+        }
+        del g
+    for M in prefill_ms:
+        per = {}
+        tot_ops, tot_us, tot_fwd_us = 0.0, 0.0, 0.0
+        for i, sh in enumerate(shapes):
+            x = _acts(M, sh, dev, outliers=True)
+            q = torch.empty(M, sh.K, dtype=torch.int8, device=dev)
+            s = torch.empty(M, dtype=torch.bfloat16, device=dev)
+            o = torch.empty(M, sh.N, dtype=torch.bfloat16, device=dev)
+            rows = [row[i] for row in layers]
+
+            def fwd(sp):
+                for w in rows:
+                    st = lib.bitlinear_forward_bf16(_p(x), _p(w), _p(o), _p(scales[i]), _p(q), _p(s), M, sh.N, sh.K, 0, sp)
+                    assert st == 0, lib.bitlinear_status_string(st)
+
+            def gemm(sp):
+                for w in rows:
+                    lib.bitlinear_int8xint2(_p(q), _p(w), _p(o), _p(s), _p(scales[i]), M, sh.N, sh.K, sp)
+                    assert lib.bitlinear_last_status() == 0
+
+            res = []
+            for fn in (fwd, gemm):  # fwd first: it fills q and s for the GEMM alone
+                g = GraphRun(fn)
+                g.replay(2)
+                _, ms = g.timed(5)
+                res.append(ms * 1e3 / (5 * len(rows)))
+                del g
+            ops = 2.0 * M * sh.N * sh.K
+            per[sh.name] = {
+                "forward_us": round(res[0], 2),
+                "gemm_us": round(res[1], 2),
+                "gemm_TOPS": round(ops / (res[1] * 1e-6) / 1e12, 1),
+                "forward_TOPS": round(ops / (res[0] * 1e-6) / 1e12, 1),
+            }
+            tot_ops += ops
+            tot_us += res[1]
+            tot_fwd_us += res[0]
+        tops = tot_ops / (tot_us * 1e-6) / 1e12
+        out["prefill"][f"M{M}"] = {
+            "per_shape": per,
+            "layer_gemm_TOPS": round(tops, 1),
+            "layer_forward_TOPS": round(tot_ops / (tot_fwd_us * 1e-6) / 1e12, 1),
+            "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": round(tops / INT8_MFMA_PEAK_TOPS, 4), "kernel": "gemm_i2_prefill_kernel, the four 2B shapes of one layer"},
+            "prefill_tokens_per_s_bitlinear_only": round(M / (tot_fwd_us * 1e-6 * len(layers)), 1),
+        }
+    return out
+
+
 def end_to_end_decode(batches=(1, 8), prompt_len=512, gen_len=128):
     """Random-init BitNet-b1.58-2B-shaped decoder (30 layers, dim 2560, ffn 6912,
     20/5 heads, vocab 128256, tied bf16 embedding / LM head): a seeded 512-token
@@ -223,6 +320,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end 2B decode measurement")
+    ap.add_argument("--no-sweeps", action="store_true", help="skip the batched-decode (M=2..16) and prefill (M=128..2048) figures")
     ap.add_argument(
         "--pmc-probe",
         action="store_true",
@@ -378,6 +476,8 @@ def main():
         "per_shape_product_only": per_shape,
         "quantizer_us_per_launch": round(quant_us, 3),
     }
+    if not args.no_sweeps:
+        result.update(batched_and_prefill(lib, shapes, layers, scales, dev))
     if not args.no_e2e:
         del path, gemv, quant, layers
         torch.cuda.empty_cache()

@@ -33,7 +33,8 @@ SIGNATURES = {
     ),
     "bitlinear_norm_forward_bf16": (
         _c_int,
-        [_c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+        [_c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+         _c_int, _c_ptr],
     ),
     "bitnet_attn_decode": (
         _c_int,

@@ -220,7 +220,7 @@ template <int UPW>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, int M, int N, int K) {
+    ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K) {
     __shared__ int red[kMaxWaves * 256];
 
     const int lane = threadIdx.x & 63;
@@ -245,10 +245,11 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     const int e_lane = threadIdx.x & 63;
     const int e_m = m0 + (e_lane & 15);
     const int e_n = nb * 16 + 4 * (e_lane >> 4) + ((threadIdx.x >> 6) & 3);
-    uint16_t e_sb = 0, e_wsb = 0;
+    uint16_t e_sb = 0, e_wsb = 0, e_res = 0;
     if (out) {
         e_sb = s[e_m < M ? e_m : M - 1];
         e_wsb = ws[scale_slot(smap, e_n)];
+        if (residual) e_res = residual[(size_t)(e_m < M ? e_m : M - 1) * N + e_n];
     }
 
     v4i acc_q = {0, 0, 0, 0};
@@ -295,7 +296,11 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
 #pragma unroll
             for (int wv = 0; wv < kMaxWaves; ++wv) sum += part[wv];
             if (acc_out) acc_out[(size_t)e_m * N + e_n] = sum;
-            if (out) out[(size_t)e_m * N + e_n] = f32_to_bf16_rne((float)sum / bf16_to_f32(e_sb) * bf16_to_f32(e_wsb));
+            if (out) {
+                uint16_t o = f32_to_bf16_rne((float)sum / bf16_to_f32(e_sb) * bf16_to_f32(e_wsb));
+                if (residual) o = f32_to_bf16_rne(bf16_to_f32(e_res) + bf16_to_f32(o));
+                out[(size_t)e_m * N + e_n] = o;
+            }
         }
         return;
     }
@@ -310,7 +315,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
         if (acc_out) acc_out[(size_t)m * N + n] = sum;
         if (out) {
             const float v = (float)sum / bf16_to_f32(s[m]) * bf16_to_f32(ws[scale_slot(smap, n)]);
-            out[(size_t)m * N + n] = f32_to_bf16_rne(v);
+            uint16_t o = f32_to_bf16_rne(v);
+            if (residual) o = f32_to_bf16_rne(bf16_to_f32(residual[(size_t)m * N + n]) + bf16_to_f32(o));
+            out[(size_t)m * N + n] = o;
         }
     }
 }
@@ -682,6 +689,7 @@ struct FusedExtras {
     const uint16_t* residual;     // bf16 [M, N]; nullptr = none; out = bf16(residual + bf16(result))
     float eps;
     int glu;                      // 1: x is [M, 2K] = (x1 | x3); h = bf16(bf16(relu(x1)^2) * x3) feeds the norm
+    const uint16_t* act_scale;    // PRO 3 only: bf16 [M], the scales of the int8 rows handed in as x
 };
 
 __device__ __forceinline__ double dpp_sum_f64_row(double v) {
@@ -756,7 +764,77 @@ __device__ __forceinline__ uint4 glu8(const uint4& a, const uint4& b) {
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-template <int UPW, int VMAX, int PRO>  // PRO 0: plain, 1: RMSNorm in front, 2: squared-ReLU gate + RMSNorm in front
+// ---------------------------------------------------------------------------
+// Gate / RMSNorm / absmax quantizer as a kernel of its own: one workgroup per
+// token row.  Used in front of the product kernels when the activation block
+// is too large for every workgroup of the fused kernel to redo this work.
+// Same arithmetic, in the same order, as the PRO 1 / 2 prologue below.
+// ---------------------------------------------------------------------------
+constexpr int kPreThreads = 512;
+constexpr int kPreVecs = 8;  // 16-byte vectors per thread: rows up to 8 * 512 * 8 = 32768 elements
+
+template <int PRO>
+__global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t* __restrict__ x,
+                                                                 const uint16_t* __restrict__ norm_weight, float eps,
+                                                                 int8_t* __restrict__ q, uint16_t* __restrict__ s,
+                                                                 int K, int mode) {
+    __shared__ uint32_t wmax[kPreThreads / 64];
+    __shared__ double wsq[kPreThreads / 64];
+    const int row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int nvec = K >> 3;
+    const int xstride = PRO == 2 ? 2 * K : K;
+    const uint16_t* xr = x + (size_t)row * xstride;
+
+    uint4 xv[kPreVecs], gv[kPreVecs], x3v[PRO == 2 ? kPreVecs : 1];
+#pragma unroll
+    for (int r = 0; r < kPreVecs; ++r) {
+        const int idx = (tid + r * kPreThreads) < nvec ? (tid + r * kPreThreads) : (nvec - 1);
+        xv[r] = *(const uint4*)(xr + idx * 8);
+        if (PRO == 2) x3v[r] = *(const uint4*)(xr + K + idx * 8);
+        gv[r] = *(const uint4*)(norm_weight + idx * 8);
+    }
+    double sq = 0.0;
+#pragma unroll
+    for (int r = 0; r < kPreVecs; ++r) {
+        if (PRO == 2) xv[r] = glu8(xv[r], x3v[r]);
+        if (tid + r * kPreThreads < nvec) sq += sumsq8(xv[r]);
+    }
+    const double wsum = wave_sum_f64(sq);
+    if (lane == 0) wsq[wave] = wsum;
+    __syncthreads();
+    double total = 0.0;
+#pragma unroll
+    for (int i = 0; i < kPreThreads / 64; ++i) total += wsq[i];
+    const float mean = (float)total / (float)K;
+    const float rstd = 1.0f / __builtin_sqrtf(mean + eps);
+    uint32_t am = 0;
+#pragma unroll
+    for (int r = 0; r < kPreVecs; ++r) {
+        xv[r] = norm8(xv[r], gv[r], rstd);
+        if (tid + r * kPreThreads < nvec) am = absmax_bits8(xv[r], am);
+    }
+    am = wave_max_u32(am);
+    if (lane == 0) wmax[wave] = am;
+    __syncthreads();
+    am = wmax[0];
+#pragma unroll
+    for (int i = 1; i < kPreThreads / 64; ++i) am = max(am, wmax[i]);
+    const float s32 = mode == 0 ? quant_scale<0>(am) : quant_scale<1>(am);
+    if (tid == 0) s[row] = f32_to_bf16_rne(s32);
+    uint2* qr = (uint2*)(q + (size_t)row * K);
+#pragma unroll
+    for (int r = 0; r < kPreVecs; ++r) {
+        const int idx = tid + r * kPreThreads;
+        if (idx < nvec) qr[idx] = mode == 0 ? quant_vec8<0>(xv[r], s32) : quant_vec8<1>(xv[r], s32);
+    }
+}
+
+// PRO 0: plain, 1: RMSNorm in front, 2: squared-ReLU gate + RMSNorm in front,
+// 3: x already holds the int8 rows [M, K] (16 per vector) and ex.act_scale their scales: no quantizer
+template <int UPW, int VMAX, int PRO>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
@@ -790,19 +868,26 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     // Loads are unconditional (indices clamped into range, surplus results
     // ignored later): a load under a branch would force a full wait for all
     // earlier loads at the first use of x.
-    const int vec_per_row = K >> 3;
+    const int vec_per_row = PRO == 3 ? K >> 4 : K >> 3;
     const int nvec = M * vec_per_row;
     const int xstride = PRO == 2 ? 2 * K : K;  // elements between token rows of x
-    uint4 xv[VMAX], x3v[PRO == 2 ? VMAX : 1], gv[PRO != 0 ? VMAX : 1];
+    uint4 xv[VMAX], x3v[PRO == 2 ? VMAX : 1], gv[(PRO == 1 || PRO == 2) ? VMAX : 1];
 #pragma unroll
     for (int v = 0; v < VMAX; ++v) {
         const int idx = (tid + v * nthreads) < nvec ? (tid + v * nthreads) : (nvec - 1);
         const int row = idx / vec_per_row;
         const int col = idx - row * vec_per_row;
-        xv[v] = *(const uint4*)(x + (size_t)row * xstride + col * 8);
+        if (PRO == 3) {
+            xv[v] = *(const uint4*)((const int8_t*)x + (size_t)row * K + col * 16);
+        } else {
+            xv[v] = *(const uint4*)(x + (size_t)row * xstride + col * 8);
+        }
         if (PRO == 2) x3v[v] = *(const uint4*)(x + (size_t)row * xstride + K + col * 8);
-        if (PRO != 0) gv[v] = *(const uint4*)(ex.norm_weight + col * 8);
+        if (PRO == 1 || PRO == 2) gv[v] = *(const uint4*)(ex.norm_weight + col * 8);
     }
+    // PRO 3: the scale of token row tid, raw bits; any other variant re-reads a weight scale and ignores it
+    const uint16_t* asp = PRO == 3 ? ex.act_scale : ws;
+    const uint16_t e_as = asp[PRO == 3 ? (tid < M ? tid : M - 1) : 0];
     // weight words of the first round
     uint32_t w[UPW];
 #pragma unroll
@@ -832,7 +917,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     }
     lds_barrier();
 
-    if (PRO != 0) {
+    if (PRO == 1 || PRO == 2) {
         // gate (PRO 2), then sum of squares per token row, then y = bf16(h * rstd * g)
 #pragma unroll
         for (int v = 0; v < VMAX; ++v) {
@@ -862,27 +947,39 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
 
     // one LDS atomic per wave and token row where the wave's 64 vectors lie in
     // one row (always so when K/8 is a multiple of 64); per lane otherwise
+    if (PRO != 3) {
 #pragma unroll
-    for (int v = 0; v < VMAX; ++v) {
-        const int idx = tid + v * nthreads;
-        const int row = idx < nvec ? idx / vec_per_row : -1;
-        const uint32_t lm = idx < nvec ? absmax_bits8(xv[v], 0u) : 0u;
-        const int row0 = __builtin_amdgcn_readfirstlane(row);
-        if (__builtin_amdgcn_ballot_w64(row != row0) == 0) {
-            const uint32_t wm = wave_max_u32(lm);
-            if (lane == 0 && row0 >= 0) atomicMax(&amax_bits[row0], wm);
-        } else if (row >= 0) {
-            atomicMax(&amax_bits[row], lm);
+        for (int v = 0; v < VMAX; ++v) {
+            const int idx = tid + v * nthreads;
+            const int row = idx < nvec ? idx / vec_per_row : -1;
+            const uint32_t lm = idx < nvec ? absmax_bits8(xv[v], 0u) : 0u;
+            const int row0 = __builtin_amdgcn_readfirstlane(row);
+            if (__builtin_amdgcn_ballot_w64(row != row0) == 0) {
+                const uint32_t wm = wave_max_u32(lm);
+                if (lane == 0 && row0 >= 0) atomicMax(&amax_bits[row0], wm);
+            } else if (row >= 0) {
+                atomicMax(&amax_bits[row], lm);
+            }
         }
+        lds_barrier();
+    } else if (tid < M) {
+        sval[tid] = bf16_to_f32(e_as);
     }
-    lds_barrier();
 
 #pragma unroll
     for (int v = 0; v < VMAX; ++v) {
         const int idx = tid + v * nthreads;
         const int prow = idx < nvec ? idx / vec_per_row : -1;
-        int part = 0;  // sum of this thread's 8 quantized values
-        if (idx < nvec) {
+        int part = 0;  // sum of this thread's quantized values
+        if (PRO == 3) {
+            if (idx < nvec) {
+                const int col = idx - prow * vec_per_row;
+                *(uint4*)(lds_q + (size_t)prow * kp + col * 16) = xv[v];
+                const int ones = 0x01010101;
+                part = __builtin_amdgcn_sdot4((int)xv[v].x, ones, __builtin_amdgcn_sdot4((int)xv[v].y, ones, 0, false), false);
+                part = __builtin_amdgcn_sdot4((int)xv[v].z, ones, __builtin_amdgcn_sdot4((int)xv[v].w, ones, part, false), false);
+            }
+        } else if (idx < nvec) {
             const int row = prow;
             const int col = idx - row * vec_per_row;
             const float sf = mode == 0 ? quant_scale<0>(amax_bits[row]) : quant_scale<1>(amax_bits[row]);
@@ -972,6 +1069,7 @@ int g_tune_decode_waves = 0;
 int g_tune_path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse
 int g_tune_fused[3] = {1, 10, 4};
 int g_tune_prefill_big = 0;
+int g_tune_staged = 0;  // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 
 int set_status(int st) {
@@ -1006,14 +1104,15 @@ void pick_launch(int K, int* waves, int* upw) {
 }
 
 int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
-                  const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+                  const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream,
+                  const uint16_t* residual = nullptr) {
     int waves, upw;
     pick_launch(K, &waves, &upw);
     const dim3 grid(N / 16, (M + 15) / 16, 1);
     const dim3 block(waves * 64, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
 #define BITLINEAR_LAUNCH(U)                                                                                  \
-    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, M, N, K)
+    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K)
     switch (upw) {
         case 1: BITLINEAR_LAUNCH(1); break;
         case 2: BITLINEAR_LAUNCH(2); break;
@@ -1053,10 +1152,19 @@ struct FusedPlan {
     bool ok;
 };
 
-FusedPlan plan_fused(int M, int N, int K) {
+// The activation block a workgroup of the fused kernel may hold in LDS: what a
+// kernel gets without asking when it also quantizes the block; the
+// pre-quantized variant raises its limit (see raise_fused_lds).
+constexpr size_t kFusedLdsPlain = 60u * 1024u;
+constexpr size_t kFusedLdsRaised = 144u * 1024u;
+// Above this many activation elements the quantizer (and what precedes it)
+// runs once in a kernel of its own instead of in every workgroup.
+constexpr int kFuseMaxElems = 16384;
+
+FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
     FusedPlan pl = {1, 1, 4, 1, false};
     if (M > kFusedMaxTokens) return pl;
-    if ((size_t)M * (K + kFusedRowPad) > 60u * 1024u) return pl;
+    if ((size_t)M * (K + kFusedRowPad) > (pro == 3 ? kFusedLdsRaised : kFusedLdsPlain)) return pl;
     const int units = K / 64;
     if (g_tune_path == 3) {
         pl.rb = g_tune_fused[0];
@@ -1080,7 +1188,7 @@ FusedPlan plan_fused(int M, int N, int K) {
         pl.s = (units + pl.upw - 1) / pl.upw;
         if (pl.s > max_s) pl.s = max_s;
     }
-    const int nvec = M * (K / 8);
+    const int nvec = M * (K / (pro == 3 ? 16 : 8));
     int need = (nvec + 64 * pl.rb * pl.s - 1) / (64 * pl.rb * pl.s);
     if (need > 8 && g_tune_path != 3) {
         // a large activation block: as many waves as a workgroup may have, so that every
@@ -1101,6 +1209,19 @@ FusedPlan plan_fused(int M, int N, int K) {
     return pl;
 }
 
+// A kernel gets 64 KiB of dynamic LDS without asking; the pre-quantized variant
+// may hold up to 16 rows of 6912 and more, so its limit is raised once per
+// instance (a host-side attribute, no stream work).
+template <int U, int V>
+void raise_fused_lds() {
+    static bool done = false;
+    if (!done) {
+        (void)hipFuncSetAttribute((const void*)bitlinear_fused_kernel<U, V, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kFusedLdsRaised);
+        done = true;
+    }
+}
+
 int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const uint16_t* ws, const ScaleMap& smap,
                  int8_t* q_out, uint16_t* s_out, const FusedExtras& ex, int M, int N, int K, int mode,
                  const FusedPlan& pl, hipStream_t stream) {
@@ -1109,7 +1230,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
     const size_t lds = (size_t)M * (K + kFusedRowPad);
     const uint32_t* wq = (const uint32_t*)packed;
-    const int pro = ex.norm_weight ? (ex.glu ? 2 : 1) : 0;
+    const int pro = ex.act_scale ? 3 : (ex.norm_weight ? (ex.glu ? 2 : 1) : 0);
 #define BITLINEAR_LAUNCH_UVP(U, V, P)                                                                             \
     hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
                        s_out, ex, M, N, K, pl.rb, pl.s, mode)
@@ -1117,7 +1238,11 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     switch (pro) {                                   \
         case 0: BITLINEAR_LAUNCH_UVP(U, V, 0); break; \
         case 1: BITLINEAR_LAUNCH_UVP(U, V, 1); break; \
-        default: BITLINEAR_LAUNCH_UVP(U, V, 2); break; \
+        case 2: BITLINEAR_LAUNCH_UVP(U, V, 2); break; \
+        default:                                     \
+            if (lds > 48u * 1024u) raise_fused_lds<U, V>(); \
+            BITLINEAR_LAUNCH_UVP(U, V, 3);           \
+            break;                                   \
     }
 #define BITLINEAR_LAUNCH_U(U)                      \
     switch (pl.vmax) {                             \
@@ -1168,10 +1293,26 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
 }
 
 int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
-                const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+                const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream,
+                const uint16_t* residual = nullptr) {
     // vector loads: 16-byte groups of both operands must be 16-byte aligned
     if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
-    if (M > kPrefillMinTokens && g_tune_path != 2) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+    if (M > kPrefillMinTokens && g_tune_path != 2) {
+        if (residual) return BITLINEAR_ERR_SHAPE;  // the residual epilogue exists at decode sizes only
+        return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+    }
+    // The kernel that stages the int8 rows in LDS once per workgroup and shares
+    // them between several row blocks: fewer activation bytes through L2 than
+    // the kernels below, which read their B operands straight from global.
+    if (out && !acc_out && g_tune_staged != 2 && g_tune_path != 1 && g_tune_path != 2) {
+        const FusedPlan pl = plan_fused(M, N, K, 3);
+        // measured: staging pays once a workgroup shares the rows between two or more row blocks
+        const bool wanted = g_tune_staged == 1 || (M > kDecodeMaxTokens && (N / 16) >= 432);
+        if (pl.ok && wanted)
+            return launch_fused((const uint16_t*)act, packed, out, ws, smap, nullptr, nullptr,
+                                FusedExtras{nullptr, residual, 0.0f, 0, s}, M, N, K, 0, pl, stream);
+    }
+    if (residual) return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
     const bool decode_fits = M <= kDecodeMaxTokens && (size_t)M * K <= (size_t)kDecodeMaxLdsBytes;
     // The one-wave-per-row-block kernel pays off once there are enough row
     // blocks to fill every SIMD; below that, splitting K across waves wins.
@@ -1213,7 +1354,12 @@ int bitlinear_ws_num(int N, int K) {
 
 int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     if (kernel == 0) {
-        g_tune_path = g_tune_waves = g_tune_upw = g_tune_decode_waves = 0;
+        g_tune_path = g_tune_waves = g_tune_upw = g_tune_decode_waves = g_tune_staged = 0;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 6) {
+        if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
+        g_tune_staged = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 1) {
@@ -1315,10 +1461,14 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* ou
     if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)q_ws)) & 15u) return set_status(BITLINEAR_ERR_ARG);
     const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
     const FusedPlan pl = plan_fused(M, N, K);
-    if (pl.ok && g_tune_path != 4)
-        return set_status(launch_fused(x, packed, output0, ws, sm, q_ws, s_ws, FusedExtras{nullptr, nullptr, 0.0f, 0}, M, N, K,
-                                       mode, pl, (hipStream_t)stream));
-    // activation block too large to quantize inside every workgroup: two kernels
+    // one kernel while the activation block is small enough for every workgroup to quantize it
+    // again (or when the caller gave no workspaces for the two-kernel path)
+    const bool small = (long long)M * K <= kFuseMaxElems || g_tune_path == 3 || !q_ws || !s_ws;
+    if (pl.ok && small && g_tune_path != 4)
+        return set_status(launch_fused(x, packed, output0, ws, sm, q_ws, s_ws,
+                                       FusedExtras{nullptr, nullptr, 0.0f, 0, nullptr}, M, N, K, mode, pl,
+                                       (hipStream_t)stream));
+    // larger blocks: the quantizer once, in a kernel of its own, then the product
     if (!q_ws || !s_ws) return set_status(BITLINEAR_ERR_NULL);
     const int st = bitlinear_quant_absmax(x, q_ws, s_ws, M, K, mode, stream);
     if (st != BITLINEAR_OK) return st;
@@ -1327,16 +1477,30 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* ou
 
 int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu,
                                 const int8_t* packed, const uint16_t* ws, const uint16_t* residual, uint16_t* output0,
-                                int M, int N, int K, int mode, void* stream) {
+                                int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !norm_weight || !packed || !ws || !output0) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
-    if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)norm_weight)) & 15u) return set_status(BITLINEAR_ERR_ARG);
-    const FusedPlan pl = plan_fused(M, N, K);
-    if (!pl.ok) return set_status(BITLINEAR_ERR_SHAPE);  // decode-sized activation blocks only
-    const FusedExtras ex = {norm_weight, residual, eps, glu ? 1 : 0};
-    return set_status(launch_fused(x, packed, output0, ws, equal_slots(N, bitlinear_ws_num(N, K)), nullptr, nullptr, ex, M,
-                                   N, K, mode, pl, (hipStream_t)stream));
+    if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)norm_weight) | ((uintptr_t)q_ws)) & 15u)
+        return set_status(BITLINEAR_ERR_ARG);
+    const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    const FusedPlan pl = plan_fused(M, N, K, glu ? 2 : 1);
+    const bool small = (long long)M * K <= kFuseMaxElems || g_tune_path == 3 || !q_ws || !s_ws;
+    if (pl.ok && small && g_tune_path != 4) {
+        const FusedExtras ex = {norm_weight, residual, eps, glu ? 1 : 0, nullptr};
+        return set_status(launch_fused(x, packed, output0, ws, sm, nullptr, nullptr, ex, M, N, K, mode, pl,
+                                       (hipStream_t)stream));
+    }
+    // larger blocks: gate / norm / quantizer once per token row, then the product with the residual epilogue
+    if (!q_ws || !s_ws) return set_status(pl.ok ? BITLINEAR_ERR_NULL : BITLINEAR_ERR_SHAPE);
+    if (K > kPreThreads * kPreVecs * 8) return set_status(BITLINEAR_ERR_SHAPE);
+    const dim3 grid(M, 1, 1), block(kPreThreads, 1, 1);
+    if (glu)
+        hipLaunchKernelGGL(norm_quant_kernel<2>, grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode);
+    else
+        hipLaunchKernelGGL(norm_quant_kernel<1>, grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode);
+    if (hipGetLastError() != hipSuccess) return set_status(BITLINEAR_ERR_LAUNCH);
+    return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream, residual));
 }
 
 }  // extern "C"

@@ -101,13 +101,17 @@ def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads
 
 def norm_bitlinear(x, norm: "RMSNorm", lin: BitLinearKernel, glu: bool = False, residual=None):
     """[squared-ReLU gate ->] RMSNorm -> BitLinearKernel.forward [-> + residual]
-    as one kernel (bitlinear_norm_forward_bf16); x bf16 [M, K] (or [M, 2K] with
-    glu), decode-sized M."""
+    through bitlinear_norm_forward_bf16: one kernel for small activation blocks,
+    a norm/quantizer kernel plus the product kernel for larger ones; x bf16
+    [M, K] (or [M, 2K] with glu), M <= 16 when there is a residual."""
     M = x.shape[0]
+    K = lin.in_features
     out = torch.empty(M, lin.out_features, dtype=torch.bfloat16, device=x.device)
+    q_ws = torch.empty(M, K, dtype=torch.int8, device=x.device)
+    s_ws = torch.empty(M, dtype=torch.bfloat16, device=x.device)
     st = _lib.load_library().bitlinear_norm_forward_bf16(
         _ptr(x), _ptr(norm.weight), norm.eps, 1 if glu else 0, _ptr(lin.weight), _ptr(lin.weight_scale),
-        _ptr(residual) if residual is not None else None, _ptr(out), M, lin.out_features, lin.in_features,
+        _ptr(residual) if residual is not None else None, _ptr(out), _ptr(q_ws), _ptr(s_ws), M, lin.out_features, K,
         lin.quant_mode, _stream_ptr(),
     )
     _lib.check(st, f"bitlinear_norm_forward_bf16(M={M}, N={lin.out_features}, K={lin.in_features})")
@@ -189,12 +193,12 @@ class Transformer(nn.Module):
                 for _ in range(a.n_layers)]
 
     def fused_decode_ok(self, batch: int) -> bool:
-        """One new token per sequence can take the five-kernels-per-layer path
-        when the library's one-kernel forward accepts the activation blocks."""
+        """One new token per sequence can take the path with the norms, the gate
+        and the residual adds folded into the BitLinear calls (residual
+        epilogue: up to 16 rows)."""
         a = self.args
         hd = a.dim // a.n_heads
-        return (hd == 128 and self.norm.weight.dtype == torch.bfloat16
-                and batch * (a.ffn_dim + 64) <= 60 * 1024 and batch <= 16)
+        return hd == 128 and self.norm.weight.dtype == torch.bfloat16 and batch <= 16
 
     @torch.no_grad()
     def forward_decode_fused(self, tokens, positions, cache, cos, sin, workspace=None):

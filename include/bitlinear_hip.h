@@ -106,14 +106,15 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s,
 /*
  * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer (mode
  * as above), product and epilogue.  While the activation block is small
- * (M <= 16, M * (K + 64) <= 60 KiB and at most 8 vectors of 8 values per
- * thread of a 1024-thread workgroup) this is ONE kernel: every workgroup quantizes x itself, keeps the
- * int8 rows in LDS and never reads s from memory.  Larger blocks run the
- * quantizer kernel and then the product kernel.
- *   q_ws (int8 [M, K]) and s_ws (bf16 [M]) receive the quantized activations
- *   and scales; they may be NULL when the one-kernel path applies and are
- *   required otherwise.  Results equal bitlinear_quant_absmax followed by
- *   bitlinear_int8xint2 bit for bit.
+ * (M * K <= 16384 elements) this is ONE kernel: every workgroup quantizes x
+ * itself, keeps the int8 rows in LDS and never reads s from memory.  Larger
+ * blocks run the quantizer once, in a kernel of its own, and then the product
+ * kernel (M <= 16: int8 rows staged in LDS per workgroup; M > 16: MFMA GEMM).
+ *   q_ws (int8 [M, K], 16-byte aligned) and s_ws (bf16 [M]) receive the
+ *   quantized activations and scales.  They may be NULL when M <= 16 and
+ *   M * (K + 64) <= 60 KiB: the call then stays one kernel whatever M * K is
+ *   (slower for large blocks); otherwise they are required.  Results equal
+ *   bitlinear_quant_absmax followed by bitlinear_int8xint2 bit for bit.
  */
 int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
                            uint16_t* output0, const uint16_t* ws,
@@ -122,9 +123,11 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
 
 /*
  * bitlinear_forward_bf16 with the operations that surround a BitLinear in the
- * reference's decoder folded into the same kernel (decode-sized activation
- * blocks only: the one-kernel conditions of bitlinear_forward_bf16, else
- * BITLINEAR_ERR_SHAPE):
+ * reference's decoder folded in.  One kernel under the one-kernel conditions of
+ * bitlinear_forward_bf16; otherwise a gate / norm / quantizer kernel (one
+ * workgroup per token row, K <= 32768) followed by the product kernel, which
+ * needs q_ws / s_ws as above.  The residual epilogue exists for M <= 16 only
+ * (BITLINEAR_ERR_SHAPE beyond):
  *   in front  y = RMSNorm(h) = bf16(h * rsqrt(mean(h^2) + eps) * norm_weight)
  *             (attention_norm / ffn_norm / attn_sub_norm / ffn_sub_norm,
  *             gpu/model.py:159, 195, 228-229); the sum of squares is taken in fp64,
@@ -140,8 +143,8 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
 int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
                                 float eps, int glu, const int8_t* packed,
                                 const uint16_t* ws, const uint16_t* residual,
-                                uint16_t* output0, int M, int N, int K,
-                                int mode, void* stream);
+                                uint16_t* output0, int8_t* q_ws, uint16_t* s_ws,
+                                int M, int N, int K, int mode, void* stream);
 
 /*
  * Kernel / launch-shape override for tuning runs and tests.  Process-wide;
@@ -157,6 +160,9 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *   kernel 4: bitlinear_forward_bf16 always as two kernels
  *   kernel 5: prefill GEMM (M > 16) with output tile a per workgroup:
  *             0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256 (tokens x columns)
+ *   kernel 6: product of int8 rows (M <= 16) through the kernel that stages
+ *             them in LDS: a = 0 built-in choice (M > 4 and N >= 6912), 1 whenever it
+ *             fits, 2 never.  Independent of kernels 1..5; kernel 0 resets it.
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 

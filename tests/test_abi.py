@@ -62,7 +62,9 @@ def test_host_only_entry_points():
     assert lib.bitlinear_set_tuning(3, 2, 8, 5) == 0
     assert lib.bitlinear_set_tuning(3, 4, 5, 4) != 0
     assert lib.bitlinear_set_tuning(5, 1, 0, 0) == 0
-    assert lib.bitlinear_set_tuning(6, 0, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(6, 1, 0, 0) == 0
+    assert lib.bitlinear_set_tuning(6, 3, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(7, 0, 0, 0) != 0
     assert lib.bitlinear_set_tuning(0, 0, 0, 0) == 0
 
 

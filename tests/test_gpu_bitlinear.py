@@ -335,16 +335,22 @@ def test_prefill_full_size_linearity_property():
 
 
 @pytest.mark.parametrize("glu,res", [(0, 0), (0, 1), (1, 1), (1, 0)])
-@pytest.mark.parametrize("m", [1, 2, 4, 8])
+@pytest.mark.parametrize("m,path", [(1, 0), (2, 0), (4, 0), (8, 0), (8, 3), (16, 0), (3, 4), (16, 3)])
 @pytest.mark.parametrize("n,k", [(2560, 2560), (3840, 2560), (2560, 6912), (48, 192), (1040, 3200)])
-def test_fused_norm_gate_residual_forward(n, k, m, glu, res):
-    """[gate ->] RMSNorm -> quantizer -> product -> epilogue [-> residual] in one
-    kernel against the oracle chain, bit for bit."""
+def test_fused_norm_gate_residual_forward(n, k, m, path, glu, res):
+    """[gate ->] RMSNorm -> quantizer -> product -> epilogue [-> residual]
+    against the oracle chain, bit for bit: as one kernel (small blocks, or
+    path 3 = forced), and as norm/quantizer kernel + product kernel (large
+    blocks, or path 4 = forced)."""
     import ctypes
 
     lib = _lib.load_library()
-    if m * (k + 64) > 60 * 1024:
+    if path == 3 and m * (k + 64) > 60 * 1024:
         pytest.skip("activation block beyond the one-kernel limit")
+    if path == 3:
+        assert lib.bitlinear_set_tuning(3, 1, 8, 16 if k > 4096 else 5) == 0
+    elif path == 4:
+        assert lib.bitlinear_set_tuning(4, 0, 0, 0) == 0
     rng = np.random.default_rng(n + k + m + 7 * glu + res)
     w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
     xin = rng.standard_normal((m, 2 * k if glu else k)).astype(np.float32) * 1.7
@@ -357,10 +363,72 @@ def test_fused_norm_gate_residual_forward(n, k, m, glu, res):
     r = dev_bf16(rb) if res else None
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
-    st = lib.bitlinear_norm_forward_bf16(P(x), P(g), 1e-5, glu, P(pk), P(wsd), P(r), P(out), m, n, k, 0, None)
-    torch.cuda.synchronize()
+    q_ws = torch.empty(m, k, dtype=torch.int8, device="cuda")
+    s_ws = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+    try:
+        st = lib.bitlinear_norm_forward_bf16(P(x), P(g), 1e-5, glu, P(pk), P(wsd), P(r), P(out), P(q_ws), P(s_ws), m, n, k, 0, None)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
     assert st == 0
     _assert_bits_equal(host_bits(out), want, f"norm forward glu={glu} res={res}")
+
+
+def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
+    import ctypes
+
+    lib = _lib.load_library()
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    n, k = 2560, 2560
+    rng = np.random.default_rng(99)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    gb = o.f32_to_bf16_bits(np.ones(k, dtype=np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.02, 0, 0, 0], dtype=np.float32))
+    pk, g, wsd = _packed_dev(w), dev_bf16(gb), dev_bf16(ws_bits)
+    # M = 8 without workspaces: still one kernel, same bits
+    xb = o.f32_to_bf16_bits(rng.standard_normal((8, k)).astype(np.float32))
+    want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=None)
+    out = torch.full((8, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    st = lib.bitlinear_norm_forward_bf16(P(dev_bf16(xb)), P(g), 1e-5, 0, P(pk), P(wsd), None, P(out), None, None, 8, n, k, 0, None)
+    torch.cuda.synchronize()
+    assert st == 0
+    _assert_bits_equal(host_bits(out), want, "norm forward, no workspaces")
+    # M = 40: norm/quantizer kernel + MFMA GEMM; a residual is refused there
+    m = 40
+    xb = o.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=None)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    q_ws = torch.empty(m, k, dtype=torch.int8, device="cuda")
+    s_ws = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+    xd = dev_bf16(xb)
+    st = lib.bitlinear_norm_forward_bf16(P(xd), P(g), 1e-5, 0, P(pk), P(wsd), None, P(out), P(q_ws), P(s_ws), m, n, k, 0, None)
+    torch.cuda.synchronize()
+    assert st == 0
+    _assert_bits_equal(host_bits(out), want, "norm forward, M=40")
+    st = lib.bitlinear_norm_forward_bf16(P(xd), P(g), 1e-5, 0, P(pk), P(wsd), P(out), P(out), P(q_ws), P(s_ws), m, n, k, 0, None)
+    assert st == 1
+    st = lib.bitlinear_norm_forward_bf16(P(xd), P(g), 1e-5, 0, P(pk), P(wsd), None, P(out), None, None, m, n, k, 0, None)
+    assert st != 0
+
+
+@pytest.mark.parametrize("m", [1, 3, 5, 8, 13, 16])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (13824, 2560), (2560, 6912), (48, 192), (1040, 3200)])
+@pytest.mark.parametrize("staged", [1, 2])
+def test_product_through_the_lds_staged_kernel(n, k, m, staged):
+    """The drop-in entry with the int8 rows staged in LDS (tuning 6 = 1) and
+    without (= 2): same bits as the oracle either way."""
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=n + k + m)
+    s_bits = o.f32_to_bf16_bits(np.linspace(3.0, 90.0, m).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    _, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    try:
+        assert lib.bitlinear_set_tuning(6, staged, 0, 0) == 0
+        out = bitlinear.bitnet_int8xint2_linear(dev_i8(a), _packed_dev(w), dev_bf16(s_bits), dev_bf16(ws_bits))
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    _assert_bits_equal(host_bits(out), want, f"staged={staged} M={m}")
 
 
 def test_3d_input_and_out_argument():
