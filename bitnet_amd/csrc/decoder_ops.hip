@@ -119,7 +119,11 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         const int s = lo + wave + j * nwaves;
         vr[j] = *(const uint32_t*)(cv + (size_t)(s < S ? s : S - 1) * cache_row + 2 * lane);
     }
-    const int p = (int)positions[b];
+    // A position outside the cache would index the rope tables and the cache rows out of range;
+    // the host cannot see this device-side value, so it is clamped here (the result for such a
+    // sequence is then meaningless, but nothing outside the buffers is touched).
+    const int64_t p_raw = positions[b];
+    const int p = p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw);
     const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's positions are [lo, hi)
     const bool owns_new = p >= lo && p < lo + span;
 
@@ -263,28 +267,32 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
             const float is = 1.0f / red_l[hh];
             *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
         } else {
+            // device-coherent (write-through) stores: the record reaches the point where the other
+            // XCDs' loads see it without a writeback of this XCD's whole L2
             float* r = rec + ((size_t)sp * G + hh) * kRecFloats;
-            r[2 * lane] = o0;
-            r[2 * lane + 1] = o1;
+            __hip_atomic_store(r + 2 * lane, o0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(r + 2 * lane + 1, o1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (lane == 0) {
-                r[kHeadDim] = red_m[hh];  // -inf for a split with no positions
-                r[kHeadDim + 1] = red_l[hh];
+                __hip_atomic_store(r + kHeadDim, red_m[hh], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // -inf: no positions
+                __hip_atomic_store(r + kHeadDim + 1, red_l[hh], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
     if (nsplit == 1) return;
 
-    // the last split of this (sequence, kv head) to finish combines the records
-    __threadfence();  // make this workgroup's record visible device-wide before it is counted
+    // The last split of this (sequence, kv head) to finish combines the records.  The barrier
+    // waits until every thread's record stores have completed (they are write-through, so
+    // completed = visible device-wide); only then is the arrival counted, with a device-scope
+    // atomic, and the last arrival reads the records with device-coherent loads.  No L2-wide
+    // writeback or invalidate is involved.
     __syncthreads();
     if (tid == 0) {
-        const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = done == nsplit - 1;
         if (is_last) __hip_atomic_store(&counters[b * n_kv_heads + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!is_last) return;
-    __threadfence();
     for (int hh = wave; hh < G; hh += nwaves) {
         // all records' loads first (independent), then the merge
         float mk[kMaxSplits], lk[kMaxSplits], p0[kMaxSplits], p1[kMaxSplits];

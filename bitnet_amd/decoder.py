@@ -287,8 +287,9 @@ class Generator:
         self.model = model
         self.fused = fused and model.fused_decode_ok(batch)
         a_ = model.args
-        # enough splits of the cached positions that a few dozen CUs share every attention call
-        n_splits = max(1, min(8, 160 // max(1, batch * a_.n_kv_heads)))
+        # split the cached positions of every (sequence, kv head) over up to 8 workgroups: one CU alone
+        # pulls a small fraction of the memory bandwidth, and merging the splits costs about a microsecond
+        n_splits = max(1, min(8, 2048 // max(1, batch * a_.n_kv_heads)))
         self.attn_ws = AttnWorkspace(batch, a_.n_heads, a_.n_kv_heads, n_splits, model.tok_embeddings.weight.device)
         self.batch = batch
         self.max_seq = max_seq

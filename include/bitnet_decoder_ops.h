@@ -24,7 +24,8 @@ extern "C" {
  *     n_heads query heads, head h using kv head h / (n_heads / n_kv_heads).
  *   qkv      bf16 [B, (n_heads + 2 n_kv_heads) * head_dim]  (q | k | v)
  *   cache_k/v bf16 [B, S, n_kv_heads, head_dim]
- *   positions int64 [B], 0 <= positions[b] < S
+ *   positions int64 [B], 0 <= positions[b] < S (a value outside is clamped
+ *            into that range by the kernel: no access leaves the buffers)
  *   cos/sin  fp32 [S, head_dim / 2]
  *   out      bf16 [B, n_heads * head_dim]
  *   workspace float [bitnet_attn_decode_workspace_floats(B, n_heads, n_kv_heads, n_splits)]
