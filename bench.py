@@ -320,6 +320,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end 2B decode measurement")
+    ap.add_argument("--e2e-only", action="store_true", help="only the end-to-end 2B decode measurement (for profiler runs)")
     ap.add_argument("--no-sweeps", action="store_true", help="skip the batched-decode (M=2..16) and prefill (M=128..2048) figures")
     ap.add_argument(
         "--pmc-probe",
@@ -345,6 +346,9 @@ def main():
         sys.exit(1)
     lib = _lib.load_library()  # raises if libbitlinear_hip.so is missing
     dev = torch.device("cuda:0")
+    if args.e2e_only:
+        print(json.dumps({"end_to_end_decode": end_to_end_decode()}))
+        return
     M = args.m
     shapes, layers, scales, acts = build_workload(M, dev)
 

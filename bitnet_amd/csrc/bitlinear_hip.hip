@@ -771,9 +771,9 @@ __device__ __forceinline__ uint4 glu8(const uint4& a, const uint4& b) {
 // Same arithmetic, in the same order, as the PRO 1 / 2 prologue below.
 // ---------------------------------------------------------------------------
 constexpr int kPreThreads = 512;
-constexpr int kPreVecs = 8;  // 16-byte vectors per thread: rows up to 8 * 512 * 8 = 32768 elements
+constexpr int kPreVecs = 8;  // at most this many 16-byte vectors per thread: rows up to 8 * 512 * 8 = 32768 elements
 
-template <int PRO>
+template <int PRO, int VQ>  // VQ: vectors per thread, VQ * 512 * 8 >= K
 __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t* __restrict__ x,
                                                                  const uint16_t* __restrict__ norm_weight, float eps,
                                                                  int8_t* __restrict__ q, uint16_t* __restrict__ s,
@@ -788,9 +788,9 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
     const int xstride = PRO == 2 ? 2 * K : K;
     const uint16_t* xr = x + (size_t)row * xstride;
 
-    uint4 xv[kPreVecs], gv[kPreVecs], x3v[PRO == 2 ? kPreVecs : 1];
+    uint4 xv[VQ], gv[VQ], x3v[PRO == 2 ? VQ : 1];
 #pragma unroll
-    for (int r = 0; r < kPreVecs; ++r) {
+    for (int r = 0; r < VQ; ++r) {
         const int idx = (tid + r * kPreThreads) < nvec ? (tid + r * kPreThreads) : (nvec - 1);
         xv[r] = *(const uint4*)(xr + idx * 8);
         if (PRO == 2) x3v[r] = *(const uint4*)(xr + K + idx * 8);
@@ -798,7 +798,7 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
     }
     double sq = 0.0;
 #pragma unroll
-    for (int r = 0; r < kPreVecs; ++r) {
+    for (int r = 0; r < VQ; ++r) {
         if (PRO == 2) xv[r] = glu8(xv[r], x3v[r]);
         if (tid + r * kPreThreads < nvec) sq += sumsq8(xv[r]);
     }
@@ -812,7 +812,7 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
     const float rstd = 1.0f / __builtin_sqrtf(mean + eps);
     uint32_t am = 0;
 #pragma unroll
-    for (int r = 0; r < kPreVecs; ++r) {
+    for (int r = 0; r < VQ; ++r) {
         xv[r] = norm8(xv[r], gv[r], rstd);
         if (tid + r * kPreThreads < nvec) am = absmax_bits8(xv[r], am);
     }
@@ -826,7 +826,7 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
     if (tid == 0) s[row] = f32_to_bf16_rne(s32);
     uint2* qr = (uint2*)(q + (size_t)row * K);
 #pragma unroll
-    for (int r = 0; r < kPreVecs; ++r) {
+    for (int r = 0; r < VQ; ++r) {
         const int idx = tid + r * kPreThreads;
         if (idx < nvec) qr[idx] = mode == 0 ? quant_vec8<0>(xv[r], s32) : quant_vec8<1>(xv[r], s32);
     }
@@ -1495,10 +1495,25 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, 
     if (!q_ws || !s_ws) return set_status(pl.ok ? BITLINEAR_ERR_NULL : BITLINEAR_ERR_SHAPE);
     if (K > kPreThreads * kPreVecs * 8) return set_status(BITLINEAR_ERR_SHAPE);
     const dim3 grid(M, 1, 1), block(kPreThreads, 1, 1);
-    if (glu)
-        hipLaunchKernelGGL(norm_quant_kernel<2>, grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode);
-    else
-        hipLaunchKernelGGL(norm_quant_kernel<1>, grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode);
+    const int per_thread = (K / 8 + kPreThreads - 1) / kPreThreads;
+#define BITLINEAR_LAUNCH_PRE(P, V) \
+    hipLaunchKernelGGL((norm_quant_kernel<P, V>), grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode)
+#define BITLINEAR_LAUNCH_PRE_V(V)    \
+    if (glu)                         \
+        BITLINEAR_LAUNCH_PRE(2, V);  \
+    else                             \
+        BITLINEAR_LAUNCH_PRE(1, V)
+    if (per_thread <= 1) {
+        BITLINEAR_LAUNCH_PRE_V(1);
+    } else if (per_thread <= 2) {
+        BITLINEAR_LAUNCH_PRE_V(2);
+    } else if (per_thread <= 4) {
+        BITLINEAR_LAUNCH_PRE_V(4);
+    } else {
+        BITLINEAR_LAUNCH_PRE_V(8);
+    }
+#undef BITLINEAR_LAUNCH_PRE_V
+#undef BITLINEAR_LAUNCH_PRE
     if (hipGetLastError() != hipSuccess) return set_status(BITLINEAR_ERR_LAUNCH);
     return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream, residual));
 }
