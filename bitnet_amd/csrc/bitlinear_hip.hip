@@ -149,26 +149,27 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
     const int neg2w = (int)0xFEFEFEFEu;
     const v4i neg2 = {neg2w, neg2w, neg2w, neg2w};
 
-    for (int base = 0; base < steps; base += R) {
-        v4u w[R];
+    // Software pipeline over K: R 1-KB steps per round, the next round's loads
+    // issued before this round's MFMAs, so a wave always has R to 2R KB in flight.
+    v4u w0[R], w1[R];
+    auto load_round = [&](v4u(&w)[R], int base) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            int st = base + j;
+            // clamped into the row block: a step (or the part of the last step) past K is ignored when used
+            st = (st < steps && (st * 256 + chunk * 16) < K) ? st : 0;
+            w[j] = __builtin_nontemporal_load(wp + (size_t)st * 64);
+        }
+    };
+    auto use_round = [&](const v4u(&w)[R], int base) {
 #pragma unroll
         for (int j = 0; j < R; ++j) {
             const int st = base + j;
             const bool live = rows_ok && st < steps && (st * 256 + chunk * 16) < K;
-            w[j] = live ? __builtin_nontemporal_load(wp + (size_t)st * 64) : v4u{0u, 0u, 0u, 0u};
-        }
-        if (base == 0) {
-            // activations -> LDS while the weight loads are in flight
-            const int nvec = (M * K) >> 4;
-            for (int i = threadIdx.x; i < nvec; i += blockDim.x)
-                *(v4i*)(lds_act + (size_t)i * 16) = *(const v4i*)(act + (size_t)i * 16);
-            __syncthreads();
-        }
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
-            const int st = base + j;
-            const bool live = st < steps && (st * 256 + chunk * 16) < K;
-            const v4i b = live ? *(const v4i*)(bp + (size_t)st * 256) : v4i{0, 0, 0, 0};
+            const int stc = st < steps ? st : steps - 1;
+            const int kc = (stc * 256 + chunk * 16) < K ? stc * 256 : 0;
+            v4i b = *(const v4i*)(bp + (size_t)kc);
+            if (!live) b = v4i{0, 0, 0, 0};
             const uint32_t wd[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
             v4i a[4];
 #pragma unroll
@@ -183,6 +184,23 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
             acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[2], b, acc2, 0, 0, 0);
             acc3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[3], b, acc3, 0, 0, 0);
             accb = __builtin_amdgcn_mfma_i32_16x16x64_i8(neg2, b, accb, 0, 0, 0);
+        }
+    };
+    load_round(w0, 0);
+    if (steps > R) load_round(w1, R);
+    {
+        // activations -> LDS while the weight loads are in flight
+        const int nvec = (M * K) >> 4;
+        for (int i = threadIdx.x; i < nvec; i += blockDim.x)
+            *(v4i*)(lds_act + (size_t)i * 16) = *(const v4i*)(act + (size_t)i * 16);
+        lds_barrier();
+    }
+    for (int base = 0; base < steps; base += 2 * R) {
+        use_round(w0, base);
+        if (base + 2 * R < steps) load_round(w0, base + 2 * R);
+        if (base + R < steps) {
+            use_round(w1, base + R);
+            if (base + 3 * R < steps) load_round(w1, base + 3 * R);
         }
     }
 
@@ -1136,11 +1154,10 @@ int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     const v4u* wq = (const v4u*)packed;
 #define BITLINEAR_LAUNCH(R)                                                                                     \
     hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, out, acc_out, s, ws, smap, M, N, K)
-    if (steps <= 4) BITLINEAR_LAUNCH(4);
-    else if (steps <= 10) BITLINEAR_LAUNCH(10);
-    else if (steps <= 16) BITLINEAR_LAUNCH(16);
-    else if (steps <= 27) BITLINEAR_LAUNCH(27);
-    else BITLINEAR_LAUNCH(32);
+    // R steps (1 KB each per wave) per round, two rounds in flight
+    if (steps <= 4) BITLINEAR_LAUNCH(2);
+    else if (steps <= 10) BITLINEAR_LAUNCH(5);
+    else BITLINEAR_LAUNCH(8);
 #undef BITLINEAR_LAUNCH
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
@@ -1299,7 +1316,20 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
     if (M > kPrefillMinTokens && g_tune_path != 2) {
         if (residual) return BITLINEAR_ERR_SHAPE;  // the residual epilogue exists at decode sizes only
-        return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+        // A few dozen tokens on a narrow matrix leave most CUs without a GEMM tile, and a tile's
+        // chain of 256-k chunks is then pure latency (about 1 us each).  There the split-K kernel,
+        // run once per 16 tokens and re-reading the weights from L2 (about 1.65 TB/s measured),
+        // finishes earlier.  Both estimates in microseconds, fitted to measurements at the 2B shapes.
+        bool gemm = true;
+        if (M <= 256 && g_tune_path == 0) {
+            const double groups = (M + 15) / 16;
+            const double splitk_us = 3.0 + groups * ((double)N * K / 4.0) / 1.65e6;
+            const double tiles = ((N + 127) / 128) * (double)((M + 63) / 64);
+            const double gemm_us = 4.0 + (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
+            gemm = gemm_us <= splitk_us;
+        }
+        if (gemm) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+        return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
     }
     // The kernel that stages the int8 rows in LDS once per workgroup and shares
     // them between several row blocks: fewer activation bytes through L2 than
@@ -1369,6 +1399,11 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 2) {
+        if (a == 0 && b == 0) {  // split-K kernel always, launch shape left to the library
+            g_tune_path = 2;
+            g_tune_waves = g_tune_upw = 0;
+            return set_status(BITLINEAR_OK);
+        }
         if (a < 1 || a > kMaxWaves || !(b == 1 || b == 2 || b == 4 || b == 8 || b == 16))
             return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 2;

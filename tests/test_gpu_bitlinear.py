@@ -316,6 +316,21 @@ def test_prefill_scaled_output_with_outliers(shape_id, m):
     _assert_bits_equal(host_bits(out), want, f"{sh.name} prefill M={m}")
 
 
+@pytest.mark.parametrize("m", [17, 24, 48, 100, 130, 250])
+@pytest.mark.parametrize("n,k", [(2560, 2560), (2560, 6912), (13824, 2560)])
+def test_mid_size_token_counts_built_in_kernel_choice(n, k, m):
+    """Between decode and prefill sizes the library picks the split-K kernel
+    or the MFMA GEMM by an estimate of their times: same bits either way."""
+    w, a = _rand_case(n, k, m, seed=n + k + m)
+    got = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+    assert np.array_equal(got.cpu().numpy(), o.acc_int32(a, w))
+    s_bits = o.f32_to_bf16_bits(np.linspace(2.0, 120.0, m).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    _, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(a), _packed_dev(w), dev_bf16(s_bits), dev_bf16(ws_bits))
+    _assert_bits_equal(host_bits(out), want, f"M={m}")
+
+
 def test_prefill_full_size_linearity_property():
     """M = 2048 at the widest shape, checked without a CPU product: the result
     for activations a + b equals the sum of the results for a and for b."""
