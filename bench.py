@@ -321,6 +321,11 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end 2B decode measurement")
     ap.add_argument("--e2e-only", action="store_true", help="only the end-to-end 2B decode measurement (for profiler runs)")
+    ap.add_argument(
+        "--prefill-probe",
+        action="store_true",
+        help="counter run for `rocprofv3 --pmc`: the prefill GEMM (drop-in entry, M=2048) once per 2B shape, then exit",
+    )
     ap.add_argument("--no-sweeps", action="store_true", help="skip the batched-decode (M=2..16) and prefill (M=128..2048) figures")
     ap.add_argument(
         "--pmc-probe",
@@ -377,6 +382,18 @@ def main():
             for i, sh in enumerate(shapes):
                 lib.bitlinear_quant_absmax(_p(acts[i]), _p(q_buf[i]), _p(s_buf[i]), M, sh.K, 0, sp)
 
+    if args.prefill_probe:
+        Mp = 2048
+        for i, sh in enumerate(shapes):
+            q = torch.randint(-127, 128, (Mp, sh.K), dtype=torch.int8, device=dev)
+            sc = torch.full((Mp,), 2.0, dtype=torch.bfloat16, device=dev)
+            o = torch.empty(Mp, sh.N, dtype=torch.bfloat16, device=dev)
+            for rep in range(3):
+                lib.bitlinear_int8xint2(_p(q), _p(layers[rep][i]), _p(o), _p(sc), _p(scales[i]), Mp, sh.N, sh.K, None)
+                assert lib.bitlinear_last_status() == 0
+            torch.cuda.synchronize()
+        print(json.dumps({"prefill_probe": "bitlinear_int8xint2 at M=2048, three launches per 2B shape (wqkv, wo, w13, w2)"}))
+        return
     if args.pmc_probe:
         launch_quant_only(None)  # fills q_buf / s_buf
         src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)

@@ -21,6 +21,7 @@
 // epilogue (gpu/bitnet_kernels/bitnet_kernels.h:79-82) is applied.
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -41,12 +42,15 @@ struct ScaleMap {
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;  // NaN
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+// fp32 -> bf16, round to nearest even: gfx950 has the conversion in hardware
+// (two values per instruction)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) { return (uint16_t)(f32x2_to_bf16x2(f, 0.0f) & 0xffffu); }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
 // for every outstanding global load of the wave, which would serialise the
@@ -383,26 +387,34 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int ksteps = K >> 5;
     const int nchunks = (ksteps + kPfSteps - 1) / kPfSteps;
 
+    // All loads of the main loop are buffer loads: base (a resource descriptor in
+    // scalar registers) + a per-lane byte offset computed once + a scalar offset
+    // that advances with k, so the loop spends no vector instructions on
+    // addresses.  The activation descriptor covers this workgroup's rows only:
+    // rows past M lie beyond it and read as zeros.
     // staging map: piece p = tid + i * NTHR is 16 bytes of row p / kPfPieces at k-offset (p % kPfPieces) * 16
-    const int8_t* a_src[PPT];
+    const int rows_here = (M - m0) < TM ? (M - m0) : TM;
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(act + (size_t)m0 * K), 0, rows_here * K, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (N >> 2) * K, 0x00020000);
+    int a_off[PPT];
     int a_dst[PPT];
     int a_koff[PPT];
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
         const int pce = tid + i * NTHR;
         const int row = pce / kPfPieces;
-        const int mrow = (m0 + row) < M ? (m0 + row) : (M - 1);
         a_koff[i] = (pce % kPfPieces) * 16;
-        a_src[i] = act + (size_t)mrow * K;
+        a_off[i] = row * K + a_koff[i];
         a_dst[i] = row * kPfRowBytes + a_koff[i];
     }
-    // packed word of (column n, 32-k step, k-half kc); columns past N re-read column N-1
-    const uint32_t* w_src[NT];
+    // packed word of (column n, 32-k step, k-half kc), as a byte offset; columns past N re-read column N-1
+    int w_off[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         int n = n0 + nt * 32 + nl;
         n = n < N ? n : N - 1;
-        w_src[nt] = wq + (size_t)(n >> 4) * K + ((n & 15) >> 3) * 16 + kc * 8 + (n & 7);
+        w_off[nt] = ((n >> 4) * K + ((n & 15) >> 3) * 16 + kc * 8 + (n & 7)) * 4;
     }
     if (tid < TM) {
         const float sv = bf16_to_f32(out ? s[(m0 + tid) < M ? (m0 + tid) : (M - 1)] : (uint16_t)0x3f80);
@@ -421,50 +433,64 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < PPT; ++i) rs[i] = 0;
 
-    // Software pipeline, two chunks deep.  While chunk c is multiplied out of
-    // LDS, chunk c+1 moves from registers into the other LDS buffer
-    // (activations) or waits in registers (weight words), and chunk c+2 is in
-    // flight from memory: every load has a whole multiply phase to land.
-    v4i areg[PPT];
-    uint32_t wc[kPfSteps][NT], wn[kPfSteps][NT], wf[kPfSteps][NT];
+    // Software pipeline over the 256-k chunks.  Two register sets by chunk parity
+    // for the activation pieces (aE / aO) and for the weight words (wE / wO):
+    // set j & 1 holds chunk j.  While chunk c is multiplied out of LDS, the
+    // pieces of chunk c+1 move from their registers into the other LDS buffer
+    // and the same registers are at once re-requested for chunk c+3; a weight
+    // word is re-requested for chunk c+2 right after the MFMAs that consumed it.
+    // Every load so has two whole multiply phases to land and no register is
+    // ever copied (a copy would wait for the load it copies).
+    v4i aE[PPT], aO[PPT];
+    uint32_t wE[kPfSteps][NT], wO[kPfSteps][NT];
     const v4i zero4 = {0, 0, 0, 0};
     const int ones = 0x01010101;
-    auto load_chunk = [&](int c, uint32_t (&wdst)[kPfSteps][NT]) {
-#pragma unroll
-        for (int i = 0; i < PPT; ++i) {
-            const int k = c * kPfChunk + a_koff[i];
-            areg[i] = *(const v4i*)(a_src[i] + (k < K ? k : 0));  // past-the-end pieces are zeroed when staged
-        }
-#pragma unroll
-        for (int ks = 0; ks < kPfSteps; ++ks) {
-            const int st = c * kPfSteps + ks;
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) wdst[ks][nt] = w_src[nt][(size_t)(st < ksteps ? st : ksteps - 1) * 32];
-        }
+    const int last_step_off = (ksteps - 1) * 128;  // byte offset of the last 32-k step inside a row block
+    auto load_piece = [&](int c, int i) -> v4i {
+        // a chunk past the end re-reads chunk 0; it is never staged into a buffer that is multiplied
+        const int k0 = c * kPfChunk < K ? c * kPfChunk : 0;
+        return __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], k0, 0);
     };
-    auto stage_chunk = [&](int c) {
-#pragma unroll
-        for (int i = 0; i < PPT; ++i) {
-            const v4i v = (c * kPfChunk + a_koff[i]) < K ? areg[i] : zero4;
-            *(v4i*)(lds_a + (c & 1) * (TM * kPfRowBytes) + a_dst[i]) = v;
-            rs[i] += __builtin_amdgcn_sdot4(v.x, ones, 0, false) + __builtin_amdgcn_sdot4(v.y, ones, 0, false) +
-                     __builtin_amdgcn_sdot4(v.z, ones, 0, false) + __builtin_amdgcn_sdot4(v.w, ones, 0, false);
-        }
+    auto load_word = [&](int c, int ks, int nt) -> uint32_t {
+        const int so = (c * kPfSteps + ks) * 128;
+        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_off[nt], so < last_step_off ? so : last_step_off, 0);
+    };
+    auto stage_piece = [&](int c, int i, const v4i& piece, int8_t* buf) {
+        const v4i v = (c * kPfChunk + a_koff[i]) >= K ? zero4 : piece;  // ragged last chunk, or a chunk past the end
+        *(v4i*)(buf + a_dst[i]) = v;
+        rs[i] = __builtin_amdgcn_sdot4(v.x, ones, rs[i], false);
+        rs[i] = __builtin_amdgcn_sdot4(v.y, ones, rs[i], false);
+        rs[i] = __builtin_amdgcn_sdot4(v.z, ones, rs[i], false);
+        rs[i] = __builtin_amdgcn_sdot4(v.w, ones, rs[i], false);
     };
 
-    load_chunk(0, wc);
-    stage_chunk(0);
-    load_chunk(1, wn);  // clamped if there is no second chunk
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) aE[i] = load_piece(0, i);
+#pragma unroll
+    for (int ks = 0; ks < kPfSteps; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wE[ks][nt] = load_word(0, ks, nt);
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) aO[i] = load_piece(1, i);
+#pragma unroll
+    for (int ks = 0; ks < kPfSteps; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wO[ks][nt] = load_word(1, ks, nt);
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) stage_piece(0, i, aE[i], lds_a);
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) aE[i] = load_piece(2, i);
     lds_barrier();
 
     // Per k-step, besides its MFMAs: one slice of the staging of chunk c+1 (LDS
-    // write + row-sum), the reload of that slice's registers for chunk c+2, this
-    // step's weight words for chunk c+2, and the LDS reads of the next step's A
-    // operands.  Spread like this the memory work issues in the shadow of the
-    // MFMAs (the matrix pipe runs a 32x32x32 for 32 cycles after a 4-cycle issue)
-    // instead of stopping all four waves at once.  Nothing is conditional: k past
-    // the end is staged as zeros and multiplies to nothing, surplus loads are clamped.
-    for (int c = 0; c < nchunks; ++c) {
+    // write + row-sum), the reload of that slice's registers for chunk c+3, the
+    // reload of this step's weight words for chunk c+2, and the LDS reads of the
+    // next step's A operands.  Spread like this the memory work issues in the
+    // shadow of the MFMAs instead of stopping all four waves at once.  Nothing is
+    // conditional: pieces at k >= K (ragged last chunk, or a whole chunk past the
+    // end) are staged as zeros and multiply to nothing; the words of a k-step
+    // past the end re-read the last step and meet those zeros.
+    auto chunk_body = [&](int c, uint32_t(&wuse)[kPfSteps][NT], v4i(&astage)[PPT]) {
         const int8_t* abuf = lds_a + (c & 1) * (TM * kPfRowBytes) + nl * kPfRowBytes + kc * 16;
         int8_t* sbuf = lds_a + ((c + 1) & 1) * (TM * kPfRowBytes);
         v4i aop[2][MT];
@@ -474,17 +500,8 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
         for (int ks = 0; ks < kPfSteps; ++ks) {
 #pragma unroll
             for (int i = ks * PPT / kPfSteps; i < (ks + 1) * PPT / kPfSteps; ++i) {
-                const v4i v = ((c + 1) * kPfChunk + a_koff[i]) < K ? areg[i] : zero4;
-                *(v4i*)(sbuf + a_dst[i]) = v;
-                rs[i] += __builtin_amdgcn_sdot4(v.x, ones, 0, false) + __builtin_amdgcn_sdot4(v.y, ones, 0, false) +
-                         __builtin_amdgcn_sdot4(v.z, ones, 0, false) + __builtin_amdgcn_sdot4(v.w, ones, 0, false);
-                const int k = (c + 2) * kPfChunk + a_koff[i];
-                areg[i] = *(const v4i*)(a_src[i] + (k < K ? k : 0));
-            }
-            {
-                const int st = (c + 2) * kPfSteps + ks;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) wf[ks][nt] = w_src[nt][(size_t)(st < ksteps ? st : ksteps - 1) * 32];
+                stage_piece(c + 1, i, astage[i], sbuf);
+                astage[i] = load_piece(c + 3, i);
             }
             if (ks + 1 < kPfSteps) {
 #pragma unroll
@@ -494,12 +511,14 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
             v4i bop[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const uint32_t wd = wc[ks][nt];
+                const uint32_t wd = wuse[ks][nt];
                 bop[nt].x = (int)(wd & 0x03030303u);
                 bop[nt].y = (int)((wd >> 2) & 0x03030303u);
                 bop[nt].z = (int)((wd >> 4) & 0x03030303u);
                 bop[nt].w = (int)((wd >> 6) & 0x03030303u);
             }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) wuse[ks][nt] = load_word(c + 2, ks, nt);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -509,14 +528,11 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
             // back in front of their first use and exposes their latency
             __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int ks = 0; ks < kPfSteps; ++ks)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                wc[ks][nt] = wn[ks][nt];
-                wn[ks][nt] = wf[ks][nt];
-            }
         lds_barrier();
+    };
+    for (int c = 0; c < nchunks; c += 2) {
+        chunk_body(c, wE, aO);
+        if (c + 1 < nchunks) chunk_body(c + 1, wO, aE);
     }
 
     // row sums: the kPfPieces (= 16) threads of one DPP row staged the pieces of one activation row
@@ -541,15 +557,28 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     // Division by the token's scale: a correctly rounded reciprocal per token
     // (one IEEE divide) and, per element, q0 = a * rinv refined by
     // e = fma(-q0, s, a), q = fma(e, rinv, q0).
+    // Weight scales of the lane's 16 * NT columns.  Nearly always the wave's whole column range
+    // lies in one scale slot (a uniform test): one load; otherwise a slot per column.
     float wsf[NT][16];
     if (out) {
+        const int n_first = n0 < N ? n0 : N - 1;
+        const int n_last = (n0 + NT * 32 - 1) < N ? (n0 + NT * 32 - 1) : N - 1;
+        const int slot_first = scale_slot(smap, n_first);
+        if (slot_first == scale_slot(smap, n_last)) {
+            const float w1 = bf16_to_f32(ws[slot_first]);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int n = n0 + nt * 32 + (r >> 2) * 8 + kc * 4 + (r & 3);
-                wsf[nt][r] = bf16_to_f32(ws[scale_slot(smap, n < N ? n : N - 1)]);
-            }
+                for (int r = 0; r < 16; ++r) wsf[nt][r] = w1;
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int n = n0 + nt * 32 + (r >> 2) * 8 + kc * 4 + (r & 3);
+                    wsf[nt][r] = bf16_to_f32(ws[scale_slot(smap, n < N ? n : N - 1)]);
+                }
+        }
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -570,15 +599,15 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
                 for (int j = 0; j < 4; ++j) sum[j] = acc[mt][nt][g4 * 4 + j] - rs2;
                 if (acc_out) *(v4i*)(acc_out + o) = v4i{sum[0], sum[1], sum[2], sum[3]};
                 if (out) {
-                    uint32_t h[4];
+                    float h[4];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float a = (float)sum[j];
                         const float q0 = a * ri;
                         const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
-                        h[j] = f32_to_bf16_rne(q * wsf[nt][g4 * 4 + j]);
+                        h[j] = q * wsf[nt][g4 * 4 + j];
                     }
-                    *(uint2*)(out + o) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                    *(uint2*)(out + o) = make_uint2(f32x2_to_bf16x2(h[0], h[1]), f32x2_to_bf16x2(h[2], h[3]));
                 }
             }
         }
@@ -762,7 +791,7 @@ __device__ __forceinline__ uint4 norm8(const uint4& v, const uint4& g, float rst
     for (int i = 0; i < 4; ++i) {
         const float lo = __uint_as_float(d[i] << 16) * rstd * __uint_as_float(w[i] << 16);
         const float hi = __uint_as_float(d[i] & 0xffff0000u) * rstd * __uint_as_float(w[i] & 0xffff0000u);
-        o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+        o[i] = f32x2_to_bf16x2(lo, hi);
     }
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
@@ -775,9 +804,10 @@ __device__ __forceinline__ uint4 glu8(const uint4& a, const uint4& b) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const float r0 = fmaxf(__uint_as_float(d[i] << 16), 0.0f), r1 = fmaxf(__uint_as_float(d[i] & 0xffff0000u), 0.0f);
-        const float s0 = bf16_to_f32(f32_to_bf16_rne(r0 * r0)), s1 = bf16_to_f32(f32_to_bf16_rne(r1 * r1));
+        const uint32_t sq = f32x2_to_bf16x2(r0 * r0, r1 * r1);
+        const float s0 = __uint_as_float(sq << 16), s1 = __uint_as_float(sq & 0xffff0000u);
         const float lo = s0 * __uint_as_float(e[i] << 16), hi = s1 * __uint_as_float(e[i] & 0xffff0000u);
-        o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+        o[i] = f32x2_to_bf16x2(lo, hi);
     }
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
@@ -1284,6 +1314,8 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                    const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     const uint32_t* wq = (const uint32_t*)packed;
+    // the kernel addresses the packed weights through a buffer descriptor with 32-bit offsets
+    if ((long long)N * K / 4 >= (1ll << 31)) return BITLINEAR_ERR_SHAPE;
     const dim3 block(kPfWaves * 64, 1, 1);
     // the large tile double-buffers 2 x 128 rows x 272 bytes = 68 KiB of LDS: above the 64 KiB a
     // kernel gets without asking (a host-side attribute, set once per process)
