@@ -368,7 +368,7 @@ template <int MT, int NT>
 __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, int M, int N, int K) {
+    ScaleMap smap, int M, int N, int K, int band) {
     constexpr int TM = MT * 32;
     constexpr int NTHR = kPfWaves * 64;
     constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
@@ -380,8 +380,25 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int m0 = blockIdx.y * TM;
-    const int n0 = (blockIdx.x * kPfWaves + wave) * NT * 32;
+    // Workgroup -> tile.  Workgroups are handed to the 8 XCDs round-robin by
+    // linear id, and each XCD has its own L2.  The tile grid is cut into bands of
+    // `band` row tiles; a band belongs to one XCD (band b -> XCD b % 8), which
+    // walks it column tile by column tile.  The workgroups running on an XCD at
+    // any time therefore share a few row tiles (kept in that L2 for the whole
+    // band) and a few column tiles, instead of every tile pulling both of its
+    // operands through the memory-side cache on its own.
+    const int row_tiles = (M + TM - 1) / TM;
+    const int col_tiles = (N + kPfWaves * NT * 32 - 1) / (kPfWaves * NT * 32);
+    const int xcd = blockIdx.x & 7;
+    const int seq = blockIdx.x >> 3;
+    const int per_band = band * col_tiles;
+    const int bidx = xcd + 8 * (seq / per_band);
+    const int within = seq % per_band;
+    const int col_tile = within / band;
+    const int row_tile = bidx * band + within % band;
+    if (row_tile >= row_tiles) return;  // ragged last band (uniform over the workgroup)
+    const int m0 = row_tile * TM;
+    const int n0 = (col_tile * kPfWaves + wave) * NT * 32;
     const int nl = lane & 31;
     const int kc = lane >> 5;
     const int ksteps = K >> 5;
@@ -490,43 +507,62 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     // conditional: pieces at k >= K (ragged last chunk, or a whole chunk past the
     // end) are staged as zeros and multiply to nothing; the words of a k-step
     // past the end re-read the last step and meet those zeros.
+    // The matrix pipe runs one 32x32x32 for 32 cycles and a wave issues in
+    // order, so a run of MFMAs back to back blocks the wave's other instructions
+    // behind it.  Every k-step is therefore written as MT*NT slots of
+    // "one MFMA + a share of the preparation of the NEXT k-step" (expanding its
+    // weight words, reading its A operands from LDS, a slice of the staging,
+    // re-requesting the words just consumed), fenced so the order survives
+    // scheduling: the preparation issues in the shadow of the MFMA before it.
+    auto expand = [&](uint32_t wd) -> v4i {
+        v4i r;
+        r.x = (int)(wd & 0x03030303u);
+        r.y = (int)((wd >> 2) & 0x03030303u);
+        r.z = (int)((wd >> 4) & 0x03030303u);
+        r.w = (int)((wd >> 6) & 0x03030303u);
+        return r;
+    };
     auto chunk_body = [&](int c, uint32_t(&wuse)[kPfSteps][NT], v4i(&astage)[PPT]) {
         const int8_t* abuf = lds_a + (c & 1) * (TM * kPfRowBytes) + nl * kPfRowBytes + kc * 16;
         int8_t* sbuf = lds_a + ((c + 1) & 1) * (TM * kPfRowBytes);
-        v4i aop[2][MT];
+        constexpr int SLOTS = MT * NT;
+        v4i aop[2][MT], bop[2][NT];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) aop[0][mt] = *(const v4i*)(abuf + mt * 32 * kPfRowBytes);
 #pragma unroll
+        for (int nt = 0; nt < NT; ++nt) bop[0][nt] = expand(wuse[0][nt]);
+#pragma unroll
         for (int ks = 0; ks < kPfSteps; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
 #pragma unroll
-            for (int i = ks * PPT / kPfSteps; i < (ks + 1) * PPT / kPfSteps; ++i) {
-                stage_piece(c + 1, i, astage[i], sbuf);
-                astage[i] = load_piece(c + 3, i);
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                const int mt = slot / NT, nt = slot % NT;
+                acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bop[cur][nt], aop[cur][mt], acc[mt][nt], 0, 0, 0);
+                // preparation items, dealt round-robin over the slots
+                // (the LDS reads first: they have the longest way to go before their first use)
+                if (ks + 1 < kPfSteps) {
+#pragma unroll
+                    for (int j = 0; j < MT; ++j)
+                        if (j % SLOTS == slot)
+                            aop[nxt][j] = *(const v4i*)(abuf + j * 32 * kPfRowBytes + (ks + 1) * 32);
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        if ((MT + j) % SLOTS == slot) bop[nxt][j] = expand(wuse[ks + 1][j]);
+                }
+                if ((NT + MT) % SLOTS == slot) {
+#pragma unroll
+                    for (int i = ks * PPT / kPfSteps; i < (ks + 1) * PPT / kPfSteps; ++i) {
+                        stage_piece(c + 1, i, astage[i], sbuf);
+                        astage[i] = load_piece(c + 3, i);
+                    }
+                }
+                if (slot == SLOTS - 1) {
+                    // the words of this step were expanded during the previous one: re-request them
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) wuse[ks][j] = load_word(c + 2, ks, j);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            if (ks + 1 < kPfSteps) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    aop[(ks + 1) & 1][mt] = *(const v4i*)(abuf + mt * 32 * kPfRowBytes + (ks + 1) * 32);
-            }
-            v4i bop[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const uint32_t wd = wuse[ks][nt];
-                bop[nt].x = (int)(wd & 0x03030303u);
-                bop[nt].y = (int)((wd >> 2) & 0x03030303u);
-                bop[nt].z = (int)((wd >> 4) & 0x03030303u);
-                bop[nt].w = (int)((wd >> 6) & 0x03030303u);
-            }
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) wuse[ks][nt] = load_word(c + 2, ks, nt);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bop[nt], aop[ks & 1][mt], acc[mt][nt], 0, 0, 0);
-            // keep each step's group together: left alone, the scheduler pulls the LDS reads
-            // back in front of their first use and exposes their latency
-            __builtin_amdgcn_sched_barrier(0);
         }
         lds_barrier();
     };
@@ -1117,6 +1153,7 @@ int g_tune_decode_waves = 0;
 int g_tune_path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse
 int g_tune_fused[3] = {1, 10, 4};
 int g_tune_prefill_big = 0;
+int g_tune_prefill_band = 0;  // row tiles per band of the prefill GEMM's tile order, 0 = built-in choice
 int g_tune_staged = 0;  // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 
@@ -1326,17 +1363,28 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
         lds_limit_raised = true;
     }
     // tile (rows x columns of the output per workgroup): 0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256
-    int tile = (N >= 8192 && M >= 512) ? 2 : 0;  // measured: the wide tile pays once there are many column tiles
+    // measured: the wide tile pays once there are many tiles (about four per CU of the narrow kind)
+    const long long narrow_tiles = (long long)((N + 127) / 128) * ((M + 63) / 64);
+    int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : 0;
     if (g_tune_path == 5) tile = g_tune_prefill_big;
+    // 1-D grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
+    // tiles, fewer when there are not enough row tiles to give every XCD a band
+    const int tm = tile == 1 ? 128 : 64;
+    const int tn = tile == 0 ? 128 : (tile == 3 ? 512 : 256);
+    const int row_tiles = (M + tm - 1) / tm, col_tiles = (N + tn - 1) / tn;
+    int band = row_tiles / 8;
+    band = band < 1 ? 1 : (band > 8 ? 8 : band);
+    if (g_tune_path == 5 && g_tune_prefill_band > 0) band = g_tune_prefill_band;
+    const int nbands = (row_tiles + band - 1) / band;
+    const dim3 grid(8 * ((nbands + 7) / 8) * band * col_tiles, 1, 1);
     if (tile == 1) {
-        const dim3 grid((N + 255) / 256, (M + 127) / 128, 1);
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
+    } else if (tile == 3) {
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
     } else if (tile == 2) {
-        const dim3 grid((N + 255) / 256, (M + 63) / 64, 1);
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
     } else {
-        const dim3 grid((N + 127) / 128, (M + 63) / 64, 1);
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
     }
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
@@ -1457,8 +1505,10 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
+        if (a < 0 || a > 3 || b < 0 || b > 64) return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 5;
         g_tune_prefill_big = a;
+        g_tune_prefill_band = b;
         return set_status(BITLINEAR_OK);
     }
     return set_status(BITLINEAR_ERR_ARG);
