@@ -1,0 +1,75 @@
+"""I2_S <-> GPU-layout transcoder against the oracle's two layout statements,
+and (on the GPU) the product on a transcoded tensor against the CPU I2_S path."""
+import numpy as np
+import pytest
+import torch
+
+from bitnet_amd import i2s
+from oracle import bitlinear_oracle as o
+
+
+def _ternary(n, k, seed):
+    return np.random.default_rng(seed).integers(-1, 2, size=(n, k), dtype=np.int8)
+
+
+@pytest.mark.parametrize("n,k", [(16, 128), (48, 384), (2560, 2560)])
+def test_unpack_and_pack_match_the_oracle(n, k):
+    w = _ternary(n, k, n + k)
+    codes = o.i2s_pack_x86(w).reshape(-1)
+    got = i2s.i2s_unpack(torch.from_numpy(codes), n, k)
+    assert np.array_equal(got.numpy(), w)
+    assert np.array_equal(i2s.i2s_pack(torch.from_numpy(w)).numpy(), codes)
+
+
+def test_single_element_lands_where_the_reference_puts_it():
+    # element j of a 128-block -> byte j % 32, shift 6 - 2 * (j / 32)   (ggml-bitnet-mad.cpp:82-87)
+    for j in (0, 31, 32, 77, 127):
+        w = np.zeros((16, 128), dtype=np.int8)
+        w[3, j] = 1
+        codes = i2s.i2s_pack(torch.from_numpy(w)).numpy().reshape(16, 32)
+        base = np.full(32, 0x55, dtype=np.uint8)  # all codes 1 (= weight 0)
+        want = base.copy()
+        want[j % 32] = (0x55 & ~(3 << (6 - 2 * (j // 32)))) | (2 << (6 - 2 * (j // 32)))
+        assert np.array_equal(codes[3], want), j
+        assert np.array_equal(codes[2], base)
+
+
+def test_fusing_three_i2s_tensors_gives_the_gpu_layout_and_scale_slots():
+    k = 256
+    parts_np = [(_ternary(64, k, 1), 0.0213), (_ternary(32, k, 2), 0.0177), (_ternary(32, k, 3), 0.0251)]
+    parts = [(torch.from_numpy(o.i2s_pack_x86(w).reshape(-1)), s, w.shape[0]) for w, s in parts_np]
+    packed, scale = i2s.i2s_to_int2(parts, k)
+    want = o.pack_int2(np.concatenate([w for w, _ in parts_np], axis=0))
+    assert np.array_equal(packed.numpy(), want)
+    want_scale = o.f32_to_bf16_bits(np.array([s for _, s in parts_np] + [0.0], dtype=np.float32))
+    assert np.array_equal(scale.view(torch.int16).numpy().astype(np.uint16), want_scale)
+    back = i2s.int2_to_i2s(packed, scale, [64, 32, 32])
+    for (codes, s, _), (codes2, s2) in zip(parts, back):
+        assert torch.equal(codes, codes2)
+        assert abs(s2 - s) <= s * 2.0 ** -8  # bf16 rounding of the stored scale
+
+
+def test_stored_tensor_split_and_join():
+    w = _ternary(16, 128, 9)
+    codes = i2s.i2s_pack(torch.from_numpy(w))
+    raw = i2s.join_i2s_tensor(codes, 0.03125)
+    assert raw.numel() == 16 * 128 // 4 + 32  # code bytes + 32 (ggml-bitnet-mad.cpp:95-96)
+    c2, s2 = i2s.split_i2s_tensor(raw, 16, 128)
+    assert torch.equal(c2, codes) and s2 == 0.03125
+    with pytest.raises(ValueError):
+        i2s.i2s_unpack(codes[:-1], 16, 128)
+
+
+@pytest.mark.gpu
+def test_product_on_a_transcoded_tensor_equals_the_cpu_i2s_path():
+    from bitnet_amd import bitlinear
+
+    n, k, m = 2560, 2560, 3
+    w = _ternary(n, k, 21)
+    y = np.random.default_rng(22).integers(-128, 128, size=(m, k), dtype=np.int8)
+    codes = torch.from_numpy(o.i2s_pack_x86(w).reshape(-1)).cuda()
+    packed, _ = i2s.i2s_to_int2([(codes, 1.0, n)], k)
+    got = bitlinear.bitnet_int8xint2_acc(torch.from_numpy(y).cuda(), packed).cpu().numpy()
+    # the CPU stack: sum (w + 1) * y per row, minus sum(y)
+    cpu = o.i2s_vec_dot(o.i2s_pack_x86(w), y, n, k) - y.astype(np.int64).sum(axis=1, keepdims=True).astype(np.int32)
+    assert np.array_equal(got, cpu)
