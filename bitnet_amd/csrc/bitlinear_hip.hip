@@ -279,25 +279,43 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     const int neg2w = (int)0xFEFEFEFEu;
     const v4i neg2 = {neg2w, neg2w, neg2w, neg2w};
 
-    for (int base = wave * UPW; base < units; base += nwaves * UPW) {
-        uint32_t w[UPW];
-        v4i b[UPW];
+    // Rounds of UPW k-steps, two register sets: the loads of the round after next are issued
+    // before a round is multiplied, so 1 to 2 rounds stay in flight.  Loads are unconditional
+    // (indices clamped); a step past the end is multiplied by zeros.
+    uint32_t w0[UPW], w1[UPW];
+    v4i b0[UPW], b1[UPW];
+    auto load_round = [&](uint32_t(&w)[UPW], v4i(&b)[UPW], int base) {
 #pragma unroll
         for (int j = 0; j < UPW; ++j) {
-            const int u = base + j;
-            const bool live = u < units;
-            w[j] = live ? __builtin_nontemporal_load(wrow + (size_t)u * 64) : 0u;
-            b[j] = (live && tok_ok) ? *(const v4i*)(arow + (size_t)u * 64) : v4i{0, 0, 0, 0};
+            const int u = (base + j) < units ? (base + j) : (units - 1);
+            w[j] = __builtin_nontemporal_load(wrow + (size_t)u * 64);
+            b[j] = *(const v4i*)(arow + (size_t)u * 64);
         }
+    };
+    auto use_round = [&](const uint32_t(&w)[UPW], const v4i(&b)[UPW], int base) {
 #pragma unroll
         for (int j = 0; j < UPW; ++j) {
+            const bool live = (base + j) < units && tok_ok;
+            const v4i bj = live ? b[j] : v4i{0, 0, 0, 0};
             v4i a;
             a.x = (int)(w[j] & 0x03030303u);
             a.y = (int)((w[j] >> 2) & 0x03030303u);
             a.z = (int)((w[j] >> 4) & 0x03030303u);
             a.w = (int)((w[j] >> 6) & 0x03030303u);
-            acc_q = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[j], acc_q, 0, 0, 0);
-            acc_b = __builtin_amdgcn_mfma_i32_16x16x64_i8(neg2, b[j], acc_b, 0, 0, 0);
+            acc_q = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bj, acc_q, 0, 0, 0);
+            acc_b = __builtin_amdgcn_mfma_i32_16x16x64_i8(neg2, bj, acc_b, 0, 0, 0);
+        }
+    };
+    const int stride = nwaves * UPW;
+    const int base0 = wave * UPW;
+    load_round(w0, b0, base0);
+    if (base0 + stride < units) load_round(w1, b1, base0 + stride);
+    for (int base = base0; base < units; base += 2 * stride) {
+        use_round(w0, b0, base);
+        if (base + 2 * stride < units) load_round(w0, b0, base + 2 * stride);
+        if (base + stride < units) {
+            use_round(w1, b1, base + stride);
+            if (base + 3 * stride < units) load_round(w1, b1, base + 3 * stride);
         }
     }
 
@@ -1176,7 +1194,7 @@ bool shape_ok(int M, int N, int K) { return M >= 1 && N >= 16 && K >= 64 && (N %
 void pick_launch(int K, int* waves, int* upw) {
     const int units = K / 64;
     int u = 1;
-    while (u < 16 && (units + u - 1) / u > kMaxWaves) u *= 2;
+    while (u < 8 && (units + u - 1) / u > kMaxWaves) u *= 2;  // at most 8: two rounds of 8 fit the register file
     if (u < 4 && units >= 4 * 4) u = 4;  // keep a few loads in flight per wave
     int w = (units + u - 1) / u;
     if (w > kMaxWaves) w = kMaxWaves;
@@ -1202,8 +1220,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
         case 1: BITLINEAR_LAUNCH(1); break;
         case 2: BITLINEAR_LAUNCH(2); break;
         case 4: BITLINEAR_LAUNCH(4); break;
-        case 8: BITLINEAR_LAUNCH(8); break;
-        default: BITLINEAR_LAUNCH(16); break;
+        default: BITLINEAR_LAUNCH(8); break;
     }
 #undef BITLINEAR_LAUNCH
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
@@ -1484,7 +1501,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
             g_tune_waves = g_tune_upw = 0;
             return set_status(BITLINEAR_OK);
         }
-        if (a < 1 || a > kMaxWaves || !(b == 1 || b == 2 || b == 4 || b == 8 || b == 16))
+        if (a < 1 || a > kMaxWaves || !(b == 1 || b == 2 || b == 4 || b == 8))
             return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 2;
         g_tune_waves = a;

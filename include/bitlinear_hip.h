@@ -153,7 +153,7 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *   kernel 1: decode kernel where it applies (M <= 4, M*K <= 48 KiB) with
  *             a (1..4) 16-row blocks per workgroup
  *   kernel 2: split-K kernel always, a (1..16) waves per workgroup each
- *             keeping b (1, 2, 4, 8 or 16) 64-wide k-steps in flight
+ *             keeping one to two rounds of b (1, 2, 4 or 8) 64-wide k-steps in flight
  *             (a = b = 0: the library's own launch shape)
  *   kernel 3: fused forward kernel with a (1..4) 16-row blocks per workgroup,
  *             b waves splitting K for each (a*b <= 16), c (4, 5, 8, 10 or 16)

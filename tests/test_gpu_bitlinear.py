@@ -168,7 +168,7 @@ def test_result_independent_of_kernel_and_launch_shape():
             w, a = _rand_case(n, k, m, seed=9 + m)
             pk, ad = _packed_dev(w), dev_i8(a)
             want = o.acc_int32(a, w)
-            settings = [(2, wv, u) for wv, u in [(1, 1), (2, 16), (3, 4), (7, 8), (16, 2), (16, 16), (5, 1)]]
+            settings = [(2, wv, u) for wv, u in [(1, 1), (2, 8), (3, 4), (7, 8), (16, 2), (16, 8), (5, 1)]]
             settings += [(1, 1, 0), (1, 2, 0), (1, 3, 0), (1, 4, 0), (0, 0, 0)]
             for setting in settings:
                 assert lib.bitlinear_set_tuning(*setting, 0) == 0
