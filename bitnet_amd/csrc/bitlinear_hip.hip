@@ -386,7 +386,7 @@ template <int MT, int NT>
 __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, int M, int N, int K, int band) {
+    ScaleMap smap, int M, int N, int K, int band, int cseg) {
     constexpr int TM = MT * 32;
     constexpr int NTHR = kPfWaves * 64;
     constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
@@ -404,17 +404,21 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     // walks it column tile by column tile.  The workgroups running on an XCD at
     // any time therefore share a few row tiles (kept in that L2 for the whole
     // band) and a few column tiles, instead of every tile pulling both of its
-    // operands through the memory-side cache on its own.
+    // operands through the memory-side cache on its own.  With fewer than 8
+    // bands the column tiles are cut into segments too, so that all XCDs work.
     const int row_tiles = (M + TM - 1) / TM;
     const int col_tiles = (N + kPfWaves * NT * 32 - 1) / (kPfWaves * NT * 32);
     const int xcd = blockIdx.x & 7;
     const int seq = blockIdx.x >> 3;
-    const int per_band = band * col_tiles;
-    const int bidx = xcd + 8 * (seq / per_band);
-    const int within = seq % per_band;
-    const int col_tile = within / band;
-    const int row_tile = bidx * band + within % band;
-    if (row_tile >= row_tiles) return;  // ragged last band (uniform over the workgroup)
+    const int nbands = (row_tiles + band - 1) / band;
+    const int seg_cols = (col_tiles + cseg - 1) / cseg;  // few bands: the columns are cut into cseg segments as well
+    const int per_unit = band * seg_cols;
+    const int unit = xcd + 8 * (seq / per_unit);         // unit = (band, column segment) -> XCD unit % 8
+    if (unit >= nbands * cseg) return;
+    const int within = seq % per_unit;
+    const int col_tile = (unit % cseg) * seg_cols + within / band;
+    const int row_tile = (unit / cseg) * band + within % band;
+    if (row_tile >= row_tiles || col_tile >= col_tiles) return;  // ragged last band / segment (uniform over the workgroup)
     const int m0 = row_tile * TM;
     const int n0 = (col_tile * kPfWaves + wave) * NT * 32;
     const int nl = lane & 31;
@@ -1393,15 +1397,19 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     band = band < 1 ? 1 : (band > 8 ? 8 : band);
     if (g_tune_path == 5 && g_tune_prefill_band > 0) band = g_tune_prefill_band;
     const int nbands = (row_tiles + band - 1) / band;
-    const dim3 grid(8 * ((nbands + 7) / 8) * band * col_tiles, 1, 1);
+    int cseg = nbands >= 8 ? 1 : (8 + nbands - 1) / nbands;  // fewer than 8 bands: cut the columns too
+    cseg = cseg > col_tiles ? col_tiles : cseg;
+    const int seg_cols = (col_tiles + cseg - 1) / cseg;
+    const int units = nbands * cseg;
+    const dim3 grid(8 * ((units + 7) / 8) * band * seg_cols, 1, 1);
     if (tile == 1) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
     } else if (tile == 3) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
     } else if (tile == 2) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
     } else {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
     }
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
@@ -1414,15 +1422,15 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     if (M > kPrefillMinTokens && g_tune_path != 2) {
         if (residual) return BITLINEAR_ERR_SHAPE;  // the residual epilogue exists at decode sizes only
         // A few dozen tokens on a narrow matrix leave most CUs without a GEMM tile, and a tile's
-        // chain of 256-k chunks is then pure latency (about 1 us each).  There the split-K kernel,
-        // run once per 16 tokens and re-reading the weights from L2 (about 1.65 TB/s measured),
+        // chain of 256-k chunks is then pure latency (about 0.64 us each).  There the split-K kernel,
+        // run once per 16 tokens and re-reading the weights from L2 (about 1.45 TB/s measured),
         // finishes earlier.  Both estimates in microseconds, fitted to measurements at the 2B shapes.
         bool gemm = true;
         if (M <= 256 && g_tune_path == 0) {
             const double groups = (M + 15) / 16;
-            const double splitk_us = 3.0 + groups * ((double)N * K / 4.0) / 1.65e6;
+            const double splitk_us = 3.5 + groups * ((double)N * K / 4.0) / 1.45e6;
             const double tiles = ((N + 127) / 128) * (double)((M + 63) / 64);
-            const double gemm_us = 4.0 + (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
+            const double gemm_us = 4.0 + 0.64 * (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
             gemm = gemm_us <= splitk_us;
         }
         if (gemm) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
