@@ -43,6 +43,12 @@ SIGNATURES = {
     ),
     "bitnet_attn_decode_workspace_floats": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
     "bitnet_attn_decode_set_threads": (_c_int, [_c_int]),
+    "bitnet_lm_head_greedy": (
+        _c_int,
+        [_c_ptr, _c_ptr, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    ),
+    "bitnet_lm_head_workgroups": (_c_int, [_c_int]),
+    "bitnet_lm_head_set_kernel": (_c_int, [_c_int]),
     "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
 }
 

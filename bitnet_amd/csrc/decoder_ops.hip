@@ -25,6 +25,7 @@ namespace {
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 constexpr int kHeadDim = 128;
 constexpr int kMaxGroup = 8;
@@ -323,6 +324,340 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// Final RMSNorm + bf16 LM head + greedy token (gpu/model.py:279-280 followed by
+// the argmax of gpu/generate.py:264-288)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));
+}
+
+// y = bf16((h * rstd) * g), rstd = 1 / sqrt(mean(h^2) + eps): the sum of squares in fp64 (exact
+// for bf16 data, so independent of the order), rounded to fp32 and divided by K in fp32.
+// One workgroup per row.
+constexpr int kNormThreads = 256;
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const uint16_t* __restrict__ h,
+                                                                    const uint16_t* __restrict__ g, float eps,
+                                                                    uint16_t* __restrict__ y, int K) {
+    __shared__ double wsum[kNormThreads / 64];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int nvec = K >> 3;
+    const uint4* hr = (const uint4*)(h + (size_t)row * K);
+    double sq = 0.0;
+    for (int i = tid; i < nvec; i += kNormThreads) {
+        const uint4 v = hr[i];
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float lo = bf16f(d[j] & 0xffffu), hi = bf16f(d[j] >> 16);
+            sq += (double)(lo * lo) + (double)(hi * hi);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+    if ((tid & 63) == 0) wsum[tid >> 6] = sq;
+    __syncthreads();
+    double total = 0.0;
+#pragma unroll
+    for (int i = 0; i < kNormThreads / 64; ++i) total += wsum[i];
+    const float mean = (float)total / (float)K;
+    const float rstd = 1.0f / __builtin_sqrtf(mean + eps);
+    uint4* yr = (uint4*)(y + (size_t)row * K);
+    for (int i = tid; i < nvec; i += kNormThreads) {
+        const uint4 v = hr[i], w = ((const uint4*)g)[i];
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w}, e[4] = {w.x, w.y, w.z, w.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            o[j] = pack_bf16x2(bf16f(d[j] & 0xffffu) * rstd * bf16f(e[j] & 0xffffu), bf16f(d[j] >> 16) * rstd * bf16f(e[j] >> 16));
+        yr[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// logits[b, v] = bf16(sum_k y[b, k] * emb[v, k]) (fp32 accumulation), token[b] = the first v with
+// the largest logit.  A wave owns 16 vocabulary rows over all of K: the embedding streams through
+// registers as the row operand of bf16 MFMA 16x16x32 (a lane holds 16 consecutive k of one row
+// per 64-k step, two MFMAs), kLmDepth steps in flight; the normalised rows sit in LDS and are
+// the column operand (columns = tokens).  Each workgroup leaves its best (value, row) per token
+// in a workspace; lm_head_final_kernel reduces them.
+constexpr int kLmThreads = 256;
+constexpr int kLmDepth = 4;
+constexpr int kLmMaxTokens = 16;
+constexpr int kLmRowPad = 32;  // bytes between token rows in LDS beyond 2 * K
+
+__device__ __forceinline__ bool lm_better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+__global__ __launch_bounds__(kLmThreads) void lm_head_kernel(const uint16_t* __restrict__ y,
+                                                             const uint16_t* __restrict__ emb, float* __restrict__ logits,
+                                                             float* __restrict__ part_val, int* __restrict__ part_idx,
+                                                             int B, int V, int K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_y[];  // [B][2 * K + pad]
+    __shared__ float wv[kLmThreads / 64][kLmMaxTokens];
+    __shared__ int wi[kLmThreads / 64][kLmMaxTokens];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int steps = K >> 6;
+    const int row_stride = 2 * K + kLmRowPad;
+    const int rb = blockIdx.x * (kLmThreads / 64) + wave;
+    int row = rb * 16 + r16;
+    row = row < V ? row : V - 1;
+    const v4u* wrow = (const v4u*)(emb + (size_t)row * K + g * 16);
+
+    v4u w[kLmDepth][2];
+#pragma unroll
+    for (int j = 0; j < kLmDepth; ++j) {
+        const int st = j < steps ? j : steps - 1;
+        w[j][0] = __builtin_nontemporal_load(wrow + st * 8);
+        w[j][1] = __builtin_nontemporal_load(wrow + st * 8 + 1);
+    }
+    // the normalised rows -> LDS while the first embedding pieces are in flight
+    {
+        const int vec_per_row = K >> 3;
+        for (int i = tid; i < B * vec_per_row; i += kLmThreads) {
+            const int b = i / vec_per_row, c = i - b * vec_per_row;
+            *(uint4*)(lds_y + (size_t)b * row_stride + c * 16) = *(const uint4*)(y + (size_t)b * K + c * 8);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    const int tok = r16 < B ? r16 : B - 1;  // columns of tokens >= B are never read
+    const uint8_t* yb = lds_y + (size_t)tok * row_stride + g * 32;
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s0 = 0; s0 < steps; s0 += kLmDepth) {
+#pragma unroll
+        for (int j = 0; j < kLmDepth; ++j) {
+            const int st = s0 + j;
+            if (st < steps) {  // uniform
+                const uint4 b0 = *(const uint4*)(yb + st * 128), b1 = *(const uint4*)(yb + st * 128 + 16);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, w[j][0]), __builtin_bit_cast(v8bf, b0), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, w[j][1]), __builtin_bit_cast(v8bf, b1), acc, 0, 0, 0);
+            }
+            const int nx = (st + kLmDepth) < steps ? (st + kLmDepth) : (steps - 1);
+            w[j][0] = __builtin_nontemporal_load(wrow + nx * 8);
+            w[j][1] = __builtin_nontemporal_load(wrow + nx * 8 + 1);
+        }
+    }
+
+    // result lane (g, token r16): rows rb*16 + 4g + r in register r
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int vr = rb * 16 + 4 * g + r;
+        const float val = bf16f(pack_bf16x2(acc[r], 0.0f) & 0xffffu);
+        if (vr < V && r16 < B) {
+            if (logits) logits[(size_t)r16 * V + vr] = val;
+            if (lm_better(val, vr, bv, bi)) {
+                bv = val;
+                bi = vr;
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 16; off < 64; off <<= 1) {
+        const float ov = __shfl_xor(bv, off);
+        const int oi = __shfl_xor(bi, off);
+        if (lm_better(ov, oi, bv, bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (g == 0) {
+        wv[wave][r16] = bv;
+        wi[wave][r16] = bi;
+    }
+    __syncthreads();
+    if (tid < kLmMaxTokens) {
+        float v = wv[0][tid];
+        int i = wi[0][tid];
+#pragma unroll
+        for (int k = 1; k < kLmThreads / 64; ++k)
+            if (lm_better(wv[k][tid], wi[k][tid], v, i)) {
+                v = wv[k][tid];
+                i = wi[k][tid];
+            }
+        part_val[(size_t)blockIdx.x * kLmMaxTokens + tid] = v;
+        part_idx[(size_t)blockIdx.x * kLmMaxTokens + tid] = i;
+    }
+}
+
+
+// The same result for up to 8 tokens without the matrix pipe: a wave owns 8 consecutive
+// vocabulary rows (40 KB of the embedding at K = 2560, contiguous), every load instruction takes
+// 1 KB of ONE row (64 lanes x 8 consecutive k), and a lane multiplies its 8 values with the
+// matching 8 of each token (bf16 dot2 with fp32 accumulation).  Long contiguous requests are
+// what the memory system serves best; the per-lane partial sums of the 8 x TB (row, token)
+// pairs are combined at the end by a halving butterfly over the lanes.
+constexpr int kLsRows = 8;
+// a + w.lo * x.lo + w.hi * x.hi on packed bf16 pairs, products and sums in fp32
+__device__ __forceinline__ float bf16_dot2(uint32_t w, uint32_t x, float a) {
+    a = __builtin_fmaf(__uint_as_float(w << 16), __uint_as_float(x << 16), a);
+    return __builtin_fmaf(__uint_as_float(w & 0xffff0000u), __uint_as_float(x & 0xffff0000u), a);
+}
+
+template <int TB>  // tokens (columns) computed: 1, 2, 4 or 8 >= B
+__global__ __launch_bounds__(kLmThreads) void lm_head_stream_kernel(const uint16_t* __restrict__ y,
+                                                                    const uint16_t* __restrict__ emb,
+                                                                    float* __restrict__ logits,
+                                                                    float* __restrict__ part_val,
+                                                                    int* __restrict__ part_idx, int B, int V, int K) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_y[];  // [B][2 * K]
+    __shared__ float cv[kLmThreads / 64][kLmMaxTokens][kLsRows];
+    __shared__ int ci[kLmThreads / 64][kLmMaxTokens][kLsRows];
+    constexpr int NV = kLsRows * TB;  // (row, token) pairs per wave and row group
+    constexpr int kShift = NV == 64 ? 0 : (NV == 32 ? 1 : (NV == 16 ? 2 : 3));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int steps = K >> 9;  // 512 k per step
+    const int groups = (V + kLsRows - 1) / kLsRows;
+    const int nwaves = gridDim.x * (kLmThreads / 64);
+    int grp = blockIdx.x * (kLmThreads / 64) + wave;  // persistent: groups grp, grp + nwaves, ...
+
+    // first 1 KB of each of the first group's rows (a wave without a group re-reads the last row)
+    const v4u* wp[kLsRows];
+    v4u w[kLsRows];
+    auto group_rows = [&](int gidx) {
+#pragma unroll
+        for (int r = 0; r < kLsRows; ++r) {
+            int row = gidx * kLsRows + r;
+            row = row < V ? row : V - 1;
+            wp[r] = (const v4u*)(emb + (size_t)row * K) + lane;
+        }
+    };
+    group_rows(grp < groups ? grp : groups - 1);
+#pragma unroll
+    for (int r = 0; r < kLsRows; ++r) w[r] = __builtin_nontemporal_load(wp[r]);
+    {
+        const int nvec = (B * K) >> 3;
+        for (int i = tid; i < nvec; i += kLmThreads) *(uint4*)(lds_y + (size_t)i * 16) = *(const uint4*)(y + (size_t)i * 8);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    // the lane that ends up with pair (row pr of a group, token pt) keeps the best over its groups
+    const int pair = lane >> kShift;
+    const int pr = pair / TB, pt = pair % TB;
+    const bool owner = (lane & ((1 << kShift) - 1)) == 0 && pt < B;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+
+    for (; grp < groups; grp += nwaves) {
+        float acc[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) acc[i] = 0.0f;
+        for (int s = 0; s < steps; ++s) {
+            v4u xs[TB];
+#pragma unroll
+            for (int t = 0; t < TB; ++t) {
+                const int tok = t < B ? t : B - 1;
+                xs[t] = *(const v4u*)(lds_y + (size_t)tok * 2 * K + (size_t)s * 1024 + lane * 16);
+            }
+            // what to request next: this group's next 1 KB per row, or the first 1 KB of the wave's next group
+            int off = (s + 1) * 64;
+            if (s + 1 == steps) {  // uniform
+                const int nxt = grp + nwaves;
+                group_rows(nxt < groups ? nxt : grp);
+                off = 0;
+            }
+#pragma unroll
+            for (int r = 0; r < kLsRows; ++r) {
+                const v4u wr = w[r];
+                w[r] = __builtin_nontemporal_load(wp[r] + off);
+#pragma unroll
+                for (int t = 0; t < TB; ++t) {
+                    float a = acc[r * TB + t];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) a = bf16_dot2(wr[j], xs[t][j], a);
+                    acc[r * TB + t] = a;
+                }
+            }
+        }
+        // halving butterfly: after the stage with lane-xor mask m a lane keeps the half of its values
+        // chosen by its bit m; after log2(NV) stages lane l holds pair l >> log2(64 / NV), still as a
+        // partial over the lanes that differ in the low bits, which a plain xor reduction finishes
+        int m = 32;
+#pragma unroll
+        for (int n = NV; n > 1; n >>= 1) {
+            const bool up = (lane & m) != 0;
+#pragma unroll
+            for (int i = 0; i < n / 2; ++i) {
+                const float keep = up ? acc[i + n / 2] : acc[i];
+                const float send = up ? acc[i] : acc[i + n / 2];
+                acc[i] = keep + __shfl_xor(send, m);
+            }
+            m >>= 1;
+        }
+        float total = acc[0];
+        for (; m > 0; m >>= 1) total += __shfl_xor(total, m);
+        const int vr = grp * kLsRows + pr;
+        const float val = bf16f(pack_bf16x2(total, 0.0f) & 0xffffu);
+        if (owner && vr < V) {
+            if (logits) logits[(size_t)pt * V + vr] = val;
+            if (lm_better(val, vr, bv, bi)) {
+                bv = val;
+                bi = vr;
+            }
+        }
+    }
+    if (owner) {
+        cv[wave][pt][pr] = bv;
+        ci[wave][pt][pr] = bi;
+    }
+    __syncthreads();
+    if (tid < kLmMaxTokens) {
+        float v = -INFINITY;
+        int i = 0x7fffffff;
+        if (tid < B) {
+#pragma unroll
+            for (int k = 0; k < kLmThreads / 64; ++k)
+#pragma unroll
+                for (int r = 0; r < kLsRows; ++r)
+                    if (lm_better(cv[k][tid][r], ci[k][tid][r], v, i)) {
+                        v = cv[k][tid][r];
+                        i = ci[k][tid][r];
+                    }
+        }
+        part_val[(size_t)blockIdx.x * kLmMaxTokens + tid] = v;
+        part_idx[(size_t)blockIdx.x * kLmMaxTokens + tid] = i;
+    }
+}
+
+// Best (value, row) per token over the workgroups' partial results: one workgroup, 16 threads per
+// token.  A kernel of its own: the kernel boundary orders the partial results for free, where a
+// device-wide arrival counter would serialise thousands of atomics on one address.
+__global__ __launch_bounds__(kLmThreads) void lm_head_final_kernel(const float* __restrict__ part_val,
+                                                                   const int* __restrict__ part_idx,
+                                                                   int64_t* __restrict__ token_out, int nparts, int B) {
+    const int tid = threadIdx.x;
+    const int t = tid >> 4, sub = tid & 15;
+    float v = -INFINITY;
+    int i = 0x7fffffff;
+    for (int k = sub; k < nparts; k += 16) {
+        const float ov = part_val[(size_t)k * kLmMaxTokens + t];
+        const int oi = part_idx[(size_t)k * kLmMaxTokens + t];
+        if (lm_better(ov, oi, v, i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        const float ov = __shfl_xor(v, off);
+        const int oi = __shfl_xor(i, off);
+        if (lm_better(ov, oi, v, i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+    if (sub == 0 && t < B) token_out[t] = (int64_t)i;
+}
+
 }  // namespace
 
 static int g_attn_threads = 0;
@@ -375,5 +710,60 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
         default: BITNET_ATTN_LAUNCH(8) break;
     }
 #undef BITNET_ATTN_LAUNCH
+    return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+static int g_lm_kernel = 0;  // 0 = built-in choice, 1 = matrix-pipe kernel, 2 = streaming kernel where it applies
+
+/* tuning override for tests and measurements; results differ only in the order of fp32 additions */
+extern "C" int bitnet_lm_head_set_kernel(int which) {
+    if (which < 0 || which > 2) return 1;
+    g_lm_kernel = which;
+    return 0;
+}
+
+extern "C" int bitnet_lm_head_workgroups(int V) {
+    if (V < 1) return -1;
+    const int rows_per_wg = kLsRows * (kLmThreads / 64);  // the kernel with the fewest rows per workgroup
+    return (V + rows_per_wg - 1) / rows_per_wg;
+}
+
+extern "C" int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_weight, float eps, const uint16_t* emb,
+                                     uint16_t* y_ws, float* logits, int64_t* token_out, float* part_val,
+                                     int* part_idx, int B, int V, int K, void* stream) {
+    if (B < 1 || B > kLmMaxTokens || V < 1 || K < 64 || (K % 64) != 0) return 1;
+    if (!h || !norm_weight || !emb || !y_ws || !token_out || !part_val || !part_idx) return 2;
+    if ((((uintptr_t)h) | ((uintptr_t)norm_weight) | ((uintptr_t)emb) | ((uintptr_t)y_ws)) & 15u) return 1;
+    const size_t lds = (size_t)B * (2 * (size_t)K + kLmRowPad);
+    if (lds > 96u * 1024u) return 1;
+    static bool raised = false;  // more than 64 KiB of dynamic LDS has to be asked for, once per process
+    if (!raised) {
+        (void)hipFuncSetAttribute((const void*)lm_head_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        raised = true;
+    }
+    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(B), dim3(kNormThreads), 0, (hipStream_t)stream, h, norm_weight, eps, y_ws, K);
+    int nparts = 0;
+    const bool stream_ok = B <= 8 && (K % 512) == 0 && (size_t)B * 2 * K <= 60u * 1024u;
+    if (stream_ok && g_lm_kernel != 1) {
+        // persistent waves: at most 4 workgroups per CU of a 256-CU part, each wave walking row groups
+        const int full = (V + kLsRows * (kLmThreads / 64) - 1) / (kLsRows * (kLmThreads / 64));
+        const dim3 grid(full < 1024 ? full : 1024);
+        nparts = (int)grid.x;
+        const size_t lds_s = (size_t)B * 2 * K;
+#define BITNET_LM_STREAM(TB)                                                                                          \
+    hipLaunchKernelGGL(lm_head_stream_kernel<TB>, grid, dim3(kLmThreads), lds_s, (hipStream_t)stream, y_ws, emb, logits, \
+                       part_val, part_idx, B, V, K)
+        if (B == 1) BITNET_LM_STREAM(1);
+        else if (B == 2) BITNET_LM_STREAM(2);
+        else if (B <= 4) BITNET_LM_STREAM(4);
+        else BITNET_LM_STREAM(8);
+#undef BITNET_LM_STREAM
+    } else {
+        const int rows_per_wg = 16 * (kLmThreads / 64);
+        nparts = (V + rows_per_wg - 1) / rows_per_wg;
+        hipLaunchKernelGGL(lm_head_kernel, dim3(nparts), dim3(kLmThreads), lds, (hipStream_t)stream, y_ws, emb, logits, part_val,
+                           part_idx, B, V, K);
+    }
+    hipLaunchKernelGGL(lm_head_final_kernel, dim3(1), dim3(kLmThreads), 0, (hipStream_t)stream, part_val, part_idx, token_out, nparts, B);
     return hipGetLastError() == hipSuccess ? 0 : 3;
 }

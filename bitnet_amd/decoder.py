@@ -99,6 +99,35 @@ def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads
     return out
 
 
+class LmHeadWorkspace:
+    """Scratch of bitnet_lm_head_greedy for one (batch, vocabulary, dim)."""
+
+    def __init__(self, batch: int, vocab: int, dim: int, device):
+        lib = _lib.load_library()
+        n = lib.bitnet_lm_head_workgroups(vocab) * 16
+        self.y = torch.empty(batch, dim, dtype=torch.bfloat16, device=device)
+        self.part_val = torch.empty(n, dtype=torch.float32, device=device)
+        self.part_idx = torch.empty(n, dtype=torch.int32, device=device)
+
+
+def lm_head_greedy(h, norm: "RMSNorm", emb_weight, workspace: LmHeadWorkspace, token_out=None, logits_out=None):
+    """Final RMSNorm + tied bf16 LM head + greedy token in three launches
+    (bitnet_lm_head_greedy).  h bf16 [B, dim]; returns int64 [B] (token_out if
+    given); logits_out fp32 [B, vocab] receives the bf16-rounded logits if given."""
+    B, K = h.shape
+    V = emb_weight.shape[0]
+    if token_out is None:
+        token_out = torch.empty(B, dtype=torch.int64, device=h.device)
+    st = _lib.load_library().bitnet_lm_head_greedy(
+        _ptr(h), _ptr(norm.weight), norm.eps, _ptr(emb_weight), _ptr(workspace.y),
+        _ptr(logits_out) if logits_out is not None else None, _ptr(token_out), _ptr(workspace.part_val),
+        _ptr(workspace.part_idx), B, V, K, _stream_ptr(),
+    )
+    if st != 0:
+        raise _lib.BitLinearLibraryError(f"bitnet_lm_head_greedy: status {st}")
+    return token_out
+
+
 def norm_bitlinear(x, norm: "RMSNorm", lin: BitLinearKernel, glu: bool = False, residual=None):
     """[squared-ReLU gate ->] RMSNorm -> BitLinearKernel.forward [-> + residual]
     through bitlinear_norm_forward_bf16: one kernel for small activation blocks,
@@ -205,6 +234,13 @@ class Transformer(nn.Module):
         """One decode step, T = 1, five kernels per layer: norm+wqkv, rope+cache+
         attention, sub-norm+wo+residual, norm+w13, gate+sub-norm+w2+residual.
         tokens / positions [B, 1].  Returns logits [B, 1, vocab] fp32."""
+        h = self.decode_hidden_fused(tokens, positions, cache, cos, sin, workspace)
+        return self.output(self.norm(h)).float().view(tokens.shape[0], 1, -1)
+
+    @torch.no_grad()
+    def decode_hidden_fused(self, tokens, positions, cache, cos, sin, workspace=None):
+        """The decoder layers of forward_decode_fused: hidden state [B, dim] in
+        front of the final norm."""
         a = self.args
         B = tokens.shape[0]
         pos = positions.reshape(B)
@@ -216,7 +252,7 @@ class Transformer(nn.Module):
             h = norm_bitlinear(o, att.attn_sub_norm, att.wo, residual=h)
             x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
             h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)
-        return self.output(self.norm(h)).float().view(B, 1, -1)
+        return h
 
     @torch.no_grad()
     def forward_tokens(self, tokens, positions, cache, cos, sin):
@@ -283,7 +319,8 @@ class Generator:
     """Greedy generation: prefill of the whole prompt in one call, then one
     graph replay per generated token (gpu/generate.py:216-288)."""
 
-    def __init__(self, model: Transformer, batch: int, max_seq: int, use_graph: bool = True, fused: bool = True):
+    def __init__(self, model: Transformer, batch: int, max_seq: int, use_graph: bool = True, fused: bool = True,
+                 fused_head: bool = True):
         self.model = model
         self.fused = fused and model.fused_decode_ok(batch)
         a_ = model.args
@@ -302,13 +339,30 @@ class Generator:
         self.next_tok = torch.zeros(batch, dtype=torch.int64, device=dev)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.use_graph = use_graph
+        # final norm + bf16 LM head + greedy token as two launches of the library
+        self.lm_head = (self.fused and fused_head and model.output.weight.dtype == torch.bfloat16 and a.dim % 64 == 0
+                        and model.output.bias is None)
+        self.lm_ws = LmHeadWorkspace(batch, a.vocab_size, a.dim, dev) if self.lm_head else None
+        # generated tokens of a decode() call, written from inside the step so that a graph replay is the whole step
+        self.history = torch.zeros(max_seq, batch, dtype=torch.int64, device=dev)
+        self.step_idx = torch.zeros(1, dtype=torch.int64, device=dev)
 
     def _step(self):
-        if self.fused:
-            logits = self.model.forward_decode_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)
+        """One decode step including its bookkeeping: next token -> history and
+        the input of the following step, position + 1."""
+        if self.lm_head:
+            h = self.model.decode_hidden_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)
+            lm_head_greedy(h, self.model.norm, self.model.output.weight, self.lm_ws, token_out=self.next_tok)
         else:
-            logits = self.model.forward_tokens(self.tok, self.pos, self.cache, self.cos, self.sin)
-        self.next_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
+            if self.fused:
+                logits = self.model.forward_decode_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)
+            else:
+                logits = self.model.forward_tokens(self.tok, self.pos, self.cache, self.cos, self.sin)
+            self.next_tok.copy_(torch.argmax(logits[:, -1, :], dim=-1))
+        self.history.index_copy_(0, self.step_idx, self.next_tok.view(1, -1))
+        self.step_idx.add_(1)
+        self.tok.copy_(self.next_tok.view(-1, 1))
+        self.pos.add_(1)
 
     def _capture(self):
         s = torch.cuda.Stream()
@@ -333,7 +387,8 @@ class Generator:
     def decode(self, first: torch.Tensor, start_pos: int, steps: int) -> torch.Tensor:
         """Feeds `first` at position start_pos and generates `steps` further
         tokens greedily.  Returns [steps, B]."""
-        out = torch.empty(steps, self.batch, dtype=torch.int64, device=first.device)
+        if steps > self.history.shape[0]:
+            raise ValueError("more steps than the generator was sized for")
         self.tok.copy_(first.view(-1, 1))
         self.pos.fill_(start_pos)
         if self.use_graph and self.graph is None:
@@ -346,12 +401,10 @@ class Generator:
                 cv.copy_(sv)
             self.tok.copy_(first.view(-1, 1))
             self.pos.fill_(start_pos)
+        self.step_idx.zero_()
         for i in range(steps):
             if self.use_graph:
                 self.graph.replay()
             else:
                 self._step()
-            out[i] = self.next_tok
-            self.tok.copy_(self.next_tok.view(-1, 1))
-            self.pos.add_(1)
-        return out
+        return self.history[:steps].clone()

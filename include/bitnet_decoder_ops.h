@@ -52,6 +52,34 @@ int bitnet_attn_decode_set_threads(int threads);
 /* Number of floats bitnet_attn_decode needs as workspace; -1 for bad arguments. */
 int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits);
 
+/*
+ * The tail of a greedy decode step (Transformer.forward's `self.output(self.norm(h))`,
+ * gpu/model.py:279-280, and the argmax of the generation loop, gpu/generate.py:264-288):
+ *   y      = RMSNorm(h) with norm_weight (same rounding points as bitlinear_norm_forward_bf16)
+ *   logits = bf16(y . emb[v, :]) with fp32 accumulation, for the V rows of the (tied) embedding
+ *   token_out[b] = the lowest v with the largest logits[b, v]
+ *   h bf16 [B, K]; norm_weight bf16 [K]; emb bf16 [V, K] row-major; y_ws bf16 [B, K] scratch;
+ *   logits fp32 [B, V] or NULL (not written then); token_out int64 [B];
+ *   part_val float / part_idx int [bitnet_lm_head_workgroups(V) * 16] scratch.
+ * B <= 16, K % 64 == 0, B * (2 K + 32) <= 96 KiB; h, norm_weight, emb, y_ws 16-byte aligned.
+ * Three launches (norm; product with a best row per workgroup; reduction of those).
+ * Returns 0, 1 (shape / alignment), 2 (null), 3 (launch).
+ * Calls that share the scratch buffers must not overlap in time.
+ */
+int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_weight, float eps,
+                          const uint16_t* emb, uint16_t* y_ws, float* logits,
+                          int64_t* token_out, float* part_val, int* part_idx,
+                          int B, int V, int K, void* stream);
+
+/* Upper bound of the workgroups bitnet_lm_head_greedy launches for V rows (sizes its scratch);
+ * -1 for V < 1. */
+int bitnet_lm_head_workgroups(int V);
+
+/* Tuning override for tests and measurements: 0 = built-in choice (up to 8 tokens and K % 512 == 0:
+ * a streaming kernel with fp32 multiply-adds on the vector pipe; otherwise a bf16 MFMA kernel), 1 = MFMA kernel always,
+ * 2 = same as 0.  Results differ only in the order of fp32 additions.  Returns 0, or 1. */
+int bitnet_lm_head_set_kernel(int which);
+
 #ifdef __cplusplus
 }
 #endif

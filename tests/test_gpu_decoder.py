@@ -5,8 +5,10 @@ import numpy as np
 import pytest
 import torch
 
-from bitnet_amd import decoder, pack_weight
+from bitnet_amd import _lib, decoder, pack_weight
 from bitnet_amd.bitlinear import BitLinearKernel
+from tests.gpu_util import host_bits
+from oracle import bitlinear_oracle as o
 
 pytestmark = pytest.mark.gpu
 
@@ -199,3 +201,54 @@ def test_fused_decode_path_against_unfused():
     torch.cuda.synchronize()
     assert torch.allclose(logits[0], logits[1], rtol=5e-2, atol=5e-2)
     assert (outs[0] == outs[1]).float().mean() > 0.8
+
+
+@pytest.mark.parametrize("which", [0, 1])
+@pytest.mark.parametrize("B,V,K", [(1, 128256, 2560), (8, 128256, 2560), (3, 1000, 256), (16, 4111, 512), (2, 48, 64),
+                                   (2, 4111, 512), (4, 77, 1024), (5, 32000, 2048)])
+def test_lm_head_greedy_kernel(B, V, K, which):
+    """Final norm + bf16 LM head + greedy token: the normalised rows bit-exact
+    against the oracle's RMSNorm, the logits within one bf16 ulp (or 1e-3 of
+    the largest logit, where sums cancel) of an fp32 torch evaluation (fp32
+    sums in another order), the token equal to the first maximum of the
+    kernel's own logits."""
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(B * 7 + V)
+    h = (torch.randn(B, K, generator=g, device=dev) * 3).to(torch.bfloat16)
+    emb = (torch.randn(V, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    norm = decoder.RMSNorm(K, 1e-5).to(dev)
+    norm.weight.data = (1 + 0.1 * torch.randn(K, generator=g, device=dev)).to(torch.bfloat16)
+    ws = decoder.LmHeadWorkspace(B, V, K, dev)
+    logits = torch.full((B, V), float("nan"), dtype=torch.float32, device=dev)
+    lib = _lib.load_library()
+    assert lib.bitnet_lm_head_set_kernel(which) == 0  # 0: built-in choice (streaming kernel where it applies), 1: MFMA kernel
+    try:
+        tok = decoder.lm_head_greedy(h, norm, emb, ws, logits_out=logits)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitnet_lm_head_set_kernel(0)
+    want_y = o.rmsnorm_bf16(host_bits(h), host_bits(norm.weight.data), 1e-5)
+    assert np.array_equal(host_bits(ws.y), want_y)
+    ref = (ws.y.float() @ emb.float().T).to(torch.bfloat16)
+    got = logits.to(torch.bfloat16)
+    assert torch.equal(got.float(), logits)  # the kernel's logits are bf16 values
+    bad = (_ulp(got, ref) > 1) & ((got.float() - ref.float()).abs() > 1e-3 * float(ref.float().abs().max()))
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} logits outside tolerance"
+    assert torch.equal(tok, torch.argmax(logits, dim=-1))
+    # without the logits buffer, and a second call on the same scratch
+    tok2 = decoder.lm_head_greedy(h, norm, emb, ws)
+    assert torch.equal(tok2, tok)
+
+
+def test_generator_with_and_without_the_lm_head_kernel_agree():
+    args = decoder.ModelArgs(dim=256, n_layers=2, n_heads=2, n_kv_heads=1, vocab_size=512, ffn_dim=512)
+    model = _build(args, seed=3)
+    prompt = torch.randint(0, args.vocab_size, (2, 9), generator=torch.Generator().manual_seed(5)).cuda()
+    outs = []
+    for fused_head in (True, False):
+        gen = decoder.Generator(model, 2, 40, use_graph=True, fused_head=fused_head)
+        assert gen.lm_head == fused_head
+        first = gen.prefill(prompt)
+        outs.append(gen.decode(first, 9, 12).cpu())
+    # greedy tokens can only differ where two logits tie within fp32 summation order; with random weights they do not
+    assert torch.equal(outs[0], outs[1])
