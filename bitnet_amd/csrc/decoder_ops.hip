@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
 
 
 // ---------------------------------------------------------------------------
-// Final RMSNorm + bf16 LM head + greedy token (gpu/model.py:279-280 followed by
+// Final RMSNorm + bf16 LM head + greedy token (gpu/model.py:280-281 followed by
 // the argmax of gpu/generate.py:264-288)
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {

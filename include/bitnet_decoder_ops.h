@@ -54,7 +54,7 @@ int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int 
 
 /*
  * The tail of a greedy decode step (Transformer.forward's `self.output(self.norm(h))`,
- * gpu/model.py:279-280, and the argmax of the generation loop, gpu/generate.py:264-288):
+ * gpu/model.py:280-281, and the argmax of the generation loop, gpu/generate.py:264-288):
  *   y      = RMSNorm(h) with norm_weight (same rounding points as bitlinear_norm_forward_bf16)
  *   logits = bf16(y . emb[v, :]) with fp32 accumulation, for the V rows of the (tied) embedding
  *   token_out[b] = the lowest v with the largest logits[b, v]
