@@ -69,6 +69,8 @@ def bitnet_int8xint2_linear(input0, input1, s, ws, out=None):
         raise ValueError("weight_scale has fewer slots than this shape uses")
     if out is None:
         out = torch.empty(*out_shape, dtype=torch.bfloat16, device=input0.device)
+    if M == 0:
+        return out  # no token rows: nothing to launch
     lib.bitlinear_int8xint2(_ptr(input0), _ptr(input1), _ptr(out), _ptr(s), _ptr(ws), M, N, K, _stream_ptr())
     _lib.check(lib.bitlinear_last_status(), f"bitlinear_int8xint2(M={M}, N={N}, K={K})")
     return out
@@ -81,6 +83,8 @@ def bitnet_int8xint2_acc(input0, input1):
     N = input1.shape[0]
     K = input1.shape[1] * 4
     acc = torch.empty(*input0.shape[:-1], N, dtype=torch.int32, device=input0.device)
+    if M == 0:
+        return acc
     lib = _lib.load_library()
     st = lib.bitlinear_int8xint2_acc_i32(_ptr(input0), _ptr(input1), _ptr(acc), None, None, None, M, N, K, _stream_ptr())
     _lib.check(st, f"bitlinear_int8xint2_acc_i32(M={M}, N={N}, K={K})")
@@ -97,6 +101,8 @@ def bitnet_int8xint2_linear_seg(input0, input1, s, ws, seg_ends, out=None):
     K = input1.shape[1] * 4
     if out is None:
         out = torch.empty(*input0.shape[:-1], N, dtype=torch.bfloat16, device=input0.device)
+    if M == 0:
+        return out
     ends = (ctypes.c_int * len(seg_ends))(*[int(e) for e in seg_ends])
     lib = _lib.load_library()
     st = lib.bitlinear_int8xint2_seg(
@@ -116,6 +122,8 @@ def quant_input(input, mode: int = QUANT_COMPILED):
     K = input.shape[-1]
     q = torch.empty(input.shape, dtype=torch.int8, device=input.device)
     s = torch.empty(*input.shape[:-1], 1, dtype=torch.bfloat16, device=input.device)
+    if M == 0:
+        return q, s
     lib = _lib.load_library()
     st = lib.bitlinear_quant_absmax(_ptr(input), _ptr(q), _ptr(s), M, K, mode, _stream_ptr())
     _lib.check(st, f"bitlinear_quant_absmax(M={M}, K={K})")
@@ -152,6 +160,8 @@ class BitLinearKernel(nn.Module):
         q = torch.empty(input.shape, dtype=torch.int8, device=input.device)
         s = torch.empty(M, dtype=torch.bfloat16, device=input.device)
         out = torch.empty(*input.shape[:-1], N, dtype=torch.bfloat16, device=input.device)
+        if M == 0:
+            return out
         lib = _lib.load_library()
         st = lib.bitlinear_forward_bf16(
             _ptr(input), _ptr(self.weight), _ptr(out), _ptr(self.weight_scale), _ptr(q), _ptr(s), M, N, K,

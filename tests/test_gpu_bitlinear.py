@@ -459,6 +459,22 @@ def test_3d_input_and_out_argument():
     _assert_bits_equal(host_bits(out).reshape(6, n), want, "3d")
 
 
+def test_empty_batch_returns_empty_outputs():
+    """No token rows (a [0, K] activation): outputs of the right shape, no launch, no error."""
+    n, k = 2560, 2560
+    pk = _packed_dev(np.zeros((n, k), dtype=np.int8))
+    ws = torch.ones(4, dtype=torch.bfloat16, device="cuda")
+    a = torch.empty(0, k, dtype=torch.int8, device="cuda")
+    s = torch.empty(0, 1, dtype=torch.bfloat16, device="cuda")
+    assert bitlinear.bitnet_int8xint2_linear(a, pk, s, ws).shape == (0, n)
+    assert bitlinear.bitnet_int8xint2_acc(a, pk).shape == (0, n)
+    x = torch.empty(2, 0, k, dtype=torch.bfloat16, device="cuda")
+    q, sc = bitlinear.quant_input(x)
+    assert q.shape == (2, 0, k) and sc.shape == (2, 0, 1)
+    mod = bitlinear.BitLinearKernel(k, n).cuda()
+    assert mod(x).shape == (2, 0, n)
+
+
 def test_unsupported_shape_reports_status_and_launches_nothing():
     lib = _lib.load_library()
     a = torch.zeros(1, 2560, dtype=torch.int8, device="cuda")
