@@ -678,36 +678,48 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
 constexpr int kQuantThreads = 256;
 constexpr int kQuantRegVecs = 4;  // 16-byte vectors (8 bf16) kept in registers per thread
 
+// max |x| over 8 packed bf16 as a bit pattern (|x| as bf16 bits orders like the values): one
+// and + one packed 16-bit max per pair
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t absmax_bits8(const uint4& v, uint32_t cur) {
     const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    u16x2_t m = {(unsigned short)0, (unsigned short)0};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        cur = max(cur, d[i] & 0x7fffu);
-        cur = max(cur, (d[i] >> 16) & 0x7fffu);
-    }
-    return cur;
+    for (int i = 0; i < 4; ++i) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2_t, d[i] & 0x7fff7fffu));
+    const uint32_t both = __builtin_bit_cast(uint32_t, m);
+    return max(cur, max(both & 0xffffu, both >> 16));
+}
+
+// One value to its int8 code, left in the low byte of the result: the product
+// x * s in fp32 (mode 1: rounded to bf16), clamped to [-128, 127], then
+// + 1.5 * 2^23, which rounds to the nearest integer (ties to even, as rint does)
+// and leaves that integer's two's complement in the low mantissa bits.
+// Clamping before rounding equals rounding before clamping: the bounds are integers.
+template <int MODE>
+__device__ __forceinline__ uint32_t quant_low_byte(uint32_t x_f32_bits, float s32) {
+    float pr = __uint_as_float(x_f32_bits) * s32;
+    if (MODE == 1) pr = bf16_to_f32(f32_to_bf16_rne(pr));
+    pr = __builtin_amdgcn_fmed3f(pr, -128.0f, 127.0f);
+    return __float_as_uint(pr + 12582912.0f);
 }
 
 template <int MODE>
 __device__ __forceinline__ int quant_one(uint32_t bits16, float s32) {
-    const float x = __uint_as_float(bits16 << 16);
-    float pr = x * s32;
-    if (MODE == 1) pr = bf16_to_f32(f32_to_bf16_rne(pr));
-    const float r = fminf(fmaxf(rintf(pr), -128.0f), 127.0f);
-    return ((int)r) & 0xff;
+    return (int)(quant_low_byte<MODE>(bits16 << 16, s32) & 0xffu);
 }
 
 template <int MODE>
 __device__ __forceinline__ uint2 quant_vec8(const uint4& v, float s32) {
     const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-    uint32_t o[2] = {0u, 0u};
+    uint32_t p[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t lo = (uint32_t)quant_one<MODE>(d[i] & 0xffffu, s32);
-        const uint32_t hi = (uint32_t)quant_one<MODE>(d[i] >> 16, s32);
-        o[i >> 1] |= (lo | (hi << 8)) << ((i & 1) * 16);
+        const uint32_t lo = quant_low_byte<MODE>(d[i] << 16, s32);
+        const uint32_t hi = quant_low_byte<MODE>(d[i] & 0xffff0000u, s32);
+        p[i] = __builtin_amdgcn_perm(hi, lo, 0x0c0c0400u);  // bytes (lo.0, hi.0, 0, 0)
     }
-    return make_uint2(o[0], o[1]);
+    // (p0.0, p0.1, p1.0, p1.1)
+    return make_uint2(__builtin_amdgcn_perm(p[1], p[0], 0x05040100u), __builtin_amdgcn_perm(p[3], p[2], 0x05040100u));
 }
 
 // Activation scale from the row's |x| maximum (as bf16 bits).  torch evaluates
@@ -950,6 +962,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     __shared__ uint32_t amax_bits[kFusedMaxTokens];
     __shared__ int qsum[kFusedMaxTokens];
     __shared__ float sval[kFusedMaxTokens];  // activation scale per token (a bf16 value)
+    __shared__ float rinv[kFusedMaxTokens];  // its correctly rounded reciprocal
     __shared__ double sumsq[kFusedMaxTokens];
 
     const int tid = threadIdx.x;
@@ -1001,18 +1014,27 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         const int u = ks * UPW + j;
         w[j] = __builtin_nontemporal_load(wrow + (size_t)(u < units ? u : units - 1) * 64);
     }
-    // epilogue operands, raw bits, nothing depends on them until the end
-    uint16_t e_wsb[kFusedMaxRB], e_res[kFusedMaxRB];
+    // Epilogue operands, raw bits, nothing depends on them until the end.  Nearly always all
+    // rows of a workgroup share one weight-scale slot (found with scalar arithmetic): one load
+    // with a uniform address here; a workgroup that straddles a slot boundary fetches per row in
+    // the epilogue.  PRO 0 never has a residual.
+    constexpr bool kHasRes = PRO != 0;
+    const int n_first = blockIdx.x * RB * 16;
+    const int n_last = (n_first + RB * 16 - 1) < N ? (n_first + RB * 16 - 1) : N - 1;
+    const int slot_first = scale_slot(smap, n_first), slot_last = scale_slot(smap, n_last);
+    const uint16_t wsb_first = ws[slot_first];
+    uint16_t e_res[kFusedMaxRB];
+    if (kHasRes) {
 #pragma unroll
-    for (int r = 0; r < kFusedMaxRB; ++r) {
-        const int t = tid + r * nthreads;  // output slot t of the workgroup: [row block][reg][lane]
-        int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
-        n = n < N ? n : N - 1;
-        const int m = (t & 15) < M ? (t & 15) : M - 1;
-        e_wsb[r] = ws[scale_slot(smap, n)];  // unconditional: no branch, no early wait
-        // also unconditional: without a residual the load re-reads a weight scale and is ignored
-        const uint16_t* rp = ex.residual ? ex.residual : ws;
-        e_res[r] = rp[ex.residual ? (size_t)m * N + n : 0];
+        for (int r = 0; r < kFusedMaxRB; ++r) {
+            const int t = tid + r * nthreads;  // output slot t of the workgroup: [row block][reg][lane]
+            int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
+            n = n < N ? n : N - 1;
+            const int m = (t & 15) < M ? (t & 15) : M - 1;
+            // unconditional: without a residual the load re-reads a weight scale and is ignored
+            const uint16_t* rp = ex.residual ? ex.residual : ws;
+            e_res[r] = rp[ex.residual ? (size_t)m * N + n : 0];
+        }
     }
 
     for (int i = tid; i < RB * 256; i += nthreads) red[i] = 0;
@@ -1070,6 +1092,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         lds_barrier();
     } else if (tid < M) {
         sval[tid] = bf16_to_f32(e_as);
+        rinv[tid] = 1.0f / bf16_to_f32(e_as);
     }
 
 #pragma unroll
@@ -1093,7 +1116,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
             *(uint2*)(lds_q + (size_t)row * kp + col * 8) = qv;
             const int ones = 0x01010101;
             part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, 0, false), false);
-            if (col == 0) sval[row] = sf;
+            if (col == 0) {
+                sval[row] = sf;
+                rinv[row] = 1.0f / sf;
+            }
             if (blockIdx.x == 0) {
                 if (q_out) *(uint2*)(q_out + (size_t)idx * 8) = qv;
                 if (s_out && col == 0) s_out[row] = f32_to_bf16_rne(sf);
@@ -1149,6 +1175,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     }
     lds_barrier();
 
+    // Division by the token's scale as in the GEMM: q0 = a * (1/s) refined by
+    // e = fma(-q0, s, a), q = fma(e, 1/s, q0) -- the same bits as the IEEE divide
+    // for these integer-valued a, at a third of the instructions.
 #pragma unroll
     for (int r = 0; r < kFusedMaxRB; ++r) {
         const int t = tid + r * nthreads;
@@ -1157,9 +1186,14 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         const int m = l & 15;
         const int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
         if (m < M && n < N) {
-            const int sum = red[t] - 2 * qsum[m];
-            uint16_t o = f32_to_bf16_rne((float)sum / sval[m] * bf16_to_f32(e_wsb[r]));
-            if (ex.residual) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
+            uint16_t wsb = wsb_first;
+            if (slot_first != slot_last) wsb = ws[scale_slot(smap, n)];  // uniform branch, rare
+            const float a = (float)(red[t] - 2 * qsum[m]);
+            const float sv = sval[m], ri = rinv[m];
+            const float q0 = a * ri;
+            const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
+            uint16_t o = f32_to_bf16_rne(q * bf16_to_f32(wsb));
+            if (kHasRes && ex.residual) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
             out[(size_t)m * N + n] = o;
         }
     }
