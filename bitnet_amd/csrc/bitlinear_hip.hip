@@ -95,6 +95,13 @@ __device__ __forceinline__ int scale_slot(const ScaleMap& smap, int n) {
     return slot;
 }
 
+// The same for a wave-uniform n: a short scalar loop instead of the unrolled select chain.
+__device__ __forceinline__ int scale_slot_uniform(const ScaleMap& smap, int n) {
+    int slot = 0;
+    while (slot < smap.nseg - 1 && n >= smap.ends[slot]) ++slot;
+    return slot;
+}
+
 // ---------------------------------------------------------------------------
 // Decode kernel, M <= 4 tokens: one wave owns a 16-row block over all of K
 // ---------------------------------------------------------------------------
@@ -796,6 +803,7 @@ __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint1
 constexpr int kFusedMaxRB = 4;
 constexpr int kFusedMaxTokens = 16;
 constexpr int kFusedRowPad = 64;  // bytes between token rows in LDS beyond K
+constexpr int kFusedTailPad = 1024;  // bytes after the last row: unclamped reads of k-steps past the end land here
 
 // What the caller wants done to x before the quantizer, and to the result
 // after the epilogue.  All of it is what sits around a BitLinear in the
@@ -956,7 +964,7 @@ template <int UPW, int VMAX, int PRO>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
-    FusedExtras ex, int M, int N, int K, int RB, int S, int mode) {
+    FusedExtras ex, int M, int N, int K, int RB, int S, int mode, float inv_vec_per_row) {
     extern __shared__ __attribute__((aligned(16))) int8_t lds_q[];  // [M][K + pad]
     __shared__ int red[kFusedMaxRB * 256];
     __shared__ uint32_t amax_bits[kFusedMaxTokens];
@@ -965,11 +973,15 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     __shared__ float rinv[kFusedMaxTokens];  // its correctly rounded reciprocal
     __shared__ double sumsq[kFusedMaxTokens];
 
+    // A wave's own instruction stream is the critical path of this kernel (a wave issues roughly one
+    // instruction per 4 cycles, and a few hundred of them are most of its lifetime), so everything
+    // in front of the first load is kept short: wave-uniform values on the scalar unit, no integer
+    // division, no 64-bit address arithmetic.
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int rbl = wave / S;  // row block inside the workgroup
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rbl = (wave >= S ? 1 : 0) + (wave >= 2 * S ? 1 : 0) + (wave >= 3 * S ? 1 : 0);  // wave / S, RB <= 4
     const int ks = wave - rbl * S;
     const int rb = blockIdx.x * RB + rbl;
     const bool rows_ok = rb < (N >> 4);
@@ -979,29 +991,47 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     const int kp = K + kFusedRowPad;
 
     const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
-    const uint32_t* wrow = wq + (size_t)(rows_ok ? rb : 0) * K + lane_word;
+    // Weight words through a buffer descriptor that spans exactly this wave's block of 16 rows
+    // (K * 4 contiguous bytes; nothing for a row block past the end): a word of a k-step past
+    // the end of K is out of the descriptor's range and reads as zero, which is also the A
+    // operand that contributes nothing, so the loads need neither clamping nor masking.  The
+    // k-step goes into the instruction's immediate offset, the round into the vector offset.
+    // The weights are read once: the non-temporal hint keeps them from displacing the
+    // activations and scales that every workgroup re-reads.
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const char*)wq + (size_t)(rows_ok ? rb : 0) * K * 4), 0, rows_ok ? K * 4 : 0, 0x00020000);
+    int w_voff = lane_word * 4 + ks * (UPW * 256);
+#define FUSED_WLOAD(j) (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + (j) * 256, 0, 2 /* nt */)
 
     // Activation block first: 16-byte vectors of 8 bf16, VMAX per thread.  The
     // memory counter retires loads in issue order, so what is needed first
     // (x) is requested first and the weight words stay outstanding behind it.
     // Loads are unconditional (indices clamped into range, surplus results
     // ignored later): a load under a branch would force a full wait for all
-    // earlier loads at the first use of x.
+    // earlier loads at the first use of x.  Row and column of a vector come
+    // from a multiplication with 1 / vec_per_row (exact: (idx + 0.5) / vec_per_row
+    // is at least 0.5 / vec_per_row > 1e-4 away from an integer and below 16, far
+    // above the fp32 rounding error of the product).
     const int vec_per_row = PRO == 3 ? K >> 4 : K >> 3;
     const int nvec = M * vec_per_row;
     const int xstride = PRO == 2 ? 2 * K : K;  // elements between token rows of x
     uint4 xv[VMAX], x3v[PRO == 2 ? VMAX : 1], gv[(PRO == 1 || PRO == 2) ? VMAX : 1];
+    int vrc[VMAX];  // row << 16 | col of the vector of round v; -1: this thread has none
 #pragma unroll
     for (int v = 0; v < VMAX; ++v) {
-        const int idx = (tid + v * nthreads) < nvec ? (tid + v * nthreads) : (nvec - 1);
-        const int row = idx / vec_per_row;
+        const int raw = tid + v * nthreads;
+        const int idx = raw < nvec ? raw : (nvec - 1);
+        const int row = M == 1 ? 0 : (int)(((float)idx + 0.5f) * inv_vec_per_row);
         const int col = idx - row * vec_per_row;
+        vrc[v] = raw < nvec ? (row << 16 | col) : -1;
         if (PRO == 3) {
-            xv[v] = *(const uint4*)((const int8_t*)x + (size_t)row * K + col * 16);
+            xv[v] = *(const uint4*)((const int8_t*)x + idx * 16);          // rows are contiguous
+        } else if (PRO == 2) {
+            xv[v] = *(const uint4*)(x + row * xstride + col * 8);
+            x3v[v] = *(const uint4*)(x + row * xstride + K + col * 8);
         } else {
-            xv[v] = *(const uint4*)(x + (size_t)row * xstride + col * 8);
+            xv[v] = *(const uint4*)(x + idx * 8);                            // rows are contiguous
         }
-        if (PRO == 2) x3v[v] = *(const uint4*)(x + (size_t)row * xstride + K + col * 8);
         if (PRO == 1 || PRO == 2) gv[v] = *(const uint4*)(ex.norm_weight + col * 8);
     }
     // PRO 3: the scale of token row tid, raw bits; any other variant re-reads a weight scale and ignores it
@@ -1010,10 +1040,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     // weight words of the first round
     uint32_t w[UPW];
 #pragma unroll
-    for (int j = 0; j < UPW; ++j) {
-        const int u = ks * UPW + j;
-        w[j] = __builtin_nontemporal_load(wrow + (size_t)(u < units ? u : units - 1) * 64);
-    }
+    for (int j = 0; j < UPW; ++j) w[j] = FUSED_WLOAD(j);
     // Epilogue operands, raw bits, nothing depends on them until the end.  Nearly always all
     // rows of a workgroup share one weight-scale slot (found with scalar arithmetic): one load
     // with a uniform address here; a workgroup that straddles a slot boundary fetches per row in
@@ -1021,7 +1048,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     constexpr bool kHasRes = PRO != 0;
     const int n_first = blockIdx.x * RB * 16;
     const int n_last = (n_first + RB * 16 - 1) < N ? (n_first + RB * 16 - 1) : N - 1;
-    const int slot_first = scale_slot(smap, n_first), slot_last = scale_slot(smap, n_last);
+    const int slot_first = scale_slot_uniform(smap, n_first), slot_last = scale_slot_uniform(smap, n_last);
     const uint16_t wsb_first = ws[slot_first];
     uint16_t e_res[kFusedMaxRB];
     if (kHasRes) {
@@ -1049,10 +1076,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         // gate (PRO 2), then sum of squares per token row, then y = bf16(h * rstd * g)
 #pragma unroll
         for (int v = 0; v < VMAX; ++v) {
-            const int idx = tid + v * nthreads;
-            const int row = idx < nvec ? idx / vec_per_row : -1;
+            const int row = vrc[v] >> 16;
             if (PRO == 2) xv[v] = glu8(xv[v], x3v[v]);
-            const double sq = idx < nvec ? sumsq8(xv[v]) : 0.0;
+            const double sq = row >= 0 ? sumsq8(xv[v]) : 0.0;
             const int row0 = __builtin_amdgcn_readfirstlane(row);
             if (__builtin_amdgcn_ballot_w64(row != row0) == 0) {
                 const double wsum = wave_sum_f64(sq);
@@ -1064,9 +1090,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         lds_barrier();
 #pragma unroll
         for (int v = 0; v < VMAX; ++v) {
-            const int idx = tid + v * nthreads;
-            if (idx < nvec) {
-                const float mean = (float)sumsq[idx / vec_per_row] / (float)K;
+            if (vrc[v] >= 0) {
+                const float mean = (float)sumsq[vrc[v] >> 16] / (float)K;
                 const float rstd = 1.0f / __builtin_sqrtf(mean + ex.eps);
                 xv[v] = norm8(xv[v], gv[v], rstd);
             }
@@ -1078,9 +1103,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     if (PRO != 3) {
 #pragma unroll
         for (int v = 0; v < VMAX; ++v) {
-            const int idx = tid + v * nthreads;
-            const int row = idx < nvec ? idx / vec_per_row : -1;
-            const uint32_t lm = idx < nvec ? absmax_bits8(xv[v], 0u) : 0u;
+            const int row = vrc[v] >> 16;
+            const uint32_t lm = row >= 0 ? absmax_bits8(xv[v], 0u) : 0u;
             const int row0 = __builtin_amdgcn_readfirstlane(row);
             if (__builtin_amdgcn_ballot_w64(row != row0) == 0) {
                 const uint32_t wm = wave_max_u32(lm);
@@ -1098,22 +1122,21 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
 #pragma unroll
     for (int v = 0; v < VMAX; ++v) {
         const int idx = tid + v * nthreads;
-        const int prow = idx < nvec ? idx / vec_per_row : -1;
+        const int prow = vrc[v] >> 16, pcol = vrc[v] & 0xffff;
         int part = 0;  // sum of this thread's quantized values
         if (PRO == 3) {
-            if (idx < nvec) {
-                const int col = idx - prow * vec_per_row;
-                *(uint4*)(lds_q + (size_t)prow * kp + col * 16) = xv[v];
+            if (prow >= 0) {
+                *(uint4*)(lds_q + prow * kp + pcol * 16) = xv[v];
                 const int ones = 0x01010101;
                 part = __builtin_amdgcn_sdot4((int)xv[v].x, ones, __builtin_amdgcn_sdot4((int)xv[v].y, ones, 0, false), false);
                 part = __builtin_amdgcn_sdot4((int)xv[v].z, ones, __builtin_amdgcn_sdot4((int)xv[v].w, ones, part, false), false);
             }
-        } else if (idx < nvec) {
+        } else if (prow >= 0) {
             const int row = prow;
-            const int col = idx - row * vec_per_row;
+            const int col = pcol;
             const float sf = mode == 0 ? quant_scale<0>(amax_bits[row]) : quant_scale<1>(amax_bits[row]);
             const uint2 qv = mode == 0 ? quant_vec8<0>(xv[v], sf) : quant_vec8<1>(xv[v], sf);
-            *(uint2*)(lds_q + (size_t)row * kp + col * 8) = qv;
+            *(uint2*)(lds_q + row * kp + col * 8) = qv;
             const int ones = 0x01010101;
             part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, 0, false), false);
             if (col == 0) {
@@ -1136,27 +1159,24 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     lds_barrier();
 
     const bool tok_ok = p < M;
-    const int8_t* brow = lds_q + (size_t)(tok_ok ? p : 0) * kp + g * 16;
+    const int8_t* brow = lds_q + (tok_ok ? p : 0) * kp + g * 16;
     v4i acc = {0, 0, 0, 0};
     for (int base = ks * UPW; base < units; base += S * UPW) {
         if (base != ks * UPW) {
+            w_voff += S * (UPW * 256);
 #pragma unroll
-            for (int j = 0; j < UPW; ++j) {
-                const int u = base + j;
-                w[j] = __builtin_nontemporal_load(wrow + (size_t)(u < units ? u : units - 1) * 64);
-            }
+            for (int j = 0; j < UPW; ++j) w[j] = FUSED_WLOAD(j);
         }
         // all B operands of the round first (independent LDS reads, one wait);
-        // a k-step past the end contributes nothing because its A operand is zero
+        // a k-step past the end contributes nothing because its A operand is zero:
+        // its B operand is whatever follows in LDS (the next token's row or the
+        // tail padding of the allocation), read without clamping
         v4i b[UPW];
 #pragma unroll
-        for (int j = 0; j < UPW; ++j) {
-            const int u = base + j;
-            b[j] = *(const v4i*)(brow + (size_t)(u < units ? u : units - 1) * 64);
-        }
+        for (int j = 0; j < UPW; ++j) b[j] = *(const v4i*)(brow + (base + j) * 64);
 #pragma unroll
         for (int j = 0; j < UPW; ++j) {
-            const uint32_t wj = (base + j < units) ? w[j] : 0u;
+            const uint32_t wj = w[j];  // zero past the end of K
             v4i a;
             a.x = (int)(wj & 0x03030303u);
             a.y = (int)((wj >> 2) & 0x03030303u);
@@ -1294,7 +1314,7 @@ struct FusedPlan {
 // The activation block a workgroup of the fused kernel may hold in LDS: what a
 // kernel gets without asking when it also quantizes the block; the
 // pre-quantized variant raises its limit (see raise_fused_lds).
-constexpr size_t kFusedLdsPlain = 60u * 1024u;
+constexpr size_t kFusedLdsPlain = 58u * 1024u;
 constexpr size_t kFusedLdsRaised = 144u * 1024u;
 // Above this many activation elements the quantizer (and what precedes it)
 // runs once in a kernel of its own instead of in every workgroup.
@@ -1303,6 +1323,7 @@ constexpr int kFuseMaxElems = 16384;
 FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
     FusedPlan pl = {1, 1, 4, 1, false};
     if (M > kFusedMaxTokens) return pl;
+    if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31) return pl;  // the kernel addresses the weights with 32-bit byte offsets
     if ((size_t)M * (K + kFusedRowPad) > (pro == 3 ? kFusedLdsRaised : kFusedLdsPlain)) return pl;
     const int units = K / 64;
     if (g_tune_path == 3) {
@@ -1356,7 +1377,7 @@ void raise_fused_lds() {
     static bool done = false;
     if (!done) {
         (void)hipFuncSetAttribute((const void*)bitlinear_fused_kernel<U, V, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)kFusedLdsRaised);
+                                  (int)(kFusedLdsRaised + kFusedTailPad));
         done = true;
     }
 }
@@ -1367,12 +1388,12 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     const int blocks16 = N / 16;
     const dim3 grid((blocks16 + pl.rb - 1) / pl.rb, 1, 1);
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
-    const size_t lds = (size_t)M * (K + kFusedRowPad);
+    const size_t lds = (size_t)M * (K + kFusedRowPad) + kFusedTailPad;
     const uint32_t* wq = (const uint32_t*)packed;
     const int pro = ex.act_scale ? 3 : (ex.norm_weight ? (ex.glu ? 2 : 1) : 0);
 #define BITLINEAR_LAUNCH_UVP(U, V, P)                                                                             \
     hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
-                       s_out, ex, M, N, K, pl.rb, pl.s, mode)
+                       s_out, ex, M, N, K, pl.rb, pl.s, mode, 1.0f / (float)(K / (pro == 3 ? 16 : 8)))
 #define BITLINEAR_LAUNCH_UV(U, V)                    \
     switch (pro) {                                   \
         case 0: BITLINEAR_LAUNCH_UVP(U, V, 0); break; \
