@@ -127,6 +127,16 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     const int p = p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw);
     const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's positions are [lo, hi)
     const bool owns_new = p >= lo && p < lo + span;
+    // Splits whose slice starts beyond the current position have nothing to do and take no part in
+    // the combination: nact splits are active (the comparison chain is p / span + 1 without a
+    // division), and a single active split writes the output itself.  They leave after the first
+    // barrier, not here: a branch on the position in front of phase 1 would make the compiler move
+    // the cache-row loads above behind it, i.e. behind the wait for the position, and serialise two
+    // memory round trips.
+    int nact = 1;
+#pragma unroll
+    for (int k = 1; k < kMaxSplits; ++k) nact += (k < nsplit && p >= k * span) ? 1 : 0;
+    const bool active = sp < nact;
 
     // (1) rope on adjacent pairs, in fp32, results rounded to bf16.  Every split needs q; the
     // split that holds position p also rotates k, keeps k and v of the new token in LDS and
@@ -136,7 +146,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         const int it = tid + u * nthreads;
         const int hh = it / (kHeadDim / 2);
         const int i = it - hh * (kHeadDim / 2);
-        if (it < kItems) {
+        if (it < kItems && active) {
             if (hh <= G) {
                 if (hh < G || owns_new) {
                     const float a = bf16f(praw[u] & 0xffffu), cc = bf16f(praw[u] >> 16);
@@ -156,6 +166,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         }
     }
     __syncthreads();
+    if (!active) return;
 
     // (2) scores with bf16 MFMA 16x16x32 (products of bf16 values are exact in fp32, sums are
     // fp32): A = the rotated q rows (heads, zero rows beyond G), B = 16 cached positions; a lane
@@ -264,7 +275,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
             o0 += part[((size_t)k * G + hh) * kHeadDim + 2 * lane];
             o1 += part[((size_t)k * G + hh) * kHeadDim + 2 * lane + 1];
         }
-        if (nsplit == 1) {
+        if (nact == 1) {
             const float is = 1.0f / red_l[hh];
             *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
         } else {
@@ -279,7 +290,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
             }
         }
     }
-    if (nsplit == 1) return;
+    if (nact == 1) return;
 
     // The last split of this (sequence, kv head) to finish combines the records.  The barrier
     // waits until every thread's record stores have completed (they are write-through, so
@@ -289,7 +300,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     __syncthreads();
     if (tid == 0) {
         const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = done == nsplit - 1;
+        is_last = done == nact - 1;
         if (is_last) __hip_atomic_store(&counters[b * n_kv_heads + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
@@ -299,7 +310,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         float mk[kMaxSplits], lk[kMaxSplits], p0[kMaxSplits], p1[kMaxSplits];
 #pragma unroll
         for (int k = 0; k < kMaxSplits; ++k) {
-            const float* r = rec + ((size_t)(k < nsplit ? k : 0) * G + hh) * kRecFloats;
+            const float* r = rec + ((size_t)(k < nact ? k : 0) * G + hh) * kRecFloats;
             mk[k] = __hip_atomic_load(r + kHeadDim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             lk[k] = __hip_atomic_load(r + kHeadDim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             p0[k] = __hip_atomic_load(r + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -308,11 +319,11 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         float mx = -INFINITY;
 #pragma unroll
         for (int k = 0; k < kMaxSplits; ++k)
-            if (k < nsplit) mx = fmaxf(mx, mk[k]);
+            if (k < nact) mx = fmaxf(mx, mk[k]);
         float l = 0.0f, o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
         for (int k = 0; k < kMaxSplits; ++k) {
-            if (k < nsplit && lk[k] > 0.0f) {
+            if (k < nact && lk[k] > 0.0f) {
                 const float w = __expf(mk[k] - mx);
                 l += lk[k] * w;
                 o0 += w * p0[k];
