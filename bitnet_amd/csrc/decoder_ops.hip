@@ -639,26 +639,38 @@ __global__ __launch_bounds__(kLmThreads) void lm_head_stream_kernel(const uint16
     }
 }
 
-// Best (value, row) per token over the workgroups' partial results: one workgroup, 16 threads per
-// token.  A kernel of its own: the kernel boundary orders the partial results for free, where a
-// device-wide arrival counter would serialise thousands of atomics on one address.
-__global__ __launch_bounds__(kLmThreads) void lm_head_final_kernel(const float* __restrict__ part_val,
-                                                                   const int* __restrict__ part_idx,
-                                                                   int64_t* __restrict__ token_out, int nparts, int B) {
+// Best (value, row) per token over the workgroups' partial results: one workgroup, one wave per
+// token, eight independent loads per lane in flight (a dependent chain of single loads would cost a
+// memory round trip each).  A kernel of its own: the kernel boundary orders the partial results for
+// free, where a device-wide arrival counter would serialise thousands of atomics on one address.
+constexpr int kLmFinalThreads = kLmMaxTokens * 64;
+__global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const float* __restrict__ part_val,
+                                                                        const int* __restrict__ part_idx,
+                                                                        int64_t* __restrict__ token_out, int nparts, int B) {
     const int tid = threadIdx.x;
-    const int t = tid >> 4, sub = tid & 15;
+    const int t = tid >> 6, sub = tid & 63;
     float v = -INFINITY;
     int i = 0x7fffffff;
-    for (int k = sub; k < nparts; k += 16) {
-        const float ov = part_val[(size_t)k * kLmMaxTokens + t];
-        const int oi = part_idx[(size_t)k * kLmMaxTokens + t];
-        if (lm_better(ov, oi, v, i)) {
-            v = ov;
-            i = oi;
+    constexpr int U = 8;
+    for (int base = sub; base < nparts; base += 64 * U) {
+        float ov[U];
+        int oi[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = base + 64 * u;
+            const size_t at = (size_t)(k < nparts ? k : nparts - 1) * kLmMaxTokens + t;
+            ov[u] = part_val[at];
+            oi[u] = part_idx[at];
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (base + 64 * u < nparts && lm_better(ov[u], oi[u], v, i)) {
+                v = ov[u];
+                i = oi[u];
+            }
     }
 #pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
+    for (int off = 1; off < 64; off <<= 1) {
         const float ov = __shfl_xor(v, off);
         const int oi = __shfl_xor(i, off);
         if (lm_better(ov, oi, v, i)) {
@@ -775,6 +787,6 @@ extern "C" int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_wei
         hipLaunchKernelGGL(lm_head_kernel, dim3(nparts), dim3(kLmThreads), lds, (hipStream_t)stream, y_ws, emb, logits, part_val,
                            part_idx, B, V, K);
     }
-    hipLaunchKernelGGL(lm_head_final_kernel, dim3(1), dim3(kLmThreads), 0, (hipStream_t)stream, part_val, part_idx, token_out, nparts, B);
+    hipLaunchKernelGGL(lm_head_final_kernel, dim3(1), dim3(kLmFinalThreads), 0, (hipStream_t)stream, part_val, part_idx, token_out, nparts, B);
     return hipGetLastError() == hipSuccess ? 0 : 3;
 }
