@@ -709,8 +709,11 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
     if (n_splits > 1 && (!workspace || !counters)) return 2;
     const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // fixed slice of the cache per split
-    // more waves per workgroup keep more cache rows in flight; a slice of 64 rows per 4 waves is plenty
-    int threads = span >= 128 ? 512 : 256;
+    // Eight waves take a slice of up to 128 rows in one round of loads (four waves: 64 rows; a
+    // second round exposes a full memory round trip, about 1 us).  Measured: that wins while every
+    // workgroup has a CU of its own (up to 256 of them); beyond that two 512-thread workgroups
+    // share a CU badly (12.9 -> 16.8 us at 320 workgroups) and 256 threads are the better choice.
+    int threads = (span > 64 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
     if (g_attn_threads) threads = g_attn_threads;
     const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * g * kHeadDim) * sizeof(float);
     if (lds > 96u * 1024u) return 1;
