@@ -40,15 +40,27 @@ __device__ __forceinline__ uint16_t to_bf16(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// Wave-wide reductions with DPP lane permutes (no LDS traffic, no waiting): two quad permutes and
+// two mirrors leave every lane of a 16-lane row with the row's result; the four row results are
+// combined through scalar registers.  All lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_f32(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
 __device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
+    v = fmaxf(v, dpp_f32<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_f32<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_f32<0x141>(v));  // row_half_mirror
+    v = fmaxf(v, dpp_f32<0x140>(v));  // row_mirror
+    return fmaxf(fmaxf(lane_f32(v, 0), lane_f32(v, 16)), fmaxf(lane_f32(v, 32), lane_f32(v, 48)));
 }
 __device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x141>(v);
+    v += dpp_f32<0x140>(v);
+    return (lane_f32(v, 0) + lane_f32(v, 16)) + (lane_f32(v, 32) + lane_f32(v, 48));
 }
 
 // Workspace record of one (sequence, kv head, split): G heads x (128 unnormalised outputs,
