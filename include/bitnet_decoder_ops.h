@@ -32,7 +32,9 @@ extern "C" {
  *   counters  int [B * n_kv_heads], zero before the first call (every call leaves them zero)
  *   n_splits  1..8 workgroups share the S cache rows of one (sequence, kv head) in fixed slices;
  *             with 1, workspace and counters may be NULL.  Calls that share a workspace
- *             must not overlap in time.
+ *             must not overlap in time.  Fastest when B * n_kv_heads * n_splits <= 256 (one
+ *             workgroup per CU: the kernel then runs eight waves per workgroup); splits whose
+ *             slice starts beyond the current position cost almost nothing.
  * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8, and
  * g * (S / n_splits + 16 + 512) * 4 bytes <= 96 KiB.  Returns 0, or 1 (shape), 2 (null
  * pointer), 3 (launch failed).  fp32 accumulation; results agree with an fp32 evaluation of
