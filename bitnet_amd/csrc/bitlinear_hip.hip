@@ -1498,8 +1498,9 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // the kernels below, which read their B operands straight from global.
     if (out && !acc_out && g_tune_staged != 2 && g_tune_path != 1 && g_tune_path != 2) {
         const FusedPlan pl = plan_fused(M, N, K, 3);
-        // measured: staging pays once a workgroup shares the rows between two or more row blocks
-        const bool wanted = g_tune_staged == 1 || (M > kDecodeMaxTokens && (N / 16) >= 432);
+        // measured: up to 4 tokens staging always wins (2.8-4.5 us against 3.1-5.1 at the 2B shapes);
+        // beyond, it pays once a workgroup shares the rows between two or more row blocks
+        const bool wanted = g_tune_staged == 1 || M <= kDecodeMaxTokens || (N / 16) >= 432;
         if (pl.ok && wanted)
             return launch_fused((const uint16_t*)act, packed, out, ws, smap, nullptr, nullptr,
                                 FusedExtras{nullptr, residual, 0.0f, 0, s}, M, N, K, 0, pl, stream);
