@@ -1330,6 +1330,30 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
         pl.rb = g_tune_fused[0];
         pl.s = g_tune_fused[1];
         pl.upw = g_tune_fused[2];
+    } else if (N / 16 >= 1024 && M <= 4) {
+        // Many row blocks (N >= 16384) and few tokens: the matrix is large enough to be bandwidth-bound, and what
+        // measured best there is many small workgroups (four or five waves per row block, several
+        // workgroups per CU covering each other's latencies) that walk K in two to four rounds:
+        // 55296 x 5120: 13.7 us against 18.8 with one large workgroup per CU; 27648 x 10240: 13.2
+        // against 16.4; 20480 x 3200: 5.4 against 7.2.  (With 8 tokens the activation block every
+        // workgroup stages is too large for that: 9.0 against 8.2 us at 20480 x 3200.)
+        const int blocks16 = N / 16;
+        pl.rb = units >= 128 ? 4 : (blocks16 >= 2048 ? 2 : 1);
+        const int cand[9][2] = {{4, 10}, {5, 8}, {4, 8}, {5, 10}, {4, 5}, {5, 5}, {4, 16}, {5, 16}, {4, 4}};
+        int best = -1, best_cost = 1 << 30;
+        for (int i = 0; i < 9; ++i) {
+            const int per_round = cand[i][0] * cand[i][1];
+            const int rounds = (units + per_round - 1) / per_round;
+            const int waste = rounds * per_round - units;
+            // few idle k-steps first, two to four rounds preferred, then the order of the list
+            const int cost = waste * 64 + (rounds > 4 ? 400 * (rounds - 4) : (rounds == 1 ? 34 : 0));
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = i;
+            }
+        }
+        pl.s = cand[best][0];
+        pl.upw = cand[best][1];
     } else {
         // enough row blocks per workgroup to keep about 200 workgroups; up to 8
         // (16 for K > 4096) waves splitting K for each, with the fewest k-steps per wave that fit
@@ -1341,12 +1365,13 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
         const int want_s = units > 64 ? (pro == 0 ? 12 : kMaxWaves) : 8;
         const int max_s = (kMaxWaves / pl.rb) < want_s ? (kMaxWaves / pl.rb) : want_s;
         const int sizes[5] = {4, 5, 8, 10, 16};
-        pl.upw = 16;
+        pl.upw = 0;
         for (int i = 0; i < 5; ++i)
             if ((units + sizes[i] - 1) / sizes[i] <= max_s) {
                 pl.upw = sizes[i];
                 break;
             }
+        if (pl.upw == 0) pl.upw = 8;  // several rounds per wave: short rounds measured best (K = 27648: 9.3 us with 8, 10.7 with 16)
         pl.s = (units + pl.upw - 1) / pl.upw;
         if (pl.s > max_s) pl.s = max_s;
     }
