@@ -263,6 +263,46 @@ def batched_and_prefill(lib, shapes, layers, scales, dev, decode_ms=(2, 4, 8, 16
     return out
 
 
+def large_shapes(lib, dev, budget_bytes=1 << 30):
+    """The other (N, K) of the reference's dispatch table (bitnet_kernels.cu:4-33:
+    the 3B-class and the largest shapes) at M = 1 through the drop-in entry
+    bitlinear_int8xint2: random packed bytes (timing only), rotating over about
+    1 GiB of distinct weight copies so that nothing is cache-hot, 60 dependent
+    launches replayed from a HIP graph."""
+    import torch
+
+    out = {}
+    for (N, K) in ((4800, 3200), (3200, 3200), (20480, 3200), (3200, 10240), (5120, 27648), (55296, 5120)):
+        nbytes = N * K // 4
+        copies = max(2, min(64, budget_bytes // nbytes))
+        w = torch.randint(0, 255, (copies, nbytes), dtype=torch.uint8, device=dev)
+        a = torch.randint(-127, 128, (1, K), dtype=torch.int8, device=dev)
+        s = torch.ones(1, dtype=torch.bfloat16, device=dev)
+        ws = torch.ones(8, dtype=torch.bfloat16, device=dev)
+        o = torch.empty(1, N, dtype=torch.bfloat16, device=dev)
+        nl = 60
+
+        def launch(sp):
+            for i in range(nl):
+                wp = ctypes.c_void_p(w.data_ptr() + (i % copies) * nbytes)
+                lib.bitlinear_int8xint2(_p(a), wp, _p(o), _p(s), _p(ws), 1, N, K, sp)
+                if lib.bitlinear_last_status() != 0:
+                    raise RuntimeError(f"bitlinear_int8xint2 rejected N={N} K={K}")
+
+        run = GraphRun(launch)
+        run.replay(3)
+        best = min(run.timed(5)[1] / 5 for _ in range(3)) * 1e3 / nl  # us per launch
+        out[f"{N}x{K}"] = {
+            "us_per_launch": round(best, 2),
+            "weight_GBps": round(nbytes / best / 1e3, 1),
+            "frac_of_hbm_peak": round(nbytes / best / 1e3 / HBM_PEAK_GBPS, 4),
+            "weight_bytes": nbytes,
+        }
+        del run, w
+        torch.cuda.empty_cache()
+    return {"large_shapes_product_only": out}
+
+
 def end_to_end_decode(batches=(1, 8), prompt_len=512, gen_len=128):
     """Random-init BitNet-b1.58-2B-shaped decoder (30 layers, dim 2560, ffn 6912,
     20/5 heads, vocab 128256, tied bf16 embedding / LM head): a seeded 512-token
@@ -533,6 +573,7 @@ def main():
     }
     if not args.no_sweeps:
         result.update(batched_and_prefill(lib, shapes, layers, scales, dev))
+        result.update(large_shapes(lib, dev))
     if not args.no_e2e:
         del path, gemv, quant, layers
         torch.cuda.empty_cache()
