@@ -233,6 +233,30 @@ def test_fused_forward_equals_oracle_chain(n, k, m, mode):
     assert np.array_equal(host_bits(sd), s_bits)
 
 
+@pytest.mark.parametrize("m", [1, 3, 4])
+@pytest.mark.parametrize("n,k", [(20480, 3200), (16384, 2560), (16400, 6912), (55296, 5120)])
+def test_many_row_blocks_launch_shape(n, k, m):
+    """N >= 16384 with up to 4 tokens runs small workgroups that walk K in
+    several rounds (one, two and three rounds, with and without idle k-steps
+    in the last one, at these K): the drop-in product and the forward call,
+    bit for bit against the oracle."""
+    lib = _lib.load_library()
+    rng = np.random.default_rng(7 * n + k + m)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    xb = o.f32_to_bf16_bits(x)
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    q, s_bits = o.quant_input(xb, 0)
+    _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    pk = _packed_dev(w)
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(q), pk, dev_bf16(s_bits), dev_bf16(ws_bits))
+    _assert_bits_equal(host_bits(out), want, "drop-in product")
+    st, out2, qd, sd = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
+    assert st == 0
+    _assert_bits_equal(host_bits(out2), want, "forward")
+    assert np.array_equal(qd.cpu().numpy(), q)
+
+
 def test_fused_forward_launch_shapes_and_null_workspaces():
     lib = _lib.load_library()
     n, k = 2560, 2560
