@@ -82,7 +82,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // on the scalar unit: loops over a wave's positions are uniform
     const int nthreads = blockDim.x;
     const int nwaves = nthreads >> 6;
     const int kvh = blockIdx.x;
@@ -98,7 +98,12 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     // This split owns positions [lo, lo + span): a fixed slice of the cache, whatever the current
     // position is, so its rows can be requested before the position is known.  span % 16 == 0.
     const int lo = sp * span;
+    // Behind the scores: one 4 KB region per wave.  During P.V it stages the wave's 16 V rows of a
+    // round (so that the loop over them need not be unrolled), afterwards it holds the wave's partial
+    // outputs [G][128] for the reduction over the waves.
+    constexpr int kWaveRegion = 1024;  // floats
     float* part = sc + (size_t)G * span;
+    uint32_t* vst = (uint32_t*)part + wave * kWaveRegion;
 
     // The kernel is a chain of memory round trips of a microsecond or more each, so everything
     // that does not depend on anything else is requested first and at once: the position, this
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     // the host cannot see this device-side value, so it is clamped here (the result for such a
     // sequence is then meaningless, but nothing outside the buffers is touched).
     const int64_t p_raw = positions[b];
-    const int p = p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw);
+    const int p = __builtin_amdgcn_readfirstlane(p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw));
     const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's positions are [lo, hi)
     const bool owns_new = p >= lo && p < lo + span;
     // Splits whose slice starts beyond the current position have nothing to do and take no part in
@@ -249,6 +254,11 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     float a0[G], a1[G];
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) a0[hh] = a1[hh] = 0.0f;
+    // Straight-line code that runs once costs instruction fetch on top of its execution (about
+    // twice as much per instruction as code in a loop), and 16 unrolled positions x G heads were
+    // the longest stretch of it in this kernel: the rows go through the wave's LDS region and a
+    // short loop walks them.
+    const int nw_shift = nwaves == 8 ? 3 : 2;  // nwaves is 4 or 8
     for (int s0 = lo + wave; s0 < hi; s0 += nwaves * U) {
         if (s0 != lo + wave) {
 #pragma unroll
@@ -258,24 +268,34 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
             }
         }
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
+        for (int j = 0; j < U; ++j) vst[j * 64 + lane] = vr[j];
+        // same wave writes and reads: LDS operations of a wave complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int left = (hi - s0 + nwaves - 1) >> nw_shift;  // positions of this wave from s0 on
+        const int cnt = left < U ? left : U;
+#pragma unroll 2
+        for (int j = 0; j < cnt; ++j) {
             const int s = s0 + j * nwaves;
-            if (s < hi) {
-                const uint32_t pr = s == p ? *(const uint32_t*)(&vnew[2 * lane]) : vr[j];
-                const float v0 = bf16f(pr & 0xffffu), v1 = bf16f(pr >> 16);
+            const uint32_t* src = s == p ? (const uint32_t*)vnew + lane : vst + j * 64 + lane;
+            const uint32_t pr = *src;
+            const float v0 = bf16f(pr & 0xffffu), v1 = bf16f(pr >> 16);
 #pragma unroll
-                for (int hh = 0; hh < G; ++hh) {
-                    const float pw = sc[(size_t)hh * span + (s - lo)];
-                    a0[hh] += pw * v0;
-                    a1[hh] += pw * v1;
-                }
+            for (int hh = 0; hh < G; ++hh) {
+                const float pw = sc[(size_t)hh * span + (s - lo)];
+                a0[hh] += pw * v0;
+                a1[hh] += pw * v1;
             }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
-        part[((size_t)wave * G + hh) * kHeadDim + 2 * lane] = a0[hh];
-        part[((size_t)wave * G + hh) * kHeadDim + 2 * lane + 1] = a1[hh];
+        part[(size_t)wave * kWaveRegion + hh * kHeadDim + 2 * lane] = a0[hh];
+        part[(size_t)wave * kWaveRegion + hh * kHeadDim + 2 * lane + 1] = a1[hh];
     }
     __syncthreads();
 
@@ -284,8 +304,8 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     for (int hh = wave; hh < G; hh += nwaves) {
         float o0 = 0.0f, o1 = 0.0f;
         for (int k = 0; k < nwaves; ++k) {
-            o0 += part[((size_t)k * G + hh) * kHeadDim + 2 * lane];
-            o1 += part[((size_t)k * G + hh) * kHeadDim + 2 * lane + 1];
+            o0 += part[(size_t)k * kWaveRegion + hh * kHeadDim + 2 * lane];
+            o1 += part[(size_t)k * kWaveRegion + hh * kHeadDim + 2 * lane + 1];
         }
         if (nact == 1) {
             const float is = 1.0f / red_l[hh];
@@ -727,7 +747,7 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     // share a CU badly (12.9 -> 16.8 us at 320 workgroups) and 256 threads are the better choice.
     int threads = (span > 64 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
     if (g_attn_threads) threads = g_attn_threads;
-    const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * g * kHeadDim) * sizeof(float);
+    const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * 1024) * sizeof(float);  // scores + one 4 KB region per wave
     if (lds > 96u * 1024u) return 1;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
 #define BITNET_ATTN_LAUNCH(GG)                                                                                        \

@@ -36,7 +36,7 @@ extern "C" {
  *             workgroup per CU: the kernel then runs eight waves per workgroup); splits whose
  *             slice starts beyond the current position cost almost nothing.
  * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8, and
- * g * (S / n_splits + 16 + 512) * 4 bytes <= 96 KiB.  Returns 0, or 1 (shape), 2 (null
+ * g * (S / n_splits + 16) * 4 bytes + 32 KiB <= 96 KiB.  Returns 0, or 1 (shape), 2 (null
  * pointer), 3 (launch failed).  fp32 accumulation; results agree with an fp32 evaluation of
  * the same formula to about 1e-2 relative on bf16 outputs.
  */
