@@ -95,6 +95,16 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     uint16_t* ck = cache_k + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
     uint16_t* cv = cache_v + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
     const int c = lane & 15, g4 = lane >> 4;
+    // Cached rows are read through buffer descriptors that span this (sequence, kv head)'s rows:
+    // 32-bit byte offsets with the uniform part formed on the scalar unit, and a row past the end
+    // of the cache is out of range and reads as zero (such rows are ignored anyway), so no index
+    // needs clamping.
+    const int row_bytes = n_kv_heads * kHeadDim * 2;  // bytes between positions
+    const int cache_bytes = (S - 1) * row_bytes + kHeadDim * 2;
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)ck, 0, cache_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cv, 0, cache_bytes, 0x00020000);
+    const int k_lane_off = c * row_bytes + g4 * 16;  // K: lane = (position c of a block of 16, 16-byte piece g4 of a 64-byte step)
+    const int v_lane_off = lane * 4;                 // V: lane = dims 2 * lane, 2 * lane + 1 of one position
     // This split owns positions [lo, lo + span): a fixed slice of the cache, whatever the current
     // position is, so its rows can be requested before the position is known.  span % 16 == 0.
     const int lo = sp * span;
@@ -123,20 +133,17 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         const int src = hh < G ? (kvh * G + hh) * kHeadDim : (hh == G ? (n_heads + kvh) : (n_heads + n_kv_heads + kvh)) * kHeadDim;
         praw[u] = *(const uint32_t*)(row + (it < kItems ? src + 2 * i : 0));
     }
-    uint4 kb[R][4];
+    v4u kb[R][4];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int s = lo + wave * 16 + r * nwaves * 16 + c;
-        const uint16_t* kr = ck + (size_t)(s < S ? s : S - 1) * cache_row + g4 * 8;
+        const int off = k_lane_off + (lo + wave * 16 + r * nwaves * 16) * row_bytes;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) kb[r][kk] = *(const uint4*)(kr + kk * 32);
+        for (int kk = 0; kk < 4; ++kk) kb[r][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
     }
     uint32_t vr[U];
 #pragma unroll
-    for (int j = 0; j < U; ++j) {
-        const int s = lo + wave + j * nwaves;
-        vr[j] = *(const uint32_t*)(cv + (size_t)(s < S ? s : S - 1) * cache_row + 2 * lane);
-    }
+    for (int j = 0; j < U; ++j)
+        vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, v_lane_off + (lo + wave + j * nwaves) * row_bytes, 0, 0);
     // A position outside the cache would index the rope tables and the cache rows out of range;
     // the host cannot see this device-side value, so it is clamped here (the result for such a
     // sequence is then meaningless, but nothing outside the buffers is touched).
@@ -202,10 +209,9 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
             if (s0 != lo + wave * 16) {  // later rounds of a long slice
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    const int s = s0 + r * nwaves * 16 + c;
-                    const uint16_t* kr = ck + (size_t)(s < S ? s : S - 1) * cache_row + g4 * 8;
+                    const int off = k_lane_off + (s0 + r * nwaves * 16) * row_bytes;
 #pragma unroll
-                    for (int kk = 0; kk < 4; ++kk) kb[r][kk] = *(const uint4*)(kr + kk * 32);
+                    for (int kk = 0; kk < 4; ++kk) kb[r][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
                 }
             }
 #pragma unroll
@@ -214,8 +220,8 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
                 v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
-                    uint4 kv = kb[r][kk];
-                    if (s == p) kv = *(const uint4*)(&knew[kk * 32 + g4 * 8]);
+                    v4u kv = kb[r][kk];
+                    if (s == p) kv = *(const v4u*)(&knew[kk * 32 + g4 * 8]);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[kk], __builtin_bit_cast(v8bf, kv), acc, 0, 0, 0);
                 }
                 // result lane: position c, heads 4 * g4 + j in register j
@@ -262,10 +268,8 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     for (int s0 = lo + wave; s0 < hi; s0 += nwaves * U) {
         if (s0 != lo + wave) {
 #pragma unroll
-            for (int j = 0; j < U; ++j) {
-                const int s = s0 + j * nwaves;
-                vr[j] = *(const uint32_t*)(cv + (size_t)(s < S ? s : S - 1) * cache_row + 2 * lane);
-            }
+            for (int j = 0; j < U; ++j)
+                vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, v_lane_off + (s0 + j * nwaves) * row_bytes, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < U; ++j) vst[j * 64 + lane] = vr[j];
@@ -740,6 +744,7 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     if (n_splits < 1 || n_splits > kMaxSplits) return 1;
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
     if (n_splits > 1 && (!workspace || !counters)) return 2;
+    if ((size_t)(S + 512) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;  // the kernel's 32-bit byte offsets into one sequence's cache
     const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // fixed slice of the cache per split
     // Eight waves take a slice of up to 128 rows in one round of loads (four waves: 64 rows; a
     // second round exposes a full memory round trip, about 1 us).  Measured: that wins while every
