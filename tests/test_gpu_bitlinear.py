@@ -257,6 +257,59 @@ def test_many_row_blocks_launch_shape(n, k, m):
     assert np.array_equal(qd.cpu().numpy(), q)
 
 
+def _random_shape_cases(count=36, seed=20240611):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        n = 16 * int(rng.integers(1, 260))
+        if len(cases) % 6 == 5:
+            n = 16 * int(rng.integers(1024, 1400))  # many row blocks: the small-workgroup launch shape
+        k = 64 * int(rng.integers(1, 121))
+        m = int(rng.integers(1, 17))
+        if n * k > 9_000_000:
+            continue
+        cases.append((n, k, m))
+    return cases
+
+
+@pytest.mark.parametrize("n,k,m", _random_shape_cases())
+def test_random_shapes_product_forward_and_norm_forward(n, k, m):
+    """Seeded random (N, K, M) outside the model shapes: ragged row blocks, K that
+    no wave count divides, every launch-shape rule; drop-in product, forward and
+    norm forward (with residual) against the oracle, bit for bit."""
+    import ctypes
+
+    lib = _lib.load_library()
+    rng = np.random.default_rng(n * 31 + k * 7 + m)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    x = rng.standard_normal((m, k)).astype(np.float32) * float(rng.choice([0.03, 1.0, 40.0]))
+    xb = o.f32_to_bf16_bits(x)
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    q, s_bits = o.quant_input(xb, 0)
+    _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    pk = _packed_dev(w)
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(q), pk, dev_bf16(s_bits), dev_bf16(ws_bits))
+    _assert_bits_equal(host_bits(out), want, "drop-in product")
+    st, out2, qd, sd = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
+    assert st == 0
+    _assert_bits_equal(host_bits(out2), want, "forward")
+    assert np.array_equal(qd.cpu().numpy(), q)
+    assert np.array_equal(host_bits(sd), s_bits)
+    # norm forward with a residual
+    gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+    rb = o.f32_to_bf16_bits(rng.standard_normal((m, n)).astype(np.float32))
+    want_n = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=rb)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    xd, g, r, wsd = dev_bf16(xb), dev_bf16(gb), dev_bf16(rb), dev_bf16(ws_bits)
+    out3 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    q_ws = torch.empty(m, k, dtype=torch.int8, device="cuda")
+    s_ws = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+    st = lib.bitlinear_norm_forward_bf16(P(xd), P(g), 1e-5, 0, P(pk), P(wsd), P(r), P(out3), P(q_ws), P(s_ws), m, n, k, 0, None)
+    torch.cuda.synchronize()
+    assert st == 0
+    _assert_bits_equal(host_bits(out3), want_n, "norm forward")
+
+
 def test_fused_forward_launch_shapes_and_null_workspaces():
     lib = _lib.load_library()
     n, k = 2560, 2560
