@@ -310,6 +310,36 @@ def test_random_shapes_product_forward_and_norm_forward(n, k, m):
     _assert_bits_equal(host_bits(out3), want_n, "norm forward")
 
 
+def _random_prefill_cases(count=14, seed=977):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        n = 16 * int(rng.integers(1, 400))
+        k = 64 * int(rng.integers(1, 60))
+        m = int(rng.integers(17, 700))
+        if n * k * m > 1_500_000_000:
+            continue
+        cases.append((n, k, m))
+    return cases
+
+
+@pytest.mark.parametrize("n,k,m", _random_prefill_cases())
+def test_random_shapes_beyond_decode_sizes(n, k, m):
+    """Seeded random (N, K, M) with M > 16: whichever of the split-K kernel and
+    the MFMA GEMM the library picks, ragged row and column tiles, a ragged last
+    k-chunk; int32 accumulators and scaled outputs bit for bit."""
+    rng = np.random.default_rng(n + 3 * k + 5 * m)
+    w, a = _rand_case(n, k, m, seed=n + k + m)
+    s_bits = o.f32_to_bf16_bits((0.5 + 3.0 * rng.random(m)).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    acc_want, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    pk = _packed_dev(w)
+    acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), pk)
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    out = bitlinear.bitnet_int8xint2_linear(dev_i8(a), pk, dev_bf16(s_bits), dev_bf16(ws_bits))
+    _assert_bits_equal(host_bits(out), want, "scaled output")
+
+
 def test_fused_forward_launch_shapes_and_null_workspaces():
     lib = _lib.load_library()
     n, k = 2560, 2560
