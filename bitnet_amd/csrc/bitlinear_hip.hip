@@ -683,6 +683,7 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
 // Per-token absmax quantizer: one workgroup per token row
 // ---------------------------------------------------------------------------
 constexpr int kQuantThreads = 256;
+constexpr int kQuantMaxThreads = 1024;
 constexpr int kQuantRegVecs = 4;  // 16-byte vectors (8 bf16) kept in registers per thread
 
 // max |x| over 8 packed bf16 as a bit pattern (|x| as bf16 bits orders like the values): one
@@ -745,10 +746,11 @@ __device__ __forceinline__ float quant_scale(uint32_t amax_bits) {
 }
 
 template <int MODE>
-__global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint16_t* __restrict__ x,
+__global__ __launch_bounds__(kQuantMaxThreads) void quant_absmax_kernel(const uint16_t* __restrict__ x,
                                                                      int8_t* __restrict__ q,
                                                                      uint16_t* __restrict__ s, int K) {
-    __shared__ uint32_t wmax[kQuantThreads / 64];
+    __shared__ uint32_t wmax[kQuantMaxThreads / 64];
+    const int nthreads = blockDim.x;  // 256, or up to 1024 for long rows so that a row still fits the registers
     const int row = blockIdx.x;
     const int tid = threadIdx.x;
     const int nvec = K >> 3;
@@ -759,7 +761,7 @@ __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint1
     uint32_t am = 0;
 #pragma unroll
     for (int r = 0; r < kQuantRegVecs; ++r) {
-        const int idx = tid + r * kQuantThreads;
+        const int idx = tid + r * nthreads;
         if (idx < nvec) {
             v[r] = xr[idx];
             am = absmax_bits8(v[r], am);
@@ -767,27 +769,25 @@ __global__ __launch_bounds__(kQuantThreads) void quant_absmax_kernel(const uint1
             v[r] = make_uint4(0, 0, 0, 0);
         }
     }
-    for (int idx = tid + kQuantRegVecs * kQuantThreads; idx < nvec; idx += kQuantThreads)
+    for (int idx = tid + kQuantRegVecs * nthreads; idx < nvec; idx += nthreads)
         am = absmax_bits8(xr[idx], am);
 
     // |x| as bf16 bit patterns orders like the values, so the max is an integer max
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) am = max(am, (uint32_t)__shfl_xor((int)am, off));
+    am = wave_max_u32(am);
     if ((tid & 63) == 0) wmax[tid >> 6] = am;
     __syncthreads();
     am = wmax[0];
-#pragma unroll
-    for (int i = 1; i < kQuantThreads / 64; ++i) am = max(am, wmax[i]);
+    for (int i = 1; i < (nthreads >> 6); ++i) am = max(am, wmax[i]);
 
     const float s32 = quant_scale<MODE>(am);
     if (tid == 0) s[row] = f32_to_bf16_rne(s32);
 
 #pragma unroll
     for (int r = 0; r < kQuantRegVecs; ++r) {
-        const int idx = tid + r * kQuantThreads;
+        const int idx = tid + r * nthreads;
         if (idx < nvec) qr[idx] = quant_vec8<MODE>(v[r], s32);
     }
-    for (int idx = tid + kQuantRegVecs * kQuantThreads; idx < nvec; idx += kQuantThreads)
+    for (int idx = tid + kQuantRegVecs * nthreads; idx < nvec; idx += nthreads)
         qr[idx] = quant_vec8<MODE>(xr[idx], s32);
 }
 
@@ -1670,7 +1670,11 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s, int M, int
     if (M < 1 || K < 8 || (K % 8) != 0) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !q || !s) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
-    const dim3 grid(M, 1, 1), block(kQuantThreads, 1, 1);
+    // 256 threads keep rows of up to 8192 elements in registers between the two passes; longer rows
+    // get more threads (a second pass that re-reads the row costs a chain of dependent loads)
+    int threads = kQuantThreads;
+    while (threads < kQuantMaxThreads && K > threads * kQuantRegVecs * 8) threads *= 2;
+    const dim3 grid(M, 1, 1), block(threads, 1, 1);
     if (mode == 0)
         hipLaunchKernelGGL(quant_absmax_kernel<0>, grid, block, 0, (hipStream_t)stream, x, q, s, K);
     else
