@@ -47,6 +47,11 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "bitnet_lm_head_greedy_step": (
+        _c_int,
+        [_c_ptr, _c_ptr, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+         _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "bitnet_lm_head_workgroups": (_c_int, [_c_int]),
     "bitnet_lm_head_set_kernel": (_c_int, [_c_int]),
     "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int, _c_int]),

@@ -680,9 +680,20 @@ __global__ __launch_bounds__(kLmThreads) void lm_head_stream_kernel(const uint16
 // memory round trip each).  A kernel of its own: the kernel boundary orders the partial results for
 // free, where a device-wide arrival counter would serialise thousands of atomics on one address.
 constexpr int kLmFinalThreads = kLmMaxTokens * 64;
+// Optional bookkeeping of a greedy decode step, done by the same kernel instead of four small
+// launches behind it: the token becomes the next step's input, goes into the history row of the
+// current step, and the positions and the step counter advance.  Null pointers: not done.
+struct LmStepBook {
+    int64_t* next_input;  // [B]
+    int64_t* positions;   // [B], each += 1
+    int64_t* history;     // [steps][B], row step_idx[0] written
+    int64_t* step_idx;    // [1], += 1
+};
+
 __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const float* __restrict__ part_val,
                                                                         const int* __restrict__ part_idx,
-                                                                        int64_t* __restrict__ token_out, int nparts, int B) {
+                                                                        int64_t* __restrict__ token_out, int nparts, int B,
+                                                                        LmStepBook book) {
     const int tid = threadIdx.x;
     const int t = tid >> 6, sub = tid & 63;
     float v = -INFINITY;
@@ -714,7 +725,16 @@ __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const fl
             i = oi;
         }
     }
-    if (sub == 0 && t < B) token_out[t] = (int64_t)i;
+    if (sub == 0 && t < B) {
+        token_out[t] = (int64_t)i;
+        if (book.next_input) book.next_input[t] = (int64_t)i;
+        if (book.positions) book.positions[t] += 1;
+        if (book.history && book.step_idx) book.history[book.step_idx[0] * B + t] = (int64_t)i;
+    }
+    if (book.step_idx) {
+        __syncthreads();  // every token's history row index has been read
+        if (tid == 0) book.step_idx[0] += 1;
+    }
 }
 
 }  // namespace
@@ -791,9 +811,9 @@ extern "C" int bitnet_lm_head_workgroups(int V) {
     return (V + rows_per_wg - 1) / rows_per_wg;
 }
 
-extern "C" int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_weight, float eps, const uint16_t* emb,
-                                     uint16_t* y_ws, float* logits, int64_t* token_out, float* part_val,
-                                     int* part_idx, int B, int V, int K, void* stream) {
+static int lm_head_greedy_impl(const uint16_t* h, const uint16_t* norm_weight, float eps, const uint16_t* emb,
+                               uint16_t* y_ws, float* logits, int64_t* token_out, float* part_val, int* part_idx,
+                               const LmStepBook& book, int B, int V, int K, void* stream) {
     if (B < 1 || B > kLmMaxTokens || V < 1 || K < 64 || (K % 64) != 0) return 1;
     if (!h || !norm_weight || !emb || !y_ws || !token_out || !part_val || !part_idx) return 2;
     if ((((uintptr_t)h) | ((uintptr_t)norm_weight) | ((uintptr_t)emb) | ((uintptr_t)y_ws)) & 15u) return 1;
@@ -827,6 +847,22 @@ extern "C" int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_wei
         hipLaunchKernelGGL(lm_head_kernel, dim3(nparts), dim3(kLmThreads), lds, (hipStream_t)stream, y_ws, emb, logits, part_val,
                            part_idx, B, V, K);
     }
-    hipLaunchKernelGGL(lm_head_final_kernel, dim3(1), dim3(kLmFinalThreads), 0, (hipStream_t)stream, part_val, part_idx, token_out, nparts, B);
+    hipLaunchKernelGGL(lm_head_final_kernel, dim3(1), dim3(kLmFinalThreads), 0, (hipStream_t)stream, part_val, part_idx, token_out, nparts, B, book);
     return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_weight, float eps, const uint16_t* emb,
+                                     uint16_t* y_ws, float* logits, int64_t* token_out, float* part_val,
+                                     int* part_idx, int B, int V, int K, void* stream) {
+    return lm_head_greedy_impl(h, norm_weight, eps, emb, y_ws, logits, token_out, part_val, part_idx,
+                               LmStepBook{nullptr, nullptr, nullptr, nullptr}, B, V, K, stream);
+}
+
+extern "C" int bitnet_lm_head_greedy_step(const uint16_t* h, const uint16_t* norm_weight, float eps, const uint16_t* emb,
+                                          uint16_t* y_ws, float* logits, int64_t* token_out, float* part_val,
+                                          int* part_idx, int64_t* next_input, int64_t* positions, int64_t* history,
+                                          int64_t* step_idx, int B, int V, int K, void* stream) {
+    if ((history != nullptr) != (step_idx != nullptr)) return 2;
+    return lm_head_greedy_impl(h, norm_weight, eps, emb, y_ws, logits, token_out, part_val, part_idx,
+                               LmStepBook{next_input, positions, history, step_idx}, B, V, K, stream);
 }

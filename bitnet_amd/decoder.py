@@ -110,21 +110,26 @@ class LmHeadWorkspace:
         self.part_idx = torch.empty(n, dtype=torch.int32, device=device)
 
 
-def lm_head_greedy(h, norm: "RMSNorm", emb_weight, workspace: LmHeadWorkspace, token_out=None, logits_out=None):
+def lm_head_greedy(h, norm: "RMSNorm", emb_weight, workspace: LmHeadWorkspace, token_out=None, logits_out=None,
+                   next_input=None, positions=None, history=None, step_idx=None):
     """Final RMSNorm + tied bf16 LM head + greedy token in three launches
     (bitnet_lm_head_greedy).  h bf16 [B, dim]; returns int64 [B] (token_out if
-    given); logits_out fp32 [B, vocab] receives the bf16-rounded logits if given."""
+    given); logits_out fp32 [B, vocab] receives the bf16-rounded logits if given.
+    With next_input / positions / history + step_idx (int64 device tensors) the
+    last launch also does a decode step's bookkeeping: next_input = token,
+    positions += 1, history[step_idx[0]] = token, step_idx += 1."""
     B, K = h.shape
     V = emb_weight.shape[0]
     if token_out is None:
         token_out = torch.empty(B, dtype=torch.int64, device=h.device)
-    st = _lib.load_library().bitnet_lm_head_greedy(
-        _ptr(h), _ptr(norm.weight), norm.eps, _ptr(emb_weight), _ptr(workspace.y),
-        _ptr(logits_out) if logits_out is not None else None, _ptr(token_out), _ptr(workspace.part_val),
-        _ptr(workspace.part_idx), B, V, K, _stream_ptr(),
+    opt = lambda t: _ptr(t) if t is not None else None
+    st = _lib.load_library().bitnet_lm_head_greedy_step(
+        _ptr(h), _ptr(norm.weight), norm.eps, _ptr(emb_weight), _ptr(workspace.y), opt(logits_out), _ptr(token_out),
+        _ptr(workspace.part_val), _ptr(workspace.part_idx), opt(next_input), opt(positions), opt(history), opt(step_idx),
+        B, V, K, _stream_ptr(),
     )
     if st != 0:
-        raise _lib.BitLinearLibraryError(f"bitnet_lm_head_greedy: status {st}")
+        raise _lib.BitLinearLibraryError(f"bitnet_lm_head_greedy_step: status {st}")
     return token_out
 
 
@@ -354,7 +359,10 @@ class Generator:
         the input of the following step, position + 1."""
         if self.lm_head:
             h = self.model.decode_hidden_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)
-            lm_head_greedy(h, self.model.norm, self.model.output.weight, self.lm_ws, token_out=self.next_tok)
+            # the step's bookkeeping rides on the last kernel of the LM head
+            lm_head_greedy(h, self.model.norm, self.model.output.weight, self.lm_ws, token_out=self.next_tok,
+                           next_input=self.tok, positions=self.pos, history=self.history, step_idx=self.step_idx)
+            return
         else:
             if self.fused:
                 logits = self.model.forward_decode_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)

@@ -73,6 +73,19 @@ int bitnet_lm_head_greedy(const uint16_t* h, const uint16_t* norm_weight, float 
                           int64_t* token_out, float* part_val, int* part_idx,
                           int B, int V, int K, void* stream);
 
+/*
+ * The same call with the bookkeeping of a greedy decode loop (gpu/generate.py:264-288: the new
+ * token is appended and fed back, the position advances) done by its last kernel instead of by
+ * separate launches: next_input[b] = token, positions[b] += 1, history[step_idx[0] * B + b] = token,
+ * step_idx[0] += 1.  Each of next_input / positions may be NULL (not done); history and step_idx
+ * are given together or not at all (2 otherwise).  All int64, device memory.
+ */
+int bitnet_lm_head_greedy_step(const uint16_t* h, const uint16_t* norm_weight, float eps,
+                               const uint16_t* emb, uint16_t* y_ws, float* logits,
+                               int64_t* token_out, float* part_val, int* part_idx,
+                               int64_t* next_input, int64_t* positions, int64_t* history,
+                               int64_t* step_idx, int B, int V, int K, void* stream);
+
 /* Upper bound of the workgroups bitnet_lm_head_greedy launches for V rows (sizes its scratch);
  * -1 for V < 1. */
 int bitnet_lm_head_workgroups(int V);
