@@ -1232,6 +1232,7 @@ int g_tune_prefill_big = 0;
 int g_tune_prefill_band = 0;  // row tiles per band of the prefill GEMM's tile order, 0 = built-in choice
 int g_tune_staged = 0;  // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
+constexpr int kPrefillFewTiles = 330;   // up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles
 
 int set_status(int st) {
     g_status = st;
@@ -1465,15 +1466,18 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
                                   2 * 128 * kPfRowBytes);
         lds_limit_raised = true;
     }
-    // tile (rows x columns of the output per workgroup): 0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256
-    // measured: the wide tile pays once there are many tiles (about four per CU of the narrow kind)
+    // tile (rows x columns of the output per workgroup): 0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256,
+    // 3 = 64 x 512, 4 = 32 x 128.  Measured: the wide tile pays once there are many tiles (about four
+    // per CU of the narrow kind); with few tiles (up to about 1.3 per CU) half-height tiles put twice as
+    // many workgroups on the machine and finish a tile's chain of k-chunks earlier (M = 128: 11.4 -> 9.0
+    // us at 3840 x 2560, 21.5 -> 16.4 at 2560 x 6912).
     const long long narrow_tiles = (long long)((N + 127) / 128) * ((M + 63) / 64);
-    int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : 0;
+    int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : (narrow_tiles <= kPrefillFewTiles ? 4 : 0);
     if (g_tune_path == 5) tile = g_tune_prefill_big;
     // 1-D grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
     // tiles, fewer when there are not enough row tiles to give every XCD a band
-    const int tm = tile == 1 ? 128 : 64;
-    const int tn = tile == 0 ? 128 : (tile == 3 ? 512 : 256);
+    const int tm = tile == 1 ? 128 : (tile == 4 ? 32 : 64);
+    const int tn = (tile == 0 || tile == 4) ? 128 : (tile == 3 ? 512 : 256);
     const int row_tiles = (M + tm - 1) / tm, col_tiles = (N + tn - 1) / tn;
     int band = row_tiles / 8;
     band = band < 1 ? 1 : (band > 8 ? 8 : band);
@@ -1484,7 +1488,9 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const int seg_cols = (col_tiles + cseg - 1) / cseg;
     const int units = nbands * cseg;
     const dim3 grid(8 * ((units + 7) / 8) * band * seg_cols, 1, 1);
-    if (tile == 1) {
+    if (tile == 4) {
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<1, 1>), grid, block, 2 * 32 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
+    } else if (tile == 1) {
         hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
     } else if (tile == 3) {
         hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
@@ -1512,7 +1518,10 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
             const double groups = (M + 15) / 16;
             const double splitk_us = 3.5 + groups * ((double)N * K / 4.0) / 1.45e6;
             const double tiles = ((N + 127) / 128) * (double)((M + 63) / 64);
-            const double gemm_us = 4.0 + 0.64 * (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
+            const double tiles32 = ((N + 127) / 128) * (double)((M + 31) / 32);
+            const double gemm_us = tiles <= kPrefillFewTiles
+                                       ? 4.4 + 0.45 * (K / 256.0) * (tiles32 > 400.0 ? tiles32 / 400.0 : 1.0)
+                                       : 4.0 + 0.64 * (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
             gemm = gemm_us <= splitk_us;
         }
         if (gemm) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
@@ -1613,7 +1622,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
-        if (a < 0 || a > 3 || b < 0 || b > 64) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 0 || a > 4 || b < 0 || b > 64) return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 5;
         g_tune_prefill_big = a;
         g_tune_prefill_band = b;

@@ -160,7 +160,7 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *             k-steps in flight per wave
  *   kernel 4: bitlinear_forward_bf16 always as two kernels
  *   kernel 5: prefill GEMM (M > 16) with output tile a per workgroup:
- *             0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256, 3 = 64 x 512 (tokens
+ *             0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256, 3 = 64 x 512, 4 = 32 x 128 (tokens
  *             x columns); b = row tiles per band of the tile order (0 = the
  *             library's choice, up to 64)
  *   kernel 6: product of int8 rows (M <= 16) through the kernel that stages

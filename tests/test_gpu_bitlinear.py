@@ -372,7 +372,7 @@ def test_fused_forward_launch_shapes_and_null_workspaces():
         lib.bitlinear_set_tuning(0, 0, 0, 0)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("m,n,k", [(17, 48, 192), (64, 128, 64), (100, 272, 320), (128, 2560, 2560), (129, 3840, 2560),
                                    (300, 1040, 3200), (512, 2560, 6912)])
 def test_prefill_gemm_acc_bit_exact(m, n, k, tile):
