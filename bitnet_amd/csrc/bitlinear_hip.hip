@@ -1320,6 +1320,10 @@ constexpr size_t kFusedLdsRaised = 144u * 1024u;
 // Above this many activation elements the quantizer (and what precedes it)
 // runs once in a kernel of its own instead of in every workgroup.
 constexpr int kFuseMaxElems = 16384;
+// The same with a norm (and gate) in front of the quantizer: the prologue is heavier, the crossover
+// earlier (measured at K = 2560: 3 tokens 5.2 us fused against 5.5, 4 tokens 6.5 against 5.7; at
+// K = 6912: 2 tokens 7.4 against 6.7).
+constexpr int kFuseMaxElemsNorm = 9216;
 
 FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
     FusedPlan pl = {1, 1, 4, 1, false};
@@ -1723,7 +1727,7 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, 
         return set_status(BITLINEAR_ERR_ARG);
     const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
     const FusedPlan pl = plan_fused(M, N, K, glu ? 2 : 1);
-    const bool small = (long long)M * K <= kFuseMaxElems || g_tune_path == 3 || !q_ws || !s_ws;
+    const bool small = (long long)M * K <= kFuseMaxElemsNorm || g_tune_path == 3 || !q_ws || !s_ws;
     if (pl.ok && small && g_tune_path != 4) {
         const FusedExtras ex = {norm_weight, residual, eps, glu ? 1 : 0, nullptr};
         return set_status(launch_fused(x, packed, output0, ws, sm, nullptr, nullptr, ex, M, N, K, mode, pl,
