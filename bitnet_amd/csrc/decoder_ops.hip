@@ -134,16 +134,23 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
         praw[u] = *(const uint32_t*)(row + (it < kItems ? src + 2 * i : 0));
     }
     v4u kb[R][4];
+    // Rows beyond this split's slice belong to other splits: their requests get an offset past the
+    // end of the descriptor instead, which costs no memory access (with eight waves a round covers
+    // 256 K rows and 128 V rows, a slice is often 96 or fewer).
+    constexpr int kPastEnd = 0x7fff0000;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int off = k_lane_off + (lo + wave * 16 + r * nwaves * 16) * row_bytes;
+        const int blk = wave * 16 + r * nwaves * 16;
+        const int off = blk < span ? k_lane_off + (lo + blk) * row_bytes : kPastEnd;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) kb[r][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
     }
     uint32_t vr[U];
 #pragma unroll
-    for (int j = 0; j < U; ++j)
-        vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, v_lane_off + (lo + wave + j * nwaves) * row_bytes, 0, 0);
+    for (int j = 0; j < U; ++j) {
+        const int rel = wave + j * nwaves;
+        vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, rel < span ? v_lane_off + (lo + rel) * row_bytes : kPastEnd, 0, 0);
+    }
     // A position outside the cache would index the rope tables and the cache rows out of range;
     // the host cannot see this device-side value, so it is clamped here (the result for such a
     // sequence is then meaningless, but nothing outside the buffers is touched).
@@ -209,7 +216,8 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
             if (s0 != lo + wave * 16) {  // later rounds of a long slice
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    const int off = k_lane_off + (s0 + r * nwaves * 16) * row_bytes;
+                    const int blk = s0 - lo + r * nwaves * 16;
+                    const int off = blk < span ? k_lane_off + (lo + blk) * row_bytes : kPastEnd;
 #pragma unroll
                     for (int kk = 0; kk < 4; ++kk) kb[r][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
                 }
@@ -268,8 +276,10 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     for (int s0 = lo + wave; s0 < hi; s0 += nwaves * U) {
         if (s0 != lo + wave) {
 #pragma unroll
-            for (int j = 0; j < U; ++j)
-                vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, v_lane_off + (s0 + j * nwaves) * row_bytes, 0, 0);
+            for (int j = 0; j < U; ++j) {
+                const int rel = s0 - lo + j * nwaves;
+                vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, rel < span ? v_lane_off + (lo + rel) * row_bytes : kPastEnd, 0, 0);
+            }
         }
 #pragma unroll
         for (int j = 0; j < U; ++j) vst[j * 64 + lane] = vr[j];
