@@ -960,7 +960,9 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
 
 // PRO 0: plain, 1: RMSNorm in front, 2: squared-ReLU gate + RMSNorm in front,
 // 3: x already holds the int8 rows [M, K] (16 per vector) and ex.act_scale their scales: no quantizer
-template <int UPW, int VMAX, int PRO>
+// RES: a residual is added in the epilogue (its values are requested at the start; an instance of
+// its own, because loads under a runtime branch would make the compiler wait conservatively later)
+template <int UPW, int VMAX, int PRO, bool RES>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
@@ -1044,23 +1046,25 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     // Epilogue operands, raw bits, nothing depends on them until the end.  Nearly always all
     // rows of a workgroup share one weight-scale slot (found with scalar arithmetic): one load
     // with a uniform address here; a workgroup that straddles a slot boundary fetches per row in
-    // the epilogue.  PRO 0 never has a residual.
-    constexpr bool kHasRes = PRO != 0;
+    // the epilogue.
+    constexpr bool kHasRes = RES;
     const int n_first = blockIdx.x * RB * 16;
     const int n_last = (n_first + RB * 16 - 1) < N ? (n_first + RB * 16 - 1) : N - 1;
     const int slot_first = scale_slot_uniform(smap, n_first), slot_last = scale_slot_uniform(smap, n_last);
     const uint16_t wsb_first = ws[slot_first];
     uint16_t e_res[kFusedMaxRB];
     if (kHasRes) {
+        // loads through a descriptor of the residual: output slots this thread does not own get an
+        // offset past its end, which costs no memory access
+        const __amdgpu_buffer_rsrc_t r_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void*)ex.residual, 0, M * N * 2, 0x00020000);
 #pragma unroll
         for (int r = 0; r < kFusedMaxRB; ++r) {
             const int t = tid + r * nthreads;  // output slot t of the workgroup: [row block][reg][lane]
-            int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
-            n = n < N ? n : N - 1;
-            const int m = (t & 15) < M ? (t & 15) : M - 1;
-            // unconditional: without a residual the load re-reads a weight scale and is ignored
-            const uint16_t* rp = ex.residual ? ex.residual : ws;
-            e_res[r] = rp[ex.residual ? (size_t)m * N + n : 0];
+            const int n = (blockIdx.x * RB + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
+            const int m = t & 15;
+            const bool live = t < RB * 256 && m < M && n < N;
+            e_res[r] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r_rsrc, live ? (m * N + n) * 2 : 0x7fff0000, 0, 0);
         }
     }
 
@@ -1213,7 +1217,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
             const float q0 = a * ri;
             const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
             uint16_t o = f32_to_bf16_rne(q * bf16_to_f32(wsb));
-            if (kHasRes && ex.residual) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
+            if (kHasRes) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
             out[(size_t)m * N + n] = o;
         }
     }
@@ -1404,11 +1408,11 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
 // A kernel gets 64 KiB of dynamic LDS without asking; the pre-quantized variant
 // may hold up to 16 rows of 6912 and more, so its limit is raised once per
 // instance (a host-side attribute, no stream work).
-template <int U, int V>
+template <int U, int V, bool R>
 void raise_fused_lds() {
     static bool done = false;
     if (!done) {
-        (void)hipFuncSetAttribute((const void*)bitlinear_fused_kernel<U, V, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        (void)hipFuncSetAttribute((const void*)bitlinear_fused_kernel<U, V, 3, R>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)(kFusedLdsRaised + kFusedTailPad));
         done = true;
     }
@@ -1423,18 +1427,29 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     const size_t lds = (size_t)M * (K + kFusedRowPad) + kFusedTailPad;
     const uint32_t* wq = (const uint32_t*)packed;
     const int pro = ex.act_scale ? 3 : (ex.norm_weight ? (ex.glu ? 2 : 1) : 0);
-#define BITLINEAR_LAUNCH_UVP(U, V, P)                                                                             \
-    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
+    if (pro == 0 && ex.residual) return BITLINEAR_ERR_ARG;  // the plain forward has no residual epilogue
+#define BITLINEAR_LAUNCH_UVPR(U, V, P, R)                                                                            \
+    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P, R>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
                        s_out, ex, M, N, K, pl.rb, pl.s, mode, 1.0f / (float)(K / (pro == 3 ? 16 : 8)))
-#define BITLINEAR_LAUNCH_UV(U, V)                    \
-    switch (pro) {                                   \
-        case 0: BITLINEAR_LAUNCH_UVP(U, V, 0); break; \
-        case 1: BITLINEAR_LAUNCH_UVP(U, V, 1); break; \
-        case 2: BITLINEAR_LAUNCH_UVP(U, V, 2); break; \
-        default:                                     \
-            if (lds > 48u * 1024u) raise_fused_lds<U, V>(); \
-            BITLINEAR_LAUNCH_UVP(U, V, 3);           \
-            break;                                   \
+#define BITLINEAR_LAUNCH_UVP(U, V, P)              \
+    if (ex.residual)                               \
+        BITLINEAR_LAUNCH_UVPR(U, V, P, true);      \
+    else                                           \
+        BITLINEAR_LAUNCH_UVPR(U, V, P, false)
+#define BITLINEAR_LAUNCH_UV(U, V)                                   \
+    switch (pro) {                                                  \
+        case 0: BITLINEAR_LAUNCH_UVPR(U, V, 0, false); break;       \
+        case 1: BITLINEAR_LAUNCH_UVP(U, V, 1); break;               \
+        case 2: BITLINEAR_LAUNCH_UVP(U, V, 2); break;               \
+        default:                                                    \
+            if (lds > 48u * 1024u) {                                \
+                if (ex.residual)                                    \
+                    raise_fused_lds<U, V, true>();                  \
+                else                                                \
+                    raise_fused_lds<U, V, false>();                 \
+            }                                                       \
+            BITLINEAR_LAUNCH_UVP(U, V, 3);                          \
+            break;                                                  \
     }
 #define BITLINEAR_LAUNCH_U(U)                      \
     switch (pl.vmax) {                             \
@@ -1453,6 +1468,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 #undef BITLINEAR_LAUNCH_U
 #undef BITLINEAR_LAUNCH_UV
 #undef BITLINEAR_LAUNCH_UVP
+#undef BITLINEAR_LAUNCH_UVPR
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
