@@ -393,7 +393,7 @@ template <int MT, int NT>
 __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, int M, int N, int K, int band, int cseg) {
+    ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K, int band, int cseg) {
     constexpr int TM = MT * 32;
     constexpr int NTHR = kPfWaves * 64;
     constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
@@ -672,7 +672,15 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
                         const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
                         h[j] = q * wsf[nt][g4 * 4 + j];
                     }
-                    *(uint2*)(out + o) = make_uint2(f32x2_to_bf16x2(h[0], h[1]), f32x2_to_bf16x2(h[2], h[3]));
+                    uint2 ob = make_uint2(f32x2_to_bf16x2(h[0], h[1]), f32x2_to_bf16x2(h[2], h[3]));
+                    if (residual) {  // out = bf16(residual + bf16(result))
+                        const uint2 rv = *(const uint2*)(residual + o);
+                        ob.x = f32x2_to_bf16x2(__uint_as_float(rv.x << 16) + __uint_as_float(ob.x << 16),
+                                               __uint_as_float(rv.x & 0xffff0000u) + __uint_as_float(ob.x & 0xffff0000u));
+                        ob.y = f32x2_to_bf16x2(__uint_as_float(rv.y << 16) + __uint_as_float(ob.y << 16),
+                                               __uint_as_float(rv.y & 0xffff0000u) + __uint_as_float(ob.y & 0xffff0000u));
+                    }
+                    *(uint2*)(out + o) = ob;
                 }
             }
         }
@@ -1473,7 +1481,8 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 }
 
 int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
-                   const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
+                   const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream,
+                   const uint16_t* residual = nullptr) {
     const uint32_t* wq = (const uint32_t*)packed;
     // the kernel addresses the packed weights through a buffer descriptor with 32-bit offsets
     if ((long long)N * K / 4 >= (1ll << 31)) return BITLINEAR_ERR_SHAPE;
@@ -1509,15 +1518,15 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const int units = nbands * cseg;
     const dim3 grid(8 * ((units + 7) / 8) * band * seg_cols, 1, 1);
     if (tile == 4) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<1, 1>), grid, block, 2 * 32 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<1, 1>), grid, block, 2 * 32 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
     } else if (tile == 1) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
     } else if (tile == 3) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
     } else if (tile == 2) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
     } else {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, M, N, K, band, cseg);
+        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
     }
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
@@ -1528,7 +1537,6 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // vector loads: 16-byte groups of both operands must be 16-byte aligned
     if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
     if (M > kPrefillMinTokens && g_tune_path != 2) {
-        if (residual) return BITLINEAR_ERR_SHAPE;  // the residual epilogue exists at decode sizes only
         // A few dozen tokens on a narrow matrix leave most CUs without a GEMM tile, and a tile's
         // chain of 256-k chunks is then pure latency (about 0.64 us each).  There the split-K kernel,
         // run once per 16 tokens and re-reading the weights from L2 (about 1.45 TB/s measured),
@@ -1544,8 +1552,8 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
                                        : 4.0 + 0.64 * (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
             gemm = gemm_us <= splitk_us;
         }
-        if (gemm) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
-        return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+        if (gemm) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
+        return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
     }
     // The kernel that stages the int8 rows in LDS once per workgroup and shares
     // them between several row blocks: fewer activation bytes through L2 than

@@ -99,6 +99,23 @@ def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads
     return out
 
 
+def rope_cache_tokens(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads):
+    """Rope + KV-cache write for T new tokens per sequence in one HIP kernel
+    (bitnet_rope_cache_tokens).  xqkv bf16 [B * T, (n_heads + 2 n_kv) * 128];
+    positions int64 [B, T]; returns the rotated q, bf16 [B, T, n_heads, 128]."""
+    B, T = positions.shape
+    S = cache_k.shape[1]
+    hd = cache_k.shape[-1]
+    q = torch.empty(B, T, n_heads, hd, dtype=torch.bfloat16, device=xqkv.device)
+    st = _lib.load_library().bitnet_rope_cache_tokens(
+        _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(q),
+        B, T, S, n_heads, n_kv_heads, hd, _stream_ptr(),
+    )
+    if st != 0:
+        raise _lib.BitLinearLibraryError(f"bitnet_rope_cache_tokens: status {st}")
+    return q
+
+
 class LmHeadWorkspace:
     """Scratch of bitnet_lm_head_greedy for one (batch, vocabulary, dim)."""
 
@@ -137,7 +154,7 @@ def norm_bitlinear(x, norm: "RMSNorm", lin: BitLinearKernel, glu: bool = False, 
     """[squared-ReLU gate ->] RMSNorm -> BitLinearKernel.forward [-> + residual]
     through bitlinear_norm_forward_bf16: one kernel for small activation blocks,
     a norm/quantizer kernel plus the product kernel for larger ones; x bf16
-    [M, K] (or [M, 2K] with glu), M <= 16 when there is a residual."""
+    [M, K] (or [M, 2K] with glu)."""
     M = x.shape[0]
     K = lin.in_features
     out = torch.empty(M, lin.out_features, dtype=torch.bfloat16, device=x.device)
@@ -258,6 +275,32 @@ class Transformer(nn.Module):
             x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
             h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)
         return h
+
+    @torch.no_grad()
+    def prefill_hidden_fused(self, tokens, cache, cos, sin):
+        """A whole prompt on an empty cache, tokens [B, T] at positions 0..T-1:
+        the layer stack of decode_hidden_fused at prompt size (norms, gate and
+        residual adds folded into the BitLinear calls, which run the int8 GEMM),
+        rope + cache write in one kernel, causal attention over the new tokens
+        by torch's scaled_dot_product_attention (the reference calls xformers'
+        flash attention here, gpu/model.py:147-155).  Returns the hidden state in
+        front of the final norm, [B, T, dim]."""
+        a = self.args
+        B, T = tokens.shape
+        hd = a.dim // a.n_heads
+        pos = torch.arange(T, device=tokens.device)[None, :].expand(B, T).contiguous()
+        h = self.tok_embeddings(tokens.reshape(B * T))
+        for layer, (ck, cv) in zip(self.layers, cache):
+            att, ffn = layer.attention, layer.feed_forward
+            xqkv = norm_bitlinear(h, layer.attention_norm, att.wqkv)
+            q = rope_cache_tokens(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads)
+            o = torch.nn.functional.scaled_dot_product_attention(
+                q.transpose(1, 2), ck[:, :T].transpose(1, 2), cv[:, :T].transpose(1, 2), is_causal=True, enable_gqa=True)
+            o = o.transpose(1, 2).reshape(B * T, a.n_heads * hd)
+            h = norm_bitlinear(o, att.attn_sub_norm, att.wo, residual=h)
+            x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
+            h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)
+        return h.view(B, T, a.dim)
 
     @torch.no_grad()
     def forward_tokens(self, tokens, positions, cache, cos, sin):
@@ -389,6 +432,10 @@ class Generator:
     def prefill(self, prompt: torch.Tensor) -> torch.Tensor:
         """prompt [B, P] int64 -> first generated token [B]."""
         B, P = prompt.shape
+        if self.lm_head:
+            # the prompt through the library's kernels; only the last token's row goes through the LM head
+            h = self.model.prefill_hidden_fused(prompt, self.cache, self.cos, self.sin)
+            return lm_head_greedy(h[:, -1].contiguous(), self.model.norm, self.model.output.weight, self.lm_ws)
         pos = torch.arange(P, device=prompt.device)[None, :].expand(B, P).contiguous()
         logits = self.model.forward_tokens(prompt, pos, self.cache, self.cos, self.sin)
         return torch.argmax(logits[:, -1, :], dim=-1)

@@ -126,8 +126,7 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
  * reference's decoder folded in.  One kernel under the one-kernel conditions of
  * bitlinear_forward_bf16; otherwise a gate / norm / quantizer kernel (one
  * workgroup per token row, K <= 32768) followed by the product kernel, which
- * needs q_ws / s_ws as above.  The residual epilogue exists for M <= 16 only
- * (BITLINEAR_ERR_SHAPE beyond):
+ * needs q_ws / s_ws as above; every product kernel has the residual epilogue:
  *   in front  y = RMSNorm(h) = bf16(h * rsqrt(mean(h^2) + eps) * norm_weight)
  *             (attention_norm / ffn_norm / attn_sub_norm / ffn_sub_norm,
  *             gpu/model.py:159, 195, 228-229); the sum of squares is taken in fp64,

@@ -46,6 +46,22 @@ int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v
                        int* counters, int n_splits, int B, int S, int n_heads,
                        int n_kv_heads, int head_dim, void* stream);
 
+/*
+ * Rotary embedding and KV-cache write for a block of T new tokens per sequence (the prompt
+ * pass of Attention.forward, gpu/model.py:128-157, where the reference calls xformers'
+ * rope_padded): for token (b, t) at position positions[b * T + t]
+ *   - q heads rotated (adjacent pairs, fp32, rounded to bf16) into q_out[b, t, h, :],
+ *   - k heads rotated and v heads copied into cache_k/v[b, position, kvh, :].
+ * The arithmetic is that of bitnet_attn_decode, so both leave identical cache rows.
+ *   qkv bf16 [B * T, (n_heads + 2 n_kv_heads) * head_dim]; positions int64 [B * T] (clamped into
+ *   [0, S) by the kernel); cos/sin fp32 [S, head_dim / 2]; q_out bf16 [B, T, n_heads, head_dim].
+ * head_dim must be 128.  Returns 0, 1 (shape), 2 (null pointer), 3 (launch failed).
+ */
+int bitnet_rope_cache_tokens(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v,
+                             const int64_t* positions, const float* cos_table,
+                             const float* sin_table, uint16_t* q_out, int B, int T, int S,
+                             int n_heads, int n_kv_heads, int head_dim, void* stream);
+
 /* Tuning override for tests and measurements: threads per workgroup of the attention kernel
  * (256 or 512; 0 restores the built-in choice).  Results do not depend on it beyond the
  * order of fp32 additions.  Returns 0, or 1 for another value. */

@@ -515,7 +515,7 @@ def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
     torch.cuda.synchronize()
     assert st == 0
     _assert_bits_equal(host_bits(out), want, "norm forward, no workspaces")
-    # M = 40: norm/quantizer kernel + MFMA GEMM; a residual is refused there
+    # M = 40: norm/quantizer kernel + MFMA GEMM
     m = 40
     xb = o.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
     want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=None)
@@ -527,10 +527,42 @@ def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
     torch.cuda.synchronize()
     assert st == 0
     _assert_bits_equal(host_bits(out), want, "norm forward, M=40")
-    st = lib.bitlinear_norm_forward_bf16(P(xd), P(g), 1e-5, 0, P(pk), P(wsd), P(out), P(out), P(q_ws), P(s_ws), m, n, k, 0, None)
-    assert st == 1
     st = lib.bitlinear_norm_forward_bf16(P(xd), P(g), 1e-5, 0, P(pk), P(wsd), None, P(out), None, None, m, n, k, 0, None)
     assert st != 0
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
+@pytest.mark.parametrize("m,n,k,glu", [(40, 2560, 2560, 0), (130, 3840, 2560, 0), (300, 2560, 6912, 1), (77, 48, 192, 1),
+                                       (513, 1040, 640, 0)])
+def test_norm_forward_with_residual_beyond_decode_sizes(m, n, k, glu, tile):
+    """Prompt-sized blocks: gate / norm / quantizer kernel, then the product with
+    the residual added in its epilogue -- through the library's own choice of
+    product kernel (tile -1: split-K or GEMM) and through every GEMM tile --
+    against the oracle chain, bit for bit."""
+    import ctypes
+
+    lib = _lib.load_library()
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    rng = np.random.default_rng(m + n + k + glu)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    xb = o.f32_to_bf16_bits(rng.standard_normal((m, 2 * k if glu else k)).astype(np.float32) * 1.3)
+    gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+    rb = o.f32_to_bf16_bits(rng.standard_normal((m, n)).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=bool(glu), residual_bits=rb)
+    x, g, pk, wsd, r = dev_bf16(xb), dev_bf16(gb), _packed_dev(w), dev_bf16(ws_bits), dev_bf16(rb)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    q_ws = torch.empty(m, k, dtype=torch.int8, device="cuda")
+    s_ws = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+    try:
+        if tile >= 0:
+            assert lib.bitlinear_set_tuning(5, tile, 0, 0) == 0
+        st = lib.bitlinear_norm_forward_bf16(P(x), P(g), 1e-5, glu, P(pk), P(wsd), P(r), P(out), P(q_ws), P(s_ws), m, n, k, 0, None)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert st == 0
+    _assert_bits_equal(host_bits(out), want, f"norm forward with residual M={m} tile={tile}")
 
 
 @pytest.mark.parametrize("m", [1, 3, 5, 8, 13, 16])

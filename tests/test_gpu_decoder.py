@@ -252,3 +252,63 @@ def test_generator_with_and_without_the_lm_head_kernel_agree():
         outs.append(gen.decode(first, 9, 12).cpu())
     # greedy tokens can only differ where two logits tie within fp32 summation order; with random weights they do not
     assert torch.equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("B,T,S,nh,nkv,start", [(1, 512, 640, 20, 5, 0), (3, 37, 64, 4, 1, 5), (2, 1, 16, 8, 8, 15)])
+def test_rope_cache_tokens_kernel_equals_torch(B, T, S, nh, nkv, start):
+    """Rope + cache write for a block of tokens: the rotated q and the cache
+    rows equal the torch restatement bit for bit (fp32 products, one fp32
+    add, one rounding to bf16), other cache rows untouched."""
+    hd = 128
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(B * 100 + T)
+    xqkv = torch.randn(B * T, (nh + 2 * nkv) * hd, generator=g, device=dev).to(torch.bfloat16)
+    ck = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    cv = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    pos = (start + torch.arange(T, device=dev))[None, :].expand(B, T).contiguous()
+    cos, sin = decoder.rope_tables(hd, S, 500000.0, dev)
+    att = decoder.Attention.__new__(decoder.Attention)
+    torch.nn.Module.__init__(att)
+    att.head_dim, att.n_heads, att.n_kv_heads = hd, nh, nkv
+    q, k, v = att.split_qkv(xqkv.view(B, T, -1))
+    c, s_ = cos[pos][:, :, None, :], sin[pos][:, :, None, :]
+    want_q, want_k = decoder.apply_rope(q, c, s_), decoder.apply_rope(k, c, s_)
+    rk, rv = ck.clone(), cv.clone()
+    rk[:, start:start + T] = want_k
+    rv[:, start:start + T] = v
+    got_q = decoder.rope_cache_tokens(xqkv, ck, cv, pos, cos, sin, nh, nkv)
+    torch.cuda.synchronize()
+    assert torch.equal(got_q, want_q)
+    assert torch.equal(ck, rk) and torch.equal(cv, rv)
+
+
+def test_prompt_through_the_library_kernels_against_the_torch_glue():
+    """Generator.prefill with the prompt-sized layer stack (norm / gate /
+    residual folded into the BitLinear calls, rope + cache kernel, torch's
+    fused attention) against forward_tokens (every op in torch around the same
+    BitLinear kernels, fp32 attention): the first layer's cache rows and the
+    last token's logits within bf16 noise (the norm's and the attention's sums
+    run in another order and precision), and each path's first token equal to
+    the argmax of its own logits."""
+    model = _build(BIG_HEADS, seed=11)
+    B, P, S = 2, 70, 96
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(12)
+    prompt = torch.randint(0, BIG_HEADS.vocab_size, (B, P), generator=g, device=dev)
+    cos, sin = decoder.rope_tables(128, S, BIG_HEADS.rope_theta, dev)
+    c1, c2 = model.make_cache(B, S, dev), model.make_cache(B, S, dev)
+    h1 = model.prefill_hidden_fused(prompt, c1, cos, sin)
+    pos = torch.arange(P, device=dev)[None].expand(B, P).contiguous()
+    logits2 = model.forward_tokens(prompt, pos, c2, cos, sin)
+    torch.cuda.synchronize()
+    for a_, b_ in zip(c1[0], c2[0]):  # the two RMSNorm evaluations differ in the last bf16 bit of a few elements
+        assert torch.allclose(a_.float(), b_.float(), rtol=2e-2, atol=2e-2)
+        assert torch.equal(a_[:, P:], b_[:, P:])  # rows behind the prompt untouched
+    logits1 = model.output(model.norm(h1[:, -1])).float()
+    assert torch.allclose(logits1, logits2[:, -1], rtol=5e-2, atol=5e-2)
+    gen = decoder.Generator(model, B, S)
+    assert gen.lm_head
+    first = gen.prefill(prompt)
+    assert torch.equal(first, torch.argmax(logits1, dim=-1))
+    gen2 = decoder.Generator(model, B, S, fused_head=False)
+    assert torch.equal(gen2.prefill(prompt), torch.argmax(logits2[:, -1], dim=-1))
