@@ -389,20 +389,26 @@ constexpr int kPfRowBytes = kPfChunk + 16;      // padded row: 16-byte reads of 
 constexpr int kPfPieces = kPfChunk / 16;        // 16-byte pieces per row and chunk
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-template <int MT, int NT>
-__global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
+template <int MT, int NT, int KS>
+__global__ __launch_bounds__(kPfWaves * 64 * KS) void gemm_i2_prefill_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
     ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K, int band, int cseg) {
     constexpr int TM = MT * 32;
     constexpr int NTHR = kPfWaves * 64;
     constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
-    extern __shared__ __attribute__((aligned(16))) int8_t lds_a[];  // [2][TM * kPfRowBytes]
-    __shared__ int rowsum[TM];
+    extern __shared__ __attribute__((aligned(16))) int8_t lds_all[];  // [KS][2][TM * kPfRowBytes]
+    __shared__ int rowsum[KS][TM];
     __shared__ float sval[TM];
     __shared__ float rinv[TM];
 
-    const int tid = threadIdx.x;
+    // KS groups of four waves share the tile and split its 256-k chunks between them (group g
+    // takes chunks g, g + KS, ...): with few tiles on the machine a tile's chain of chunks is
+    // pure latency, and KS groups walk it in 1/KS of the time.  Each group stages its own chunks
+    // in its own LDS buffers; the groups' accumulators are added through LDS at the end.
+    const int grp = KS > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x / NTHR) : 0;
+    int8_t* lds_a = lds_all + grp * (2 * TM * kPfRowBytes);
+    const int tid = threadIdx.x % NTHR;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     // Workgroup -> tile.  Workgroups are handed to the 8 XCDs round-robin by
@@ -411,8 +417,9 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     // walks it column tile by column tile.  The workgroups running on an XCD at
     // any time therefore share a few row tiles (kept in that L2 for the whole
     // band) and a few column tiles, instead of every tile pulling both of its
-    // operands through the memory-side cache on its own.  With fewer than 8
-    // bands the column tiles are cut into segments too, so that all XCDs work.
+    // operands through the memory-side cache on its own.  Unless the number of
+    // bands is a multiple of 8, the column tiles are cut into segments too, so
+    // that every XCD gets the same number of (band, segment) units.
     const int row_tiles = (M + TM - 1) / TM;
     const int col_tiles = (N + kPfWaves * NT * 32 - 1) / (kPfWaves * NT * 32);
     const int xcd = blockIdx.x & 7;
@@ -431,7 +438,7 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int nl = lane & 31;
     const int kc = lane >> 5;
     const int ksteps = K >> 5;
-    const int nchunks = (ksteps + kPfSteps - 1) / kPfSteps;
+    const int nchunks = ((ksteps + kPfSteps - 1) / kPfSteps + KS - 1) / KS;  // per group; chunk c of group g is chunk c * KS + g of the row
 
     // All loads of the main loop are buffer loads: base (a resource descriptor in
     // scalar registers) + a per-lane byte offset computed once + a scalar offset
@@ -462,7 +469,7 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
         n = n < N ? n : N - 1;
         w_off[nt] = ((n >> 4) * K + ((n & 15) >> 3) * 16 + kc * 8 + (n & 7)) * 4;
     }
-    if (tid < TM) {
+    if (threadIdx.x < TM) {
         const float sv = bf16_to_f32(out ? s[(m0 + tid) < M ? (m0 + tid) : (M - 1)] : (uint16_t)0x3f80);
         sval[tid] = sv;
         rinv[tid] = 1.0f / sv;
@@ -494,15 +501,15 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     const int last_step_off = (ksteps - 1) * 128;  // byte offset of the last 32-k step inside a row block
     auto load_piece = [&](int c, int i) -> v4i {
         // a chunk past the end re-reads chunk 0; it is never staged into a buffer that is multiplied
-        const int k0 = c * kPfChunk < K ? c * kPfChunk : 0;
+        const int k0 = (c * KS + grp) * kPfChunk < K ? (c * KS + grp) * kPfChunk : 0;
         return __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], k0, 0);
     };
     auto load_word = [&](int c, int ks, int nt) -> uint32_t {
-        const int so = (c * kPfSteps + ks) * 128;
+        const int so = ((c * KS + grp) * kPfSteps + ks) * 128;
         return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_off[nt], so < last_step_off ? so : last_step_off, 0);
     };
     auto stage_piece = [&](int c, int i, const v4i& piece, int8_t* buf) {
-        const v4i v = (c * kPfChunk + a_koff[i]) >= K ? zero4 : piece;  // ragged last chunk, or a chunk past the end
+        const v4i v = ((c * KS + grp) * kPfChunk + a_koff[i]) >= K ? zero4 : piece;  // ragged last chunk, or a chunk past the end
         *(v4i*)(buf + a_dst[i]) = v;
         rs[i] = __builtin_amdgcn_sdot4(v.x, ones, rs[i], false);
         rs[i] = __builtin_amdgcn_sdot4(v.y, ones, rs[i], false);
@@ -608,9 +615,35 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
         v += dpp_move<0x4E>(v);
         v += dpp_move<0x141>(v);
         v += dpp_move<0x140>(v);
-        if ((tid & 15) == 0) rowsum[(tid + i * NTHR) / kPfPieces] = v;
+        if ((tid & 15) == 0) rowsum[grp][(tid + i * NTHR) / kPfPieces] = v;
     }
-    lds_barrier();
+    if (KS > 1) {
+        // groups 1.. leave their accumulators in LDS (the staging buffers are free: every wave is
+        // past the barrier of its last chunk) and are done; group 0 adds them up and finishes the tile
+        int* red = (int*)lds_all;  // [KS - 1][kPfWaves][MT * NT * 16][64]
+        if (grp > 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        red[(((grp - 1) * kPfWaves + wave) * (MT * NT * 16) + (mt * NT + nt) * 16 + r) * 64 + lane] = acc[mt][nt][r];
+        }
+        lds_barrier();
+        if (grp > 0) return;
+#pragma unroll
+        for (int g = 1; g < KS; ++g)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[mt][nt][r] += red[(((g - 1) * kPfWaves + wave) * (MT * NT * 16) + (mt * NT + nt) * 16 + r) * 64 + lane];
+    } else {
+        lds_barrier();
+    }
 
     // The weights are the MFMA's row operand, so a result lane holds one token
     // (m = lane % 32 of the row tile) and, in register r, output column
@@ -649,7 +682,9 @@ __global__ __launch_bounds__(kPfWaves * 64) void gemm_i2_prefill_kernel(
     for (int mt = 0; mt < MT; ++mt) {
         const int ml = mt * 32 + nl;
         const int m = m0 + ml;
-        const int rs2 = 2 * rowsum[ml];
+        int rs2 = 0;
+#pragma unroll
+        for (int g = 0; g < KS; ++g) rs2 += 2 * rowsum[g][ml];
         const float sv = sval[ml], ri = rinv[ml];
         if (m >= M) continue;
 #pragma unroll
@@ -1242,9 +1277,13 @@ int g_tune_path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K ker
 int g_tune_fused[3] = {1, 10, 4};
 int g_tune_prefill_big = 0;
 int g_tune_prefill_band = 0;  // row tiles per band of the prefill GEMM's tile order, 0 = built-in choice
+int g_tune_prefill_ks = 0;    // groups of waves splitting K in the small prefill tiles, 0 = built-in choice
 int g_tune_staged = 0;  // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 constexpr int kPrefillFewTiles = 330;   // up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles
+constexpr int kPrefillSplit2Tiles = 320;  // up to this many 32 x 128 tiles two groups of waves split a tile's K,
+constexpr int kPrefillSplit4Tiles = 160;  // up to this many, and a long K, four
+constexpr int kPrefillSplit4MinK = 5120;
 
 int set_status(int st) {
     g_status = st;
@@ -1486,13 +1525,16 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const uint32_t* wq = (const uint32_t*)packed;
     // the kernel addresses the packed weights through a buffer descriptor with 32-bit offsets
     if ((long long)N * K / 4 >= (1ll << 31)) return BITLINEAR_ERR_SHAPE;
-    const dim3 block(kPfWaves * 64, 1, 1);
-    // the large tile double-buffers 2 x 128 rows x 272 bytes = 68 KiB of LDS: above the 64 KiB a
-    // kernel gets without asking (a host-side attribute, set once per process)
+    // the large tile double-buffers 2 x 128 rows x 272 bytes = 68 KiB of LDS (so do four groups of the
+    // small one): above the 64 KiB a kernel gets without asking (a host-side attribute, set once per process)
     static bool lds_limit_raised = false;
     if (!lds_limit_raised) {
-        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<4, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<4, 2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   2 * 128 * kPfRowBytes);
+        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<1, 1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  4 * 2 * 32 * kPfRowBytes);
+        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<2, 1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  2 * 2 * 64 * kPfRowBytes);
         lds_limit_raised = true;
     }
     // tile (rows x columns of the output per workgroup): 0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256,
@@ -1503,6 +1545,19 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const long long narrow_tiles = (long long)((N + 127) / 128) * ((M + 63) / 64);
     int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : (narrow_tiles <= kPrefillFewTiles ? 4 : 0);
     if (g_tune_path == 5) tile = g_tune_prefill_big;
+    // groups of waves that split a tile's K between them (small tiles only): while the small tiles
+    // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
+    // instruction stream, and more groups shorten it
+    const long long small_tiles = (long long)((N + 127) / 128) * ((M + 31) / 32);
+    int ks = 1;
+    // measured at M = 128: 9.0 -> 8.0 us at K = 2560 with two groups (four: 9.0), 16.6 -> 13.1 -> 12.6 at
+    // K = 6912 with two and four; with more than one tile per CU the groups only compete (M = 512, 3840 x 2560:
+    // 11.6 -> 13.6 us)
+    if (tile == 4 && small_tiles <= kPrefillSplit2Tiles)
+        ks = (small_tiles <= kPrefillSplit4Tiles && K >= kPrefillSplit4MinK) ? 4 : 2;
+    if (g_tune_path == 5 && g_tune_prefill_ks > 0) ks = (tile == 4 || (tile == 0 && g_tune_prefill_ks == 2)) ? g_tune_prefill_ks : 1;
+    if (K <= kPfChunk * (ks - 1)) ks = 1;  // fewer chunks than groups
+    const dim3 block(kPfWaves * 64 * ks, 1, 1);
     // 1-D grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
     // tiles, fewer when there are not enough row tiles to give every XCD a band
     const int tm = tile == 1 ? 128 : (tile == 4 ? 32 : 64);
@@ -1512,22 +1567,40 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     band = band < 1 ? 1 : (band > 8 ? 8 : band);
     if (g_tune_path == 5 && g_tune_prefill_band > 0) band = g_tune_prefill_band;
     const int nbands = (row_tiles + band - 1) / band;
-    int cseg = nbands >= 8 ? 1 : (8 + nbands - 1) / nbands;  // fewer than 8 bands: cut the columns too
+    // the columns are cut into segments as well, as many as it takes for the number of (band,
+    // segment) units to be a multiple of the 8 XCDs: every XCD then gets the same number of units
+    // (3 bands x 3 segments left one XCD with two units and the others with one: M = 96 took longer
+    // than M = 128)
+    int g8 = nbands & 7;
+    g8 = g8 == 0 ? 8 : (g8 & -g8);  // gcd(nbands, 8)
+    int cseg = 8 / g8;
     cseg = cseg > col_tiles ? col_tiles : cseg;
     const int seg_cols = (col_tiles + cseg - 1) / cseg;
     const int units = nbands * cseg;
     const dim3 grid(8 * ((units + 7) / 8) * band * seg_cols, 1, 1);
+#define BITLINEAR_LAUNCH_PF(MT_, NT_, KS_)                                                                          \
+    hipLaunchKernelGGL((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
+                       act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg)
     if (tile == 4) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<1, 1>), grid, block, 2 * 32 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
+        if (ks == 4) {
+            BITLINEAR_LAUNCH_PF(1, 1, 4);
+        } else if (ks == 2) {
+            BITLINEAR_LAUNCH_PF(1, 1, 2);
+        } else {
+            BITLINEAR_LAUNCH_PF(1, 1, 1);
+        }
     } else if (tile == 1) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<4, 2>), grid, block, 2 * 128 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
+        BITLINEAR_LAUNCH_PF(4, 2, 1);
     } else if (tile == 3) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 4>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
+        BITLINEAR_LAUNCH_PF(2, 4, 1);
     } else if (tile == 2) {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 2>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
+        BITLINEAR_LAUNCH_PF(2, 2, 1);
+    } else if (ks == 2) {
+        BITLINEAR_LAUNCH_PF(2, 1, 2);
     } else {
-        hipLaunchKernelGGL((gemm_i2_prefill_kernel<2, 1>), grid, block, 2 * 64 * kPfRowBytes, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg);
+        BITLINEAR_LAUNCH_PF(2, 1, 1);
     }
+#undef BITLINEAR_LAUNCH_PF
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
@@ -1547,9 +1620,11 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
             const double splitk_us = 3.5 + groups * ((double)N * K / 4.0) / 1.45e6;
             const double tiles = ((N + 127) / 128) * (double)((M + 63) / 64);
             const double tiles32 = ((N + 127) / 128) * (double)((M + 31) / 32);
-            const double gemm_us = tiles <= kPrefillFewTiles
-                                       ? 4.4 + 0.45 * (K / 256.0) * (tiles32 > 400.0 ? tiles32 / 400.0 : 1.0)
-                                       : 4.0 + 0.64 * (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0);
+            const double gemm_us = tiles32 <= kPrefillSplit2Tiles
+                                       ? 5.1 + ((tiles32 <= kPrefillSplit4Tiles && K >= kPrefillSplit4MinK) ? 0.267 : 0.29) * (K / 256.0)
+                                       : (tiles <= kPrefillFewTiles
+                                              ? 4.4 + 0.45 * (K / 256.0) * (tiles32 > 400.0 ? tiles32 / 400.0 : 1.0)
+                                              : 4.0 + 0.64 * (K / 256.0) * (tiles > 256.0 ? tiles / 256.0 : 1.0));
             gemm = gemm_us <= splitk_us;
         }
         if (gemm) return launch_prefill(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
@@ -1650,10 +1725,11 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
-        if (a < 0 || a > 4 || b < 0 || b > 64) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 0 || a > 4 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
         g_tune_path = 5;
         g_tune_prefill_big = a;
         g_tune_prefill_band = b;
+        g_tune_prefill_ks = c;
         return set_status(BITLINEAR_OK);
     }
     return set_status(BITLINEAR_ERR_ARG);

@@ -161,7 +161,9 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *   kernel 5: prefill GEMM (M > 16) with output tile a per workgroup:
  *             0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256, 3 = 64 x 512, 4 = 32 x 128 (tokens
  *             x columns); b = row tiles per band of the tile order (0 = the
- *             library's choice, up to 64)
+ *             library's choice, up to 64); c = groups of four waves that split a
+ *             tile's K between them (0 = the library's choice, 1, 2 (tiles 0 and 4)
+ *             or 4 (tile 4))
  *   kernel 6: product of int8 rows (M <= 16) through the kernel that stages
  *             them in LDS: a = 0 built-in choice (M > 4 and N >= 6912), 1 whenever it
  *             fits, 2 never.  Independent of kernels 1..5; kernel 0 resets it.

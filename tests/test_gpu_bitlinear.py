@@ -387,6 +387,30 @@ def test_prefill_gemm_acc_bit_exact(m, n, k, tile):
     assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
 
 
+@pytest.mark.parametrize("tile,ks", [(4, 2), (4, 4), (0, 2)])
+@pytest.mark.parametrize("m,n,k", [(17, 48, 192), (64, 128, 64), (100, 272, 320), (128, 2560, 2560), (33, 3840, 2560),
+                                   (300, 1040, 3200), (512, 2560, 6912), (70, 256, 768), (40, 512, 1024)])
+def test_prefill_gemm_with_k_split_between_wave_groups(m, n, k, tile, ks):
+    """The small GEMM tiles with 2 or 4 groups of waves splitting a tile's K
+    (chunk counts that do and do not divide by the number of groups, a K of
+    fewer chunks than groups): accumulators bit-exact, and the scaled bf16
+    output equal to the oracle's."""
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=m + n + k + ks)
+    s_bits = o.f32_to_bf16_bits(np.linspace(3.0, 90.0, m).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    _, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    try:
+        assert lib.bitlinear_set_tuning(5, tile, 0, ks) == 0
+        acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+        out = bitlinear.bitnet_int8xint2_linear(dev_i8(a), _packed_dev(w), dev_bf16(s_bits), dev_bf16(ws_bits))
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
+    _assert_bits_equal(host_bits(out), want, f"k-split tile={tile} ks={ks}")
+
+
 def test_prefill_extreme_values_and_split_k_agreement():
     lib = _lib.load_library()
     n, k, m = 256, 6912, 64
