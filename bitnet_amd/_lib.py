@@ -42,6 +42,10 @@ SIGNATURES = {
          _c_int, _c_ptr],
     ),
     "bitnet_attn_decode_workspace_floats": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
+    "bitnet_attn_prefill": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "bitnet_rope_cache_tokens": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],

@@ -13,7 +13,14 @@ import sys
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
-SOURCES = [os.path.join(PKG_DIR, "csrc", "bitlinear_hip.hip"), os.path.join(PKG_DIR, "csrc", "decoder_ops.hip")]
+# source -> extra flags of that translation unit
+SOURCES = {
+    os.path.join(PKG_DIR, "csrc", "bitlinear_hip.hip"): [],
+    os.path.join(PKG_DIR, "csrc", "decoder_ops.hip"): [],
+    # keep the attention kernel's accumulators in the vector register file (see the file's header)
+    os.path.join(PKG_DIR, "csrc", "attn_prefill.hip"): ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+OBJ_DIR = os.path.join(PKG_DIR, "lib", "obj")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libbitlinear_hip.so")
 
@@ -22,7 +29,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-ffp-contract=off",
     # packed fp32 VALU forms are kept out of all device code
@@ -37,18 +43,35 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found; the HIP library cannot be built")
 
 
-def build_library(verbose: bool = True) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", os.path.join(REPO_ROOT, "include"), *SOURCES, "-o", LIB_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
+def _finish(cmd, res, verbose):
     # the host pass warns that it does not know the packed-fp32 feature: harmless
     err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + res.stdout + err)
+        raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + res.stdout + err)
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build_library(verbose: bool = True) -> str:
+    """One object per source (compiled side by side), then one link."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    hipcc = hipcc_path()
+    jobs = []
+    for src, extra in SOURCES.items():
+        obj = os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(src))[0] + ".o")
+        cmd = [hipcc, *HIPCC_FLAGS, *extra, "-I", os.path.join(REPO_ROOT, "include"), "-c", src, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        jobs.append((cmd, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+    objs = []
+    for cmd, obj, proc in jobs:
+        out, err = proc.communicate()
+        _finish(cmd, subprocess.CompletedProcess(cmd, proc.returncode, out, err), verbose)
+        objs.append(obj)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    _finish(cmd, subprocess.run(cmd, capture_output=True, text=True), verbose)
     return LIB_PATH
 
 

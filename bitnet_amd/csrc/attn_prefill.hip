@@ -1,0 +1,307 @@
+// Prompt-side glue of the BitNet decoder's attention block (Attention.forward,
+// gpu/model.py:128-157, where the reference calls xformers' rope_padded and
+// flash attention): rotary embedding + KV-cache write for a block of new
+// tokens, and their causal attention over the cache.  Floating-point kernels,
+// checked against torch fp32 restatements within stated tolerances.
+//
+// This file is compiled with -mllvm -amdgpu-mfma-vgpr-form=1: the attention
+// kernel rescales its output accumulators with vector instructions between
+// matrix instructions, and with the accumulators in the other register file the
+// compiler moves all of them across and back in every step.
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include "bitnet_decoder_ops.h"
+
+namespace {
+
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kHeadDim = 128;
+
+__device__ __forceinline__ float bf16f(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+// fp32 -> bf16, round to nearest even, NaN kept: the same expression as the decode-step kernel's
+__device__ __forceinline__ uint16_t to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {  // round to nearest even, one instruction on gfx950
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// Rotary embedding and cache write for a block of new tokens (a prompt): one workgroup per
+// token.  Items are (head, pair) of the token's q | k | v row; q heads are rotated into q_out,
+// k heads rotated into the cache row of the token's position, v heads copied there.  The same
+// expressions as phase 1 of attn_decode_kernel, so a prompt processed here and a token
+// processed there leave identical cache rows.
+constexpr int kRopeThreads = 256;
+__global__ __launch_bounds__(kRopeThreads) void rope_cache_tokens_kernel(
+    const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
+    const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    uint16_t* __restrict__ q_out, int T, int S, int n_heads, int n_kv_heads) {
+    const int tok = blockIdx.x;  // b * T + t
+    const int b = tok / T;
+    const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
+    const uint16_t* row = qkv + (size_t)tok * row_elems;
+    const int64_t p_raw = positions[tok];
+    const int p = p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw);  // clamped: nothing outside the buffers is touched
+    const size_t cache_off = ((size_t)b * S + p) * n_kv_heads * kHeadDim;
+    const int items = (n_heads + 2 * n_kv_heads) * (kHeadDim / 2);
+    for (int it = threadIdx.x; it < items; it += kRopeThreads) {
+        const int hh = it / (kHeadDim / 2);
+        const int i = it - hh * (kHeadDim / 2);
+        const uint32_t raw = *(const uint32_t*)(row + (size_t)hh * kHeadDim + 2 * i);
+        if (hh < n_heads + n_kv_heads) {
+            const float a = bf16f(raw & 0xffffu), cc = bf16f(raw >> 16);
+            const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
+            const uint32_t rot = (uint32_t)to_bf16(a * cs - cc * sn) | ((uint32_t)to_bf16(a * sn + cc * cs) << 16);
+            if (hh < n_heads)
+                *(uint32_t*)(q_out + ((size_t)tok * n_heads + hh) * kHeadDim + 2 * i) = rot;
+            else
+                *(uint32_t*)(cache_k + cache_off + (size_t)(hh - n_heads) * kHeadDim + 2 * i) = rot;
+        } else {
+            *(uint32_t*)(cache_v + cache_off + (size_t)(hh - n_heads - n_kv_heads) * kHeadDim + 2 * i) = raw;
+        }
+    }
+}
+
+
+// Causal attention of a block of T new tokens per sequence (a prompt) over the cache rows
+// written for them: flash-attention style, scores and output on the bf16 matrix pipe (16x16x32).
+// One wave = 16 consecutive tokens of one query head; the G waves of a workgroup are the G heads
+// that share a kv head, so they walk the same cache rows together: the workgroup brings every
+// block of 32 K and V rows into LDS once (double buffered, requested two steps ahead, one
+// LDS-only barrier per step) and each wave takes its operands from there.
+//   S^T block = K rows (A operand: 16 positions x 32 dims per step) x q^T (B operand: 16 tokens),
+//   so a result lane (c, g4) holds, for token c, positions 4 g4 + j of the block (j = 0..3).  Two
+//   blocks make the 8 positions that this lane contributes, as its k-slots, to the B operand of
+//   O^T += V^T P^T: the probabilities go from the accumulators straight into the next MFMA.
+//   The matching A operand is V transposed: lane (d, g4) loads, for each of those 8 positions, the
+//   16-byte piece d of the V row (dims 8 d .. 8 d + 7); output tile t takes element t of every
+//   piece (one byte-permute per pair of positions), i.e. tile t's row d is dim 8 d + t.  A result
+//   lane (c, g4) then holds, for token c, dims 32 g4 + 8 j + t: eight contiguous dims per j.
+// Online softmax per 32 positions: the running maximum of a token is agreed between its four lanes
+// (c, c + 16, c + 32, c + 48) with two lane permutes; the sums stay per lane until the end.
+// Workgroup barrier that orders LDS traffic only (__syncthreads() would also wait for the global
+// loads in flight).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+constexpr int kApRowBytes = kHeadDim * 2 + 16;  // padded LDS row: the 16 rows of a K operand read spread over all banks
+__device__ __forceinline__ float xor_lane_f32(float v, int lane, int mask) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __float_as_int(v)));
+}
+
+template <int G>
+__global__ __launch_bounds__(64 * G) void attn_prefill_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache_k, const uint16_t* __restrict__ cache_v,
+    uint16_t* __restrict__ out, int T, int S, int start, int n_heads, int n_kv_heads) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g4 = lane >> 4;
+    const int qb = gridDim.x - 1 - blockIdx.x;  // the blocks with the most positions start first
+    const int kvh = blockIdx.y, b = blockIdx.z;
+    const int head = kvh * G + wave;
+    const int t0 = qb * 16;
+    const int tq = (t0 + c) < T ? (t0 + c) : (T - 1);
+    const int pq = start + t0 + c;  // position of this lane's token: cache rows 0..pq are visible to it
+    const int n_pos = start + ((t0 + 16) < T ? (t0 + 16) : T);  // rows [0, n_pos) matter to this block
+    const int steps = (n_pos + 31) >> 5;
+
+    // q^T as the B operand of the four 32-dim steps
+    v8bf qa[4];
+    {
+        const uint16_t* qrow = q + (((size_t)b * T + tq) * n_heads + head) * kHeadDim;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) qa[kk] = __builtin_bit_cast(v8bf, *(const uint4*)(qrow + kk * 32 + g4 * 8));
+    }
+    // cache rows through descriptors that end behind row n_pos - 1: requests beyond read as zero
+    // at no cost, so neither the last step nor the prefetch past it needs a clamped index, and no
+    // stale row behind the prompt can put a NaN into the products
+    const int row_bytes = n_kv_heads * kHeadDim * 2;
+    const int span_bytes = (n_pos - 1) * row_bytes + kHeadDim * 2;
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(cache_k + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim), 0, span_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(cache_v + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim), 0, span_bytes, 0x00020000);
+    // staging map: piece p = tid + i * NT is the 16-byte piece p % 16 of row p / 16 of a 32-row block
+    constexpr int NT = 64 * G;
+    constexpr int PPT = 512 / NT;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_kv[2][2][32 * kApRowBytes];  // [buffer][K | V]
+    const int tid = threadIdx.x;
+    int g_off[PPT], l_off[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        const int pce = tid + i * NT;
+        g_off[i] = (pce >> 4) * row_bytes + (pce & 15) * 16;
+        l_off[i] = (pce >> 4) * kApRowBytes + (pce & 15) * 16;
+    }
+    v4u kst[PPT], vst[PPT];
+    // the whole offset goes into the per-lane operand: that is the one the range check looks at
+    auto request = [&](int st) {
+        const int base = st * 32 * row_bytes;
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+            kst[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, base + g_off[i], 0, 0);
+            vst[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, base + g_off[i], 0, 0);
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PPT; ++i) {
+            *(v4u*)(&lds_kv[buf][0][l_off[i]]) = kst[i];
+            *(v4u*)(&lds_kv[buf][1][l_off[i]]) = vst[i];
+        }
+    };
+    const int k_lds_off = c * kApRowBytes + g4 * 16;        // K operand: row c of a 16-row block, piece g4 of a 64-byte step
+    const int v_lds_off = 4 * g4 * kApRowBytes + c * 16;    // V: rows 4 g4 + jj (and 16 + 4 g4 + jj), piece c
+
+    v4f o_acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) o_acc[t] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    // softmax in base 2: exp(x * scale - m) = exp2(x * c2 - m2) with c2 = scale * log2(e); the running
+    // maximum m_run is kept in raw score units (the scale is positive, so maxima commute with it)
+    float m_run = -INFINITY, l_run = 0.0f;
+    const float c2 = 0.08838834764831845f * 1.4426950408889634f;  // 128^-0.5 * log2(e)
+
+    auto step = [&](int st) {
+        const uint8_t* kl = &lds_kv[st & 1][0][k_lds_off];
+        const uint8_t* vl = &lds_kv[st & 1][1][v_lds_off];
+        v4u kb[2][4], vb[8];
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) kb[bi][kk] = *(const v4u*)(kl + bi * 16 * kApRowBytes + kk * 64);
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) vb[jj] = *(const v4u*)(vl + ((jj & 3) + (jj >> 2) * 16) * kApRowBytes);
+        float sc[8];
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+            v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kb[bi][kk]), qa[kk], acc, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sc[bi * 4 + j] = acc[j];
+        }
+        // only the steps that reach beyond the block's first token need the causal mask (uniform test)
+        if (st * 32 + 31 > start + t0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int pos = st * 32 + (i >> 2) * 16 + 4 * g4 + (i & 3);
+                sc[i] = pos <= pq ? sc[i] : -INFINITY;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mx = fmaxf(mx, xor_lane_f32(mx, lane, 16));
+        mx = fmaxf(mx, xor_lane_f32(mx, lane, 32));
+        const float m_new = fmaxf(m_run, mx);  // finite from the first step on: position 0 is visible to every token
+        const float m2 = m_new * c2;
+        float p[8], psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c2, -m2));
+            psum += p[i];
+        }
+        // the accumulated outputs are rescaled only when some token's maximum has moved (uniform test):
+        // after the first few steps it rarely does
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f(__builtin_fmaf(m_run, c2, -m2));
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o_acc[t][j] *= alpha;
+            m_run = m_new;
+        }
+        l_run += psum;
+        v4u pw;
+        pw.x = pack_bf16x2(p[0], p[1]);
+        pw.y = pack_bf16x2(p[2], p[3]);
+        pw.z = pack_bf16x2(p[4], p[5]);
+        pw.w = pack_bf16x2(p[6], p[7]);
+        const v8bf pb = __builtin_bit_cast(v8bf, pw);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;  // both high halves / both low halves
+            v4u va;
+            va.x = __builtin_amdgcn_perm(vb[1][t >> 1], vb[0][t >> 1], sel);
+            va.y = __builtin_amdgcn_perm(vb[3][t >> 1], vb[2][t >> 1], sel);
+            va.z = __builtin_amdgcn_perm(vb[5][t >> 1], vb[4][t >> 1], sel);
+            va.w = __builtin_amdgcn_perm(vb[7][t >> 1], vb[6][t >> 1], sel);
+            o_acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, va), pb, o_acc[t], 0, 0, 0);
+        }
+    };
+
+    request(0);
+    stage(0);
+    request(1);
+    lds_barrier();
+    for (int st = 0; st < steps; ++st) {
+        step(st);
+        stage((st + 1) & 1);  // rows of step st + 1, requested a step ago, into the buffer that step st - 1 used
+        request(st + 2);
+        lds_barrier();
+    }
+
+    float l_tot = l_run + xor_lane_f32(l_run, lane, 16);
+    l_tot += xor_lane_f32(l_tot, lane, 32);
+    const float inv = 1.0f / l_tot;
+    if (t0 + c < T) {
+        uint16_t* orow = out + ((size_t)b * T + t0 + c) * n_heads * kHeadDim + (size_t)head * kHeadDim + 32 * g4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v4u w;
+            w.x = pack_bf16x2(o_acc[0][j] * inv, o_acc[1][j] * inv);
+            w.y = pack_bf16x2(o_acc[2][j] * inv, o_acc[3][j] * inv);
+            w.z = pack_bf16x2(o_acc[4][j] * inv, o_acc[5][j] * inv);
+            w.w = pack_bf16x2(o_acc[6][j] * inv, o_acc[7][j] * inv);
+            *(v4u*)(orow + 8 * j) = w;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int bitnet_rope_cache_tokens(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
+                                        const float* cos_table, const float* sin_table, uint16_t* q_out, int B, int T,
+                                        int S, int n_heads, int n_kv_heads, int head_dim, void* stream) {
+    if (B < 1 || T < 1 || S < 1 || n_heads < 1 || n_kv_heads < 1 || head_dim != kHeadDim) return 1;
+    if ((long long)B * T >= (1ll << 31)) return 1;
+    if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !q_out) return 2;
+    hipLaunchKernelGGL(rope_cache_tokens_kernel, dim3(B * T, 1, 1), dim3(kRopeThreads, 1, 1), 0, (hipStream_t)stream, qkv,
+                       cache_k, cache_v, positions, cos_table, sin_table, q_out, T, S, n_heads, n_kv_heads);
+    return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int bitnet_attn_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v, uint16_t* out, int B,
+                                   int T, int S, int start, int n_heads, int n_kv_heads, int head_dim, void* stream) {
+    if (B < 1 || T < 1 || S < 1 || start < 0 || n_heads < 1 || n_kv_heads < 1 || head_dim != kHeadDim) return 1;
+    if ((long long)start + T > S || n_heads % n_kv_heads) return 1;
+    const int g = n_heads / n_kv_heads;
+    if (g != 1 && g != 2 && g != 4 && g != 8) return 1;
+    if ((size_t)(S + 64) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;  // 32-bit byte offsets into one sequence's cache
+    if (B > 65535 || n_kv_heads > 65535) return 1;
+    if (!q || !cache_k || !cache_v || !out) return 2;
+    if ((((uintptr_t)q) | ((uintptr_t)cache_k) | ((uintptr_t)cache_v) | ((uintptr_t)out)) & 15u) return 1;
+    const dim3 grid((T + 15) / 16, n_kv_heads, B), block(64 * g, 1, 1);
+    switch (g) {
+        case 1: hipLaunchKernelGGL(attn_prefill_kernel<1>, grid, block, 0, (hipStream_t)stream, q, cache_k, cache_v, out, T, S, start, n_heads, n_kv_heads); break;
+        case 2: hipLaunchKernelGGL(attn_prefill_kernel<2>, grid, block, 0, (hipStream_t)stream, q, cache_k, cache_v, out, T, S, start, n_heads, n_kv_heads); break;
+        case 4: hipLaunchKernelGGL(attn_prefill_kernel<4>, grid, block, 0, (hipStream_t)stream, q, cache_k, cache_v, out, T, S, start, n_heads, n_kv_heads); break;
+        default: hipLaunchKernelGGL(attn_prefill_kernel<8>, grid, block, 0, (hipStream_t)stream, q, cache_k, cache_v, out, T, S, start, n_heads, n_kv_heads); break;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+

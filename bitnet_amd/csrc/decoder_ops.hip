@@ -748,42 +748,6 @@ __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const fl
 }
 
 
-// Rotary embedding and cache write for a block of new tokens (a prompt): one workgroup per
-// token.  Items are (head, pair) of the token's q | k | v row; q heads are rotated into q_out,
-// k heads rotated into the cache row of the token's position, v heads copied there.  The same
-// expressions as phase 1 of attn_decode_kernel, so a prompt processed here and a token
-// processed there leave identical cache rows.
-constexpr int kRopeThreads = 256;
-__global__ __launch_bounds__(kRopeThreads) void rope_cache_tokens_kernel(
-    const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
-    const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    uint16_t* __restrict__ q_out, int T, int S, int n_heads, int n_kv_heads) {
-    const int tok = blockIdx.x;  // b * T + t
-    const int b = tok / T;
-    const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
-    const uint16_t* row = qkv + (size_t)tok * row_elems;
-    const int64_t p_raw = positions[tok];
-    const int p = p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw);  // clamped: nothing outside the buffers is touched
-    const size_t cache_off = ((size_t)b * S + p) * n_kv_heads * kHeadDim;
-    const int items = (n_heads + 2 * n_kv_heads) * (kHeadDim / 2);
-    for (int it = threadIdx.x; it < items; it += kRopeThreads) {
-        const int hh = it / (kHeadDim / 2);
-        const int i = it - hh * (kHeadDim / 2);
-        const uint32_t raw = *(const uint32_t*)(row + (size_t)hh * kHeadDim + 2 * i);
-        if (hh < n_heads + n_kv_heads) {
-            const float a = bf16f(raw & 0xffffu), cc = bf16f(raw >> 16);
-            const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
-            const uint32_t rot = (uint32_t)to_bf16(a * cs - cc * sn) | ((uint32_t)to_bf16(a * sn + cc * cs) << 16);
-            if (hh < n_heads)
-                *(uint32_t*)(q_out + ((size_t)tok * n_heads + hh) * kHeadDim + 2 * i) = rot;
-            else
-                *(uint32_t*)(cache_k + cache_off + (size_t)(hh - n_heads) * kHeadDim + 2 * i) = rot;
-        } else {
-            *(uint32_t*)(cache_v + cache_off + (size_t)(hh - n_heads - n_kv_heads) * kHeadDim + 2 * i) = raw;
-        }
-    }
-}
-
 }  // namespace
 
 static int g_attn_threads = 0;
@@ -840,17 +804,6 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
         default: BITNET_ATTN_LAUNCH(8) break;
     }
 #undef BITNET_ATTN_LAUNCH
-    return hipGetLastError() == hipSuccess ? 0 : 3;
-}
-
-extern "C" int bitnet_rope_cache_tokens(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
-                                        const float* cos_table, const float* sin_table, uint16_t* q_out, int B, int T,
-                                        int S, int n_heads, int n_kv_heads, int head_dim, void* stream) {
-    if (B < 1 || T < 1 || S < 1 || n_heads < 1 || n_kv_heads < 1 || head_dim != kHeadDim) return 1;
-    if ((long long)B * T >= (1ll << 31)) return 1;
-    if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !q_out) return 2;
-    hipLaunchKernelGGL(rope_cache_tokens_kernel, dim3(B * T, 1, 1), dim3(kRopeThreads, 1, 1), 0, (hipStream_t)stream, qkv,
-                       cache_k, cache_v, positions, cos_table, sin_table, q_out, T, S, n_heads, n_kv_heads);
     return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

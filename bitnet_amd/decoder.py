@@ -116,6 +116,20 @@ def rope_cache_tokens(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv
     return q
 
 
+def attn_prefill(q, cache_k, cache_v, start: int = 0):
+    """Causal grouped-query attention of T new tokens per sequence over cache
+    rows 0 .. start + t in one HIP kernel (bitnet_attn_prefill).  q bf16
+    [B, T, n_heads, 128] (rotated); returns bf16 [B * T, n_heads * 128]."""
+    B, T, n_heads, hd = q.shape
+    S, n_kv = cache_k.shape[1], cache_k.shape[2]
+    out = torch.empty(B * T, n_heads * hd, dtype=torch.bfloat16, device=q.device)
+    st = _lib.load_library().bitnet_attn_prefill(
+        _ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(out), B, T, S, start, n_heads, n_kv, hd, _stream_ptr())
+    if st != 0:
+        raise _lib.BitLinearLibraryError(f"bitnet_attn_prefill: status {st}")
+    return out
+
+
 class LmHeadWorkspace:
     """Scratch of bitnet_lm_head_greedy for one (batch, vocabulary, dim)."""
 
@@ -282,21 +296,18 @@ class Transformer(nn.Module):
         the layer stack of decode_hidden_fused at prompt size (norms, gate and
         residual adds folded into the BitLinear calls, which run the int8 GEMM),
         rope + cache write in one kernel, causal attention over the new tokens
-        by torch's scaled_dot_product_attention (the reference calls xformers'
-        flash attention here, gpu/model.py:147-155).  Returns the hidden state in
-        front of the final norm, [B, T, dim]."""
+        in another (the reference calls xformers' rope_padded and flash attention
+        here, gpu/model.py:128-155).  Returns the hidden state in front of the
+        final norm, [B, T, dim]."""
         a = self.args
         B, T = tokens.shape
-        hd = a.dim // a.n_heads
         pos = torch.arange(T, device=tokens.device)[None, :].expand(B, T).contiguous()
         h = self.tok_embeddings(tokens.reshape(B * T))
         for layer, (ck, cv) in zip(self.layers, cache):
             att, ffn = layer.attention, layer.feed_forward
             xqkv = norm_bitlinear(h, layer.attention_norm, att.wqkv)
             q = rope_cache_tokens(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads)
-            o = torch.nn.functional.scaled_dot_product_attention(
-                q.transpose(1, 2), ck[:, :T].transpose(1, 2), cv[:, :T].transpose(1, 2), is_causal=True, enable_gqa=True)
-            o = o.transpose(1, 2).reshape(B * T, a.n_heads * hd)
+            o = attn_prefill(q, ck, cv, 0)
             h = norm_bitlinear(o, att.attn_sub_norm, att.wo, residual=h)
             x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
             h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)

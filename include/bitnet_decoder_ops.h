@@ -62,6 +62,24 @@ int bitnet_rope_cache_tokens(const uint16_t* qkv, uint16_t* cache_k, uint16_t* c
                              const float* sin_table, uint16_t* q_out, int B, int T, int S,
                              int n_heads, int n_kv_heads, int head_dim, void* stream);
 
+/*
+ * Causal grouped-query attention of a block of T new tokens per sequence over the cache rows
+ * 0 .. start + t (the prompt pass of Attention.forward, gpu/model.py:147-155, where the reference
+ * calls xformers' flash attention): token t of sequence b sits at position start + t, its rotated
+ * q in q[b, t, h, :] and the k / v of positions 0 .. start + T - 1 already in the cache (written by
+ * bitnet_rope_cache_tokens, and by earlier calls for positions below start):
+ *   out[b * T + t, h, :] = softmax(q . K[0 .. start + t] / sqrt(head_dim)) V[0 .. start + t]
+ *   q bf16 [B, T, n_heads, head_dim]; cache_k/v bf16 [B, S, n_kv_heads, head_dim];
+ *   out bf16 [B * T, n_heads * head_dim]; start >= 0, start + T <= S.
+ * Scores and outputs on the bf16 matrix pipe with fp32 accumulation, probabilities rounded to
+ * bf16 in between; an online softmax over steps of 32 positions.  head_dim must be 128,
+ * n_heads / n_kv_heads one of 1, 2, 4, 8, all pointers 16-byte aligned.
+ * Returns 0, 1 (shape / alignment), 2 (null pointer), 3 (launch failed).
+ */
+int bitnet_attn_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16_t* cache_v,
+                        uint16_t* out, int B, int T, int S, int start, int n_heads,
+                        int n_kv_heads, int head_dim, void* stream);
+
 /* Tuning override for tests and measurements: threads per workgroup of the attention kernel
  * (256 or 512; 0 restores the built-in choice).  Results do not depend on it beyond the
  * order of fp32 additions.  Returns 0, or 1 for another value. */

@@ -284,8 +284,8 @@ def test_rope_cache_tokens_kernel_equals_torch(B, T, S, nh, nkv, start):
 
 def test_prompt_through_the_library_kernels_against_the_torch_glue():
     """Generator.prefill with the prompt-sized layer stack (norm / gate /
-    residual folded into the BitLinear calls, rope + cache kernel, torch's
-    fused attention) against forward_tokens (every op in torch around the same
+    residual folded into the BitLinear calls, rope + cache kernel, the prompt
+    attention kernel) against forward_tokens (every op in torch around the same
     BitLinear kernels, fp32 attention): the first layer's cache rows and the
     last token's logits within bf16 noise (the norm's and the attention's sums
     run in another order and precision), and each path's first token equal to
@@ -312,3 +312,32 @@ def test_prompt_through_the_library_kernels_against_the_torch_glue():
     assert torch.equal(first, torch.argmax(logits1, dim=-1))
     gen2 = decoder.Generator(model, B, S, fused_head=False)
     assert torch.equal(gen2.prefill(prompt), torch.argmax(logits2[:, -1], dim=-1))
+
+
+@pytest.mark.parametrize("B,T,S,nh,nkv,start", [(1, 512, 640, 20, 5, 0), (2, 70, 96, 4, 1, 0), (3, 33, 80, 8, 8, 40),
+                                               (1, 1, 16, 16, 2, 9), (2, 200, 256, 8, 4, 17), (1, 16, 16, 2, 2, 0)])
+def test_attention_prefill_kernel_against_torch_fp32(B, T, S, nh, nkv, start):
+    """Floating-point kernel: compared with the fp32 torch restatement
+    softmax(QK^T/sqrt(d))V over cache rows 0..start+t.  The kernel rounds the
+    probabilities to bf16 for the matrix pipe (relative error 2^-9 each), so
+    the tolerance is 3 bf16 ulp or 4e-3 absolute on the bf16 outputs.  Cache
+    rows behind the last position hold NaNs: they must not be touched."""
+    hd = 128
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(B * 1000 + T + start)
+    q = torch.randn(B, T, nh, hd, generator=g, device=dev).to(torch.bfloat16)
+    ck = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    cv = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    ck[:, start + T:] = float("nan")
+    cv[:, start + T:] = float("nan")
+    att = decoder.Attention.__new__(decoder.Attention)
+    torch.nn.Module.__init__(att)
+    att.head_dim, att.n_heads, att.n_kv_heads = hd, nh, nkv
+    pos = start + torch.arange(T, device=dev)
+    mask = (torch.arange(start + T, device=dev)[None, None, :] <= pos[None, :, None]).expand(B, T, start + T)
+    want = att.attend(q, ck[:, :start + T], cv[:, :start + T], mask).reshape(B * T, nh * hd)
+    got = decoder.attn_prefill(q, ck, cv, start)
+    torch.cuda.synchronize()
+    assert not torch.isnan(got.float()).any()
+    bad = (_ulp(got, want) > 3) & ((got.float() - want.float()).abs() > 4e-3)
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance, max abs {float((got.float() - want.float()).abs().max())}"
