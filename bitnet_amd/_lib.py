@@ -51,6 +51,7 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
     "bitnet_attn_decode_set_threads": (_c_int, [_c_int]),
+    "bitnet_attn_decode_set_kernel": (_c_int, [_c_int]),
     "bitnet_lm_head_greedy": (
         _c_int,
         [_c_ptr, _c_ptr, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],

@@ -272,7 +272,303 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// Decode step (one new token per sequence) with the same matrix-pipe scheme
+// ---------------------------------------------------------------------------
+// One workgroup per (kv head, sequence, split of the cached positions), as attn_decode_kernel; the
+// difference is what happens between the rope and the records: every wave takes 32 positions of
+// the slice at a time and does scores, softmax and P.V for the G query heads (columns c < G of the
+// 16-column tiles) entirely in registers; the waves' (maximum, sum, outputs) are combined through
+// LDS once.  No score buffer, no barrier between scores, softmax and P.V.
+constexpr int kDfRecFloats = kHeadDim + 2;  // record of one (sequence, kv head, split, head): 128 outputs, maximum, sum
+constexpr int kDfMaxSplits = 16;
+constexpr int kDfMaxWaves = 8;
+
+template <int G>
+__global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
+    const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
+    const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    uint16_t* __restrict__ out, float* workspace, int* counters, int S, int span, int n_heads, int n_kv_heads) {
+    __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
+    __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
+    __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
+    __shared__ __attribute__((aligned(16))) float part_o[kDfMaxWaves][G][kHeadDim];
+    __shared__ float part_m[kDfMaxWaves][G], part_l[kDfMaxWaves][G];
+    __shared__ int is_last;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nthreads = blockDim.x;
+    const int nwaves = nthreads >> 6;
+    const int kvh = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
+    const int nsplit = gridDim.z;
+    const int c = lane & 15, g4 = lane >> 4;
+    const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
+    const uint16_t* row = qkv + (size_t)b * row_elems;
+    const size_t cache_row = (size_t)n_kv_heads * kHeadDim;
+    uint16_t* ck = cache_k + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
+    uint16_t* cv = cache_v + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
+    const int row_bytes = n_kv_heads * kHeadDim * 2;
+    const int cache_bytes = (S - 1) * row_bytes + kHeadDim * 2;
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)ck, 0, cache_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cv, 0, cache_bytes, 0x00020000);
+    const int lo = sp * span;  // this split owns positions [lo, lo + span), span % 16 == 0
+    constexpr int kPastEnd = 0x7fff0000;
+
+    // Everything that depends on nothing is requested first: the token's q / k / v, the position,
+    // and the wave's first 32 K and V rows of the slice (rows outside the slice get an offset past
+    // the end of the descriptor, which costs no memory access).
+    constexpr int kItems = (G + 2) * (kHeadDim / 2);
+    constexpr int kIters = (kItems + 255) / 256;
+    uint32_t praw[kIters];
+#pragma unroll
+    for (int u = 0; u < kIters; ++u) {
+        const int it = tid + u * nthreads;
+        const int hh = it / (kHeadDim / 2);
+        const int i = it - hh * (kHeadDim / 2);
+        const int src = hh < G ? (kvh * G + hh) * kHeadDim : (hh == G ? (n_heads + kvh) : (n_heads + n_kv_heads + kvh)) * kHeadDim;
+        praw[u] = *(const uint32_t*)(row + (it < kItems ? src + 2 * i : 0));
+    }
+    v4u kb[2][4], vb[8];
+    auto load_rows = [&](int r0) {  // rows r0 .. r0 + 31 of the slice
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+            const int rel = r0 + bi * 16 + c;
+            const int off = rel < span ? (lo + rel) * row_bytes + g4 * 16 : kPastEnd;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) kb[bi][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
+        }
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+            const int rel = r0 + (jj & 3) + (jj >> 2) * 16 + 4 * g4;
+            vb[jj] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, rel < span ? (lo + rel) * row_bytes + c * 16 : kPastEnd, 0, 0);
+        }
+    };
+    load_rows(wave * 32);
+    const int64_t p_raw = positions[b];
+    const int p = __builtin_amdgcn_readfirstlane(p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw));  // clamped into the cache
+    const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's visible positions are [lo, hi)
+    const bool owns_new = p >= lo && p < lo + span;
+    int nact = 1;  // splits whose slice starts at or below the position
+#pragma unroll
+    for (int k = 1; k < kDfMaxSplits; ++k) nact += (k < nsplit && p >= k * span) ? 1 : 0;
+    const bool active = sp < nact;
+
+    // rope on adjacent pairs, fp32, rounded to bf16: q into LDS; the split that holds position p also
+    // rotates k, keeps k and v of the new token in LDS and writes them to the cache
+#pragma unroll
+    for (int u = 0; u < kIters; ++u) {
+        const int it = tid + u * nthreads;
+        const int hh = it / (kHeadDim / 2);
+        const int i = it - hh * (kHeadDim / 2);
+        if (it < kItems && active) {
+            if (hh <= G) {
+                if (hh < G || owns_new) {
+                    const float a = bf16f(praw[u] & 0xffffu), cc = bf16f(praw[u] >> 16);
+                    const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
+                    const uint32_t rot = (uint32_t)to_bf16(a * cs - cc * sn) | ((uint32_t)to_bf16(a * sn + cc * cs) << 16);
+                    if (hh < G) {
+                        *(uint32_t*)(&qb[hh][2 * i]) = rot;
+                    } else {
+                        *(uint32_t*)(&knew[2 * i]) = rot;
+                        *(uint32_t*)(ck + (size_t)p * cache_row + 2 * i) = rot;
+                    }
+                }
+            } else if (owns_new) {
+                *(uint32_t*)(&vnew[2 * i]) = praw[u];
+                *(uint32_t*)(cv + (size_t)p * cache_row + 2 * i) = praw[u];
+            }
+        }
+    }
+    __syncthreads();
+    if (!active) return;  // after the barrier: a branch on the position in front of the loads above would delay them
+
+    // q^T as the B operand: column c = head c (zero beyond G)
+    v8bf qa[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        uint4 t = make_uint4(0, 0, 0, 0);
+        if (c < G) t = *(const uint4*)(&qb[c][kk * 32 + g4 * 8]);
+        qa[kk] = __builtin_bit_cast(v8bf, t);
+    }
+    v4f o_acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) o_acc[t] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY, l_run = 0.0f;
+    const float scale = 0.08838834764831845f;           // 128^-0.5
+    const float c2 = scale * 1.4426950408889634f;        // * log2(e): the softmax runs in base 2
+    for (int r0 = wave * 32; lo + r0 < hi; r0 += nwaves * 32) {
+        if (r0 != wave * 32) load_rows(r0);
+        // the new token's own row is not in the cache yet for this kernel's loads: it comes from LDS
+        if (owns_new && p - lo >= r0 && p - lo < r0 + 32) {
+#pragma unroll
+            for (int bi = 0; bi < 2; ++bi)
+                if (lo + r0 + bi * 16 + c == p) {
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk) kb[bi][kk] = *(const v4u*)(&knew[kk * 32 + g4 * 8]);
+                }
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj)
+                if (lo + r0 + (jj & 3) + (jj >> 2) * 16 + 4 * g4 == p) vb[jj] = *(const v4u*)(&vnew[c * 8]);
+        }
+        float sc[8];
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+            v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kb[bi][kk]), qa[kk], acc, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int pos = lo + r0 + bi * 16 + 4 * g4 + j;
+                sc[bi * 4 + j] = pos < hi ? acc[j] : -INFINITY;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mx = fmaxf(mx, xor_lane_f32(mx, lane, 16));
+        mx = fmaxf(mx, xor_lane_f32(mx, lane, 32));
+        const float m_new = fmaxf(m_run, mx);  // finite: the step holds at least position lo + r0 < hi
+        const float m2 = m_new * c2;
+        float pr[8], psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pr[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c2, -m2));
+            psum += pr[i];
+        }
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f(__builtin_fmaf(m_run, c2, -m2));
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o_acc[t][j] *= alpha;
+            m_run = m_new;
+        }
+        l_run += psum;
+        v4u pw;
+        pw.x = pack_bf16x2(pr[0], pr[1]);
+        pw.y = pack_bf16x2(pr[2], pr[3]);
+        pw.z = pack_bf16x2(pr[4], pr[5]);
+        pw.w = pack_bf16x2(pr[6], pr[7]);
+        const v8bf pb = __builtin_bit_cast(v8bf, pw);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+            v4u va;
+            va.x = __builtin_amdgcn_perm(vb[1][t >> 1], vb[0][t >> 1], sel);
+            va.y = __builtin_amdgcn_perm(vb[3][t >> 1], vb[2][t >> 1], sel);
+            va.z = __builtin_amdgcn_perm(vb[5][t >> 1], vb[4][t >> 1], sel);
+            va.w = __builtin_amdgcn_perm(vb[7][t >> 1], vb[6][t >> 1], sel);
+            o_acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, va), pb, o_acc[t], 0, 0, 0);
+        }
+    }
+    // the wave's result for head c (lanes c < G): maximum, sum over its positions, 32 outputs per lane
+    float l_tot = l_run + xor_lane_f32(l_run, lane, 16);
+    l_tot += xor_lane_f32(l_tot, lane, 32);
+    if (c < G) {
+        if (g4 == 0) {
+            part_m[wave][c] = m_run;  // -inf, and a sum of 0, for a wave without visible positions
+            part_l[wave][c] = l_tot;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) part_o[wave][c][32 * g4 + 8 * j + t] = o_acc[t][j];
+    }
+    __syncthreads();
+
+    uint16_t* orow = out + (size_t)b * n_heads * kHeadDim + (size_t)(kvh * G) * kHeadDim;
+    float* rec = workspace + ((size_t)(b * n_kv_heads + kvh) * nsplit) * G * kDfRecFloats;
+    for (int hh = wave; hh < G; hh += nwaves) {
+        float mx = -INFINITY;
+        for (int k = 0; k < nwaves; ++k) mx = fmaxf(mx, part_m[k][hh]);
+        float o0 = 0.0f, o1 = 0.0f, l = 0.0f;
+        for (int k = 0; k < nwaves; ++k) {
+            const float lk = part_l[k][hh];
+            if (lk > 0.0f) {
+                const float w = __builtin_amdgcn_exp2f((part_m[k][hh] - mx) * c2);
+                l += lk * w;
+                o0 += w * part_o[k][hh][2 * lane];
+                o1 += w * part_o[k][hh][2 * lane + 1];
+            }
+        }
+        if (nact == 1) {
+            const float is = 1.0f / l;
+            *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
+        } else {
+            // device-coherent (write-through) stores: the record reaches the point where the other
+            // XCDs' loads see it without a writeback of this XCD's whole L2
+            float* r = rec + ((size_t)sp * G + hh) * kDfRecFloats;
+            __hip_atomic_store(r + 2 * lane, o0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(r + 2 * lane + 1, o1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) {
+                __hip_atomic_store(r + kHeadDim, mx * scale, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // in units of the scaled scores
+                __hip_atomic_store(r + kHeadDim + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    if (nact == 1) return;
+
+    // The last split of this (sequence, kv head) to finish combines the records: the barrier waits
+    // until every thread's record stores have completed (write-through: completed = visible
+    // device-wide); then the arrival is counted with a device-scope atomic, and the last arrival
+    // reads the records with device-coherent loads.
+    __syncthreads();
+    if (tid == 0) {
+        const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = done == nact - 1;
+        if (is_last) __hip_atomic_store(&counters[b * n_kv_heads + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    for (int hh = wave; hh < G; hh += nwaves) {
+        float mk[kDfMaxSplits], lk[kDfMaxSplits], p0[kDfMaxSplits], p1[kDfMaxSplits];
+#pragma unroll
+        for (int k = 0; k < kDfMaxSplits; ++k) {
+            const float* r = rec + ((size_t)(k < nact ? k : 0) * G + hh) * kDfRecFloats;
+            mk[k] = __hip_atomic_load(r + kHeadDim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lk[k] = __hip_atomic_load(r + kHeadDim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            p0[k] = __hip_atomic_load(r + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            p1[k] = __hip_atomic_load(r + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < kDfMaxSplits; ++k)
+            if (k < nact) mx = fmaxf(mx, mk[k]);
+        float l = 0.0f, o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kDfMaxSplits; ++k) {
+            if (k < nact && lk[k] > 0.0f) {
+                const float w = __expf(mk[k] - mx);
+                l += lk[k] * w;
+                o0 += w * p0[k];
+                o1 += w * p1[k];
+            }
+        }
+        const float is = 1.0f / l;
+        *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
+    }
+}
+
 }  // namespace
+
+// Launcher used by bitnet_attn_decode (decoder_ops.hip), which has validated the arguments.
+int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
+                                    const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
+                                    int* counters, int n_splits, int span, int threads, int B, int S, int n_heads,
+                                    int n_kv_heads, hipStream_t stream) {
+    const int g = n_heads / n_kv_heads;
+    const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
+    switch (g) {
+        case 1: hipLaunchKernelGGL(attn_decode_flash_kernel<1>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
+        case 2: hipLaunchKernelGGL(attn_decode_flash_kernel<2>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
+        case 4: hipLaunchKernelGGL(attn_decode_flash_kernel<4>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
+        default: hipLaunchKernelGGL(attn_decode_flash_kernel<8>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 3;
+}
 
 extern "C" int bitnet_rope_cache_tokens(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
                                         const float* cos_table, const float* sin_table, uint16_t* q_out, int B, int T,

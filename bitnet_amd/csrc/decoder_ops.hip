@@ -751,6 +751,20 @@ __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const fl
 }  // namespace
 
 static int g_attn_threads = 0;
+static int g_attn_kernel = 0;  // 0 = built-in choice, 1 = score buffer in LDS + vector-pipe P.V, 2 = everything on the matrix pipe
+
+// in attn_prefill.hip
+int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
+                                    const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
+                                    int* counters, int n_splits, int span, int threads, int B, int S, int n_heads,
+                                    int n_kv_heads, hipStream_t stream);
+
+/* tuning override for tests and measurements: which of the two decode-step attention kernels runs */
+extern "C" int bitnet_attn_decode_set_kernel(int which) {
+    if (which < 0 || which > 2) return 1;
+    g_attn_kernel = which;
+    return 0;
+}
 
 /* tuning override: threads per workgroup of the attention kernel (0 = built-in choice) */
 extern "C" int bitnet_attn_decode_set_threads(int threads) {
@@ -772,7 +786,8 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     if (n_heads % n_kv_heads) return 1;
     const int g = n_heads / n_kv_heads;
     if (g != 1 && g != 2 && g != 4 && g != 8) return 1;
-    if (n_splits < 1 || n_splits > kMaxSplits) return 1;
+    const bool flash = g_attn_kernel != 1;  // the built-in choice is the matrix-pipe kernel
+    if (n_splits < 1 || n_splits > (flash ? 16 : kMaxSplits)) return 1;
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
     if (n_splits > 1 && (!workspace || !counters)) return 2;
     if ((size_t)(S + 512) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;  // the kernel's 32-bit byte offsets into one sequence's cache
@@ -782,7 +797,13 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     // workgroup has a CU of its own (up to 256 of them); beyond that two 512-thread workgroups
     // share a CU badly (12.9 -> 16.8 us at 320 workgroups) and 256 threads are the better choice.
     int threads = (span > 64 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
+    // the matrix-pipe kernel: a wave takes 32 rows per round, so four waves cover a slice of up to 128 rows
+    // in one round (measured at 96 rows: 6.85 us with four waves, 7.12 with eight; at 272 rows 8.77 / 8.46)
+    if (flash) threads = (span > 128 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
     if (g_attn_threads) threads = g_attn_threads;
+    if (flash)
+        return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters,
+                                               n_splits, span, threads, B, S, n_heads, n_kv_heads, (hipStream_t)stream);
     const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * 1024) * sizeof(float);  // scores + one 4 KB region per wave
     if (lds > 96u * 1024u) return 1;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);

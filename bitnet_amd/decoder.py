@@ -383,11 +383,11 @@ class Generator:
         self.model = model
         self.fused = fused and model.fused_decode_ok(batch)
         a_ = model.args
-        # split the cached positions of every (sequence, kv head) over up to 8 workgroups: one CU alone
-        # pulls a small fraction of the memory bandwidth, and merging the splits costs about a microsecond.
-        # No more workgroups than CUs (256): with a CU of its own a workgroup runs eight waves and takes
-        # its slice in one round of loads (measured: batch 8, 641 rows: 6 splits 11.5 us, 8 splits 12.9 us)
-        n_splits = max(1, min(8, 256 // max(1, batch * a_.n_kv_heads)))
+        # split the cached positions of every (sequence, kv head) over up to 8 workgroups (16 for caches
+        # beyond 2048 rows: measured 16.5 -> 12.3 us at 8200 rows, nothing at 642): one CU alone pulls a
+        # small fraction of the memory bandwidth, and merging the splits costs about a microsecond.
+        # No more workgroups than CUs (256)
+        n_splits = max(1, min(16 if max_seq > 2048 else 8, 256 // max(1, batch * a_.n_kv_heads)))
         self.attn_ws = AttnWorkspace(batch, a_.n_heads, a_.n_kv_heads, n_splits, model.tok_embeddings.weight.device)
         self.batch = batch
         self.max_seq = max_seq
