@@ -285,11 +285,16 @@ constexpr int kDfRecFloats = kHeadDim + 2;  // record of one (sequence, kv head,
 constexpr int kDfMaxSplits = 16;
 constexpr int kDfMaxWaves = 8;
 
-template <int G>
+// ROWS: the rotation's cos / sin values of every sequence's position come as a ready row
+// (rope_rows[b] = cos[64] | sin[64], written once per step by decode_step_begin_kernel) instead of
+// from the tables at an index that has to be loaded first: one memory round trip less in front of
+// the rope.
+template <int G, bool ROWS>
 __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    uint16_t* __restrict__ out, float* workspace, int* counters, int S, int span, int n_heads, int n_kv_heads) {
+    const float* __restrict__ rope_rows, uint16_t* __restrict__ out, float* workspace, int* counters, int S, int span,
+    int n_heads, int n_kv_heads) {
     __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
     __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
     __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
@@ -323,6 +328,7 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     constexpr int kItems = (G + 2) * (kHeadDim / 2);
     constexpr int kIters = (kItems + 255) / 256;
     uint32_t praw[kIters];
+    float rcs[kIters], rsn[kIters];
 #pragma unroll
     for (int u = 0; u < kIters; ++u) {
         const int it = tid + u * nthreads;
@@ -330,6 +336,10 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
         const int i = it - hh * (kHeadDim / 2);
         const int src = hh < G ? (kvh * G + hh) * kHeadDim : (hh == G ? (n_heads + kvh) : (n_heads + n_kv_heads + kvh)) * kHeadDim;
         praw[u] = *(const uint32_t*)(row + (it < kItems ? src + 2 * i : 0));
+        if (ROWS) {
+            rcs[u] = rope_rows[(size_t)b * kHeadDim + i];
+            rsn[u] = rope_rows[(size_t)b * kHeadDim + kHeadDim / 2 + i];
+        }
     }
     v4u kb[2][4], vb[8];
     auto load_rows = [&](int r0) {  // rows r0 .. r0 + 31 of the slice
@@ -367,7 +377,8 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
             if (hh <= G) {
                 if (hh < G || owns_new) {
                     const float a = bf16f(praw[u] & 0xffffu), cc = bf16f(praw[u] >> 16);
-                    const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
+                    const float cs = ROWS ? rcs[u] : cos_t[(size_t)p * (kHeadDim / 2) + i];
+                    const float sn = ROWS ? rsn[u] : sin_t[(size_t)p * (kHeadDim / 2) + i];
                     const uint32_t rot = (uint32_t)to_bf16(a * cs - cc * sn) | ((uint32_t)to_bf16(a * sn + cc * cs) << 16);
                     if (hh < G) {
                         *(uint32_t*)(&qb[hh][2 * i]) = rot;
@@ -554,19 +565,64 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
 
 }  // namespace
 
-// Launcher used by bitnet_attn_decode (decoder_ops.hip), which has validated the arguments.
+// Launcher used by bitnet_attn_decode / bitnet_attn_decode_rows (decoder_ops.hip), which have validated
+// the arguments.  rope_rows may be null: the rotation values then come from the tables.
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
-                                    const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
-                                    int* counters, int n_splits, int span, int threads, int B, int S, int n_heads,
-                                    int n_kv_heads, hipStream_t stream) {
+                                    const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
+                                    float* workspace, int* counters, int n_splits, int span, int threads, int B, int S,
+                                    int n_heads, int n_kv_heads, hipStream_t stream) {
     const int g = n_heads / n_kv_heads;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
+#define BITNET_DF_LAUNCH(GG, RR)                                                                                           \
+    hipLaunchKernelGGL((attn_decode_flash_kernel<GG, RR>), grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, \
+                       sin_table, rope_rows, out, workspace, counters, S, span, n_heads, n_kv_heads)
+#define BITNET_DF_LAUNCH_G(GG)     \
+    if (rope_rows)                 \
+        BITNET_DF_LAUNCH(GG, true); \
+    else                           \
+        BITNET_DF_LAUNCH(GG, false)
     switch (g) {
-        case 1: hipLaunchKernelGGL(attn_decode_flash_kernel<1>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
-        case 2: hipLaunchKernelGGL(attn_decode_flash_kernel<2>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
-        case 4: hipLaunchKernelGGL(attn_decode_flash_kernel<4>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
-        default: hipLaunchKernelGGL(attn_decode_flash_kernel<8>, grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads); break;
+        case 1: BITNET_DF_LAUNCH_G(1); break;
+        case 2: BITNET_DF_LAUNCH_G(2); break;
+        case 4: BITNET_DF_LAUNCH_G(4); break;
+        default: BITNET_DF_LAUNCH_G(8); break;
     }
+#undef BITNET_DF_LAUNCH_G
+#undef BITNET_DF_LAUNCH
+    return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+namespace {
+// Start of a decode step: the embedding row of every sequence's input token (tok_embeddings,
+// gpu/model.py:272) and the cos | sin row of its position, so that the layers' attention kernels
+// need not look the position up before they can rotate.  One workgroup per sequence.
+__global__ __launch_bounds__(256) void decode_step_begin_kernel(
+    const int64_t* __restrict__ tokens, const int64_t* __restrict__ positions, const uint16_t* __restrict__ emb,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, uint16_t* __restrict__ h_out,
+    float* __restrict__ rope_rows, int V, int dim, int S) {
+    const int b = blockIdx.x;
+    const int64_t t_raw = tokens[b], p_raw = positions[b];
+    const int64_t t = t_raw < 0 ? 0 : (t_raw >= (int64_t)V ? V - 1 : t_raw);       // clamped: nothing outside the buffers is read
+    const int p = p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw);
+    const uint4* src = (const uint4*)(emb + (size_t)t * dim);
+    uint4* dst = (uint4*)(h_out + (size_t)b * dim);
+    for (int i = threadIdx.x; i < dim / 8; i += 256) dst[i] = src[i];
+    if (threadIdx.x < kHeadDim) {
+        const int i = threadIdx.x & (kHeadDim / 2 - 1);
+        rope_rows[(size_t)b * kHeadDim + threadIdx.x] =
+            threadIdx.x < kHeadDim / 2 ? cos_t[(size_t)p * (kHeadDim / 2) + i] : sin_t[(size_t)p * (kHeadDim / 2) + i];
+    }
+}
+}  // namespace
+
+extern "C" int bitnet_decode_step_begin(const int64_t* tokens, const int64_t* positions, const uint16_t* emb,
+                                        const float* cos_table, const float* sin_table, uint16_t* h_out, float* rope_rows,
+                                        int B, int V, int dim, int S, int head_dim, void* stream) {
+    if (B < 1 || V < 1 || dim < 8 || dim % 8 || S < 1 || head_dim != kHeadDim) return 1;
+    if (!tokens || !positions || !emb || !cos_table || !sin_table || !h_out || !rope_rows) return 2;
+    if ((((uintptr_t)emb) | ((uintptr_t)h_out)) & 15u) return 1;
+    hipLaunchKernelGGL(decode_step_begin_kernel, dim3(B, 1, 1), dim3(256, 1, 1), 0, (hipStream_t)stream, tokens, positions, emb,
+                       cos_table, sin_table, h_out, rope_rows, V, dim, S);
     return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

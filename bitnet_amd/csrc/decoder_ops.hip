@@ -755,9 +755,9 @@ static int g_attn_kernel = 0;  // 0 = built-in choice, 1 = score buffer in LDS +
 
 // in attn_prefill.hip
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
-                                    const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
-                                    int* counters, int n_splits, int span, int threads, int B, int S, int n_heads,
-                                    int n_kv_heads, hipStream_t stream);
+                                    const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
+                                    float* workspace, int* counters, int n_splits, int span, int threads, int B, int S,
+                                    int n_heads, int n_kv_heads, hipStream_t stream);
 
 /* tuning override for tests and measurements: which of the two decode-step attention kernels runs */
 extern "C" int bitnet_attn_decode_set_kernel(int which) {
@@ -778,10 +778,10 @@ extern "C" int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_
     return B * n_kv_heads * n_splits * (n_heads / n_kv_heads) * kRecFloats;
 }
 
-extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
-                                  const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
-                                  int* counters, int n_splits, int B, int S, int n_heads, int n_kv_heads, int head_dim,
-                                  void* stream) {
+static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
+                            const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
+                            float* workspace, int* counters, int n_splits, int B, int S, int n_heads, int n_kv_heads,
+                            int head_dim, void* stream) {
     if (B < 1 || S < 1 || n_heads < 1 || n_kv_heads < 1 || head_dim != kHeadDim) return 1;
     if (n_heads % n_kv_heads) return 1;
     const int g = n_heads / n_kv_heads;
@@ -802,8 +802,8 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     if (flash) threads = (span > 128 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
     if (g_attn_threads) threads = g_attn_threads;
     if (flash)
-        return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, out, workspace, counters,
-                                               n_splits, span, threads, B, S, n_heads, n_kv_heads, (hipStream_t)stream);
+        return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, rope_rows, out, workspace,
+                                               counters, n_splits, span, threads, B, S, n_heads, n_kv_heads, (hipStream_t)stream);
     const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * 1024) * sizeof(float);  // scores + one 4 KB region per wave
     if (lds > 96u * 1024u) return 1;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
@@ -826,6 +826,23 @@ extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16
     }
 #undef BITNET_ATTN_LAUNCH
     return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
+                                  const float* cos_table, const float* sin_table, uint16_t* out, float* workspace,
+                                  int* counters, int n_splits, int B, int S, int n_heads, int n_kv_heads, int head_dim,
+                                  void* stream) {
+    return attn_decode_impl(qkv, cache_k, cache_v, positions, cos_table, sin_table, nullptr, out, workspace, counters, n_splits,
+                            B, S, n_heads, n_kv_heads, head_dim, stream);
+}
+
+extern "C" int bitnet_attn_decode_rows(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
+                                       const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
+                                       float* workspace, int* counters, int n_splits, int B, int S, int n_heads,
+                                       int n_kv_heads, int head_dim, void* stream) {
+    if (!rope_rows) return 2;
+    return attn_decode_impl(qkv, cache_k, cache_v, positions, cos_table, sin_table, rope_rows, out, workspace, counters,
+                            n_splits, B, S, n_heads, n_kv_heads, head_dim, stream);
 }
 
 static int g_lm_kernel = 0;  // 0 = built-in choice, 1 = matrix-pipe kernel, 2 = streaming kernel where it applies

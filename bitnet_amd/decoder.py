@@ -79,21 +79,44 @@ class AttnWorkspace:
         self.counters = torch.zeros(batch * n_kv_heads, dtype=torch.int32, device=device)
 
 
-def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads, workspace: "AttnWorkspace" = None):
+def decode_step_begin(tokens, positions, emb_weight, cos, sin):
+    """Embedding rows of the step's input tokens and the cos | sin rows of their
+    positions in one launch (bitnet_decode_step_begin).  tokens / positions
+    int64 [B]; returns (h bf16 [B, dim], rope_rows fp32 [B, 128])."""
+    B = tokens.shape[0]
+    V, dim = emb_weight.shape
+    h = torch.empty(B, dim, dtype=torch.bfloat16, device=tokens.device)
+    rows = torch.empty(B, 2 * cos.shape[1], dtype=torch.float32, device=tokens.device)
+    st = _lib.load_library().bitnet_decode_step_begin(
+        _ptr(tokens), _ptr(positions), _ptr(emb_weight), _ptr(cos), _ptr(sin), _ptr(h), _ptr(rows),
+        B, V, dim, cos.shape[0], 2 * cos.shape[1], _stream_ptr())
+    if st != 0:
+        raise _lib.BitLinearLibraryError(f"bitnet_decode_step_begin: status {st}")
+    return h, rows
+
+
+def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads, workspace: "AttnWorkspace" = None,
+                rope_rows=None):
     """Rope + KV-cache write + grouped-query attention of one new token per
-    sequence in one HIP kernel (bitnet_attn_decode).  xqkv bf16 [B, (n_heads +
-    2 n_kv) * 128]; positions int64 [B]; returns bf16 [B, n_heads * 128]."""
+    sequence in one HIP kernel (bitnet_attn_decode; bitnet_attn_decode_rows
+    when the positions' cos | sin rows are handed over).  xqkv bf16 [B,
+    (n_heads + 2 n_kv) * 128]; positions int64 [B]; returns bf16 [B, n_heads * 128]."""
     B = xqkv.shape[0]
     S = cache_k.shape[1]
     hd = cache_k.shape[-1]
     out = torch.empty(B, n_heads * hd, dtype=torch.bfloat16, device=xqkv.device)
     ns = workspace.n_splits if workspace is not None else 1
-    st = _lib.load_library().bitnet_attn_decode(
-        _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out),
-        _ptr(workspace.partials) if workspace is not None else None,
-        _ptr(workspace.counters) if workspace is not None else None,
-        ns, B, S, n_heads, n_kv_heads, hd, _stream_ptr(),
-    )
+    lib = _lib.load_library()
+    wsp = _ptr(workspace.partials) if workspace is not None else None
+    wsc = _ptr(workspace.counters) if workspace is not None else None
+    if rope_rows is not None:
+        st = lib.bitnet_attn_decode_rows(
+            _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(rope_rows), _ptr(out),
+            wsp, wsc, ns, B, S, n_heads, n_kv_heads, hd, _stream_ptr())
+    else:
+        st = lib.bitnet_attn_decode(
+            _ptr(xqkv), _ptr(cache_k), _ptr(cache_v), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out),
+            wsp, wsc, ns, B, S, n_heads, n_kv_heads, hd, _stream_ptr())
     if st != 0:
         raise _lib.BitLinearLibraryError(f"bitnet_attn_decode: status {st}")
     return out
@@ -280,11 +303,14 @@ class Transformer(nn.Module):
         a = self.args
         B = tokens.shape[0]
         pos = positions.reshape(B)
-        h = self.tok_embeddings(tokens.reshape(B))
+        if self.tok_embeddings.weight.dtype == torch.bfloat16 and a.dim % 8 == 0:
+            h, rows = decode_step_begin(tokens.reshape(B), pos, self.tok_embeddings.weight, cos, sin)
+        else:
+            h, rows = self.tok_embeddings(tokens.reshape(B)), None
         for layer, (ck, cv) in zip(self.layers, cache):
             att, ffn = layer.attention, layer.feed_forward
             xqkv = norm_bitlinear(h, layer.attention_norm, att.wqkv)
-            o = attn_decode(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads, workspace)
+            o = attn_decode(xqkv, ck, cv, pos, cos, sin, a.n_heads, a.n_kv_heads, workspace, rope_rows=rows)
             h = norm_bitlinear(o, att.attn_sub_norm, att.wo, residual=h)
             x13 = norm_bitlinear(h, layer.ffn_norm, ffn.w13)
             h = norm_bitlinear(x13, ffn.ffn_sub_norm, ffn.w2, glu=True, residual=h)

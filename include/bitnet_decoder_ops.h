@@ -49,6 +49,31 @@ int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v
                        int n_kv_heads, int head_dim, void* stream);
 
 /*
+ * Start of a decode step: h_out[b, :] = emb[tokens[b], :] (tok_embeddings, gpu/model.py:272) and
+ * rope_rows[b, :] = cos_table[positions[b], :] | sin_table[positions[b], :] (64 + 64 floats), one
+ * launch.  The rows let the step's attention kernels rotate without first loading the position
+ * (bitnet_attn_decode_rows).  tokens / positions int64 [B] (clamped into [0, V) / [0, S) by the
+ * kernel); emb bf16 [V, dim], dim % 8 == 0, emb and h_out 16-byte aligned; cos/sin fp32
+ * [S, head_dim / 2]; head_dim must be 128.  Returns 0, 1 (shape / alignment), 2 (null), 3 (launch).
+ */
+int bitnet_decode_step_begin(const int64_t* tokens, const int64_t* positions, const uint16_t* emb,
+                             const float* cos_table, const float* sin_table, uint16_t* h_out,
+                             float* rope_rows, int B, int V, int dim, int S, int head_dim,
+                             void* stream);
+
+/*
+ * bitnet_attn_decode with the rotation values of every sequence's position handed over as ready
+ * rows (rope_rows float [B, head_dim], as bitnet_decode_step_begin writes them; they must be the
+ * tables' rows at positions[b]): results are identical, the kernel saves the memory round trip of
+ * the table lookup behind the position.  With kernel 1 selected the rows are ignored.
+ */
+int bitnet_attn_decode_rows(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v,
+                            const int64_t* positions, const float* cos_table,
+                            const float* sin_table, const float* rope_rows, uint16_t* out,
+                            float* workspace, int* counters, int n_splits, int B, int S,
+                            int n_heads, int n_kv_heads, int head_dim, void* stream);
+
+/*
  * Rotary embedding and KV-cache write for a block of T new tokens per sequence (the prompt
  * pass of Attention.forward, gpu/model.py:128-157, where the reference calls xformers'
  * rope_padded): for token (b, t) at position positions[b * T + t]

@@ -181,6 +181,15 @@ def test_attention_decode_kernel_against_torch_fp32(B, S, nh, nkv, n_splits, whi
             assert int(ws.counters.abs().sum()) == 0  # arrival counters reset by the last split
             again = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)  # same cache row rewritten
             assert torch.equal(again, got)
+        # the same call with the positions' cos | sin rows handed over: identical bits
+        emb = torch.randn(16, 64, generator=g, device=dev).to(torch.bfloat16)
+        toks = torch.randint(0, 16, (B,), generator=g, device=dev)
+        h0, rows = decoder.decode_step_begin(toks, pos, emb, cos, sin)
+        assert torch.equal(h0, emb[toks]) and torch.equal(rows, torch.cat([cos[pos], sin[pos]], dim=1))
+        ck2, cv2 = ck.clone(), cv.clone()
+        with_rows = decoder.attn_decode(xqkv, ck2, cv2, pos, cos, sin, nh, nkv, ws, rope_rows=rows)
+        torch.cuda.synchronize()
+        assert torch.equal(with_rows, got) and torch.equal(ck2, rk) and torch.equal(cv2, rv)
     finally:
         lib.bitnet_attn_decode_set_kernel(0)
     ulps, tol = (2, 2e-3) if which == 1 else (3, 4e-3)
