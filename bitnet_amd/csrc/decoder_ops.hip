@@ -26,6 +26,7 @@ namespace {
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kHeadDim = 128;
 constexpr int kMaxGroup = 8;
@@ -685,8 +686,8 @@ __global__ __launch_bounds__(kLmThreads) void lm_head_stream_kernel(const uint16
     }
 }
 
-// Best (value, row) per token over the workgroups' partial results: one workgroup, one wave per
-// token, eight independent loads per lane in flight (a dependent chain of single loads would cost a
+// Best (value, row) per token over the workgroups' partial results: one workgroup, all loads of a
+// thread independent and in flight together (a dependent chain of single loads would cost a
 // memory round trip each).  A kernel of its own: the kernel boundary orders the partial results for
 // free, where a device-wide arrival counter would serialise thousands of atomics on one address.
 constexpr int kLmFinalThreads = kLmMaxTokens * 64;
@@ -704,42 +705,82 @@ __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const fl
                                                                         const int* __restrict__ part_idx,
                                                                         int64_t* __restrict__ token_out, int nparts, int B,
                                                                         LmStepBook book) {
-    const int tid = threadIdx.x;
-    const int t = tid >> 6, sub = tid & 63;
-    float v = -INFINITY;
-    int i = 0x7fffffff;
-    constexpr int U = 8;
-    for (int base = sub; base < nparts; base += 64 * U) {
-        float ov[U];
-        int oi[U];
+    // The candidates are [nparts][16 token slots]; a thread reads whole 16-byte pieces (four token
+    // slots of one workgroup's candidates), consecutive threads consecutive pieces.  One workgroup's
+    // loads all go through one CU's address path, which handles one 64-byte segment per cycle: with
+    // a lane per candidate and a wave per token every load instruction touched 64 segments and the
+    // kernel took 16 us; now a load instruction touches 16.
+    __shared__ float sv[kLmFinalThreads / 64][kLmMaxTokens];
+    __shared__ int si[kLmFinalThreads / 64][kLmMaxTokens];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = tid & 3;  // this thread's token slots are 4 q .. 4 q + 3
+    float v[4];
+    int i[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        v[e] = -INFINITY;
+        i[e] = 0x7fffffff;
+    }
+    const int nvec = nparts * 4;
+    constexpr int U = 4;
+    for (int base = tid; base < nvec; base += kLmFinalThreads * U) {
+        v4f ov[U];
+        v4i oi[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int k = base + 64 * u;
-            const size_t at = (size_t)(k < nparts ? k : nparts - 1) * kLmMaxTokens + t;
-            ov[u] = part_val[at];
-            oi[u] = part_idx[at];
+            const int k = base + kLmFinalThreads * u;
+            const int at = k < nvec ? k : nvec - 4 + q;  // a piece of the same token slots
+            ov[u] = ((const v4f*)part_val)[at];
+            oi[u] = ((const v4i*)part_idx)[at];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (base + 64 * u < nparts && lm_better(ov[u], oi[u], v, i)) {
-                v = ov[u];
-                i = oi[u];
+            if (base + kLmFinalThreads * u < nvec) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (lm_better(ov[u][e], oi[u][e], v[e], i[e])) {
+                        v[e] = ov[u][e];
+                        i[e] = oi[u][e];
+                    }
             }
     }
+    // the 16 lanes of a wave that hold the same token slots
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float ov = __shfl_xor(v, off);
-        const int oi = __shfl_xor(i, off);
-        if (lm_better(ov, oi, v, i)) {
-            v = ov;
-            i = oi;
+    for (int off = 4; off < 64; off <<= 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float ov = __shfl_xor(v[e], off);
+            const int oi = __shfl_xor(i[e], off);
+            if (lm_better(ov, oi, v[e], i[e])) {
+                v[e] = ov;
+                i[e] = oi;
+            }
         }
     }
-    if (sub == 0 && t < B) {
-        token_out[t] = (int64_t)i;
-        if (book.next_input) book.next_input[t] = (int64_t)i;
-        if (book.positions) book.positions[t] += 1;
-        if (book.history && book.step_idx) book.history[book.step_idx[0] * B + t] = (int64_t)i;
+    if (lane < 4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            sv[wave][4 * lane + e] = v[e];
+            si[wave][4 * lane + e] = i[e];
+        }
+    }
+    __syncthreads();
+    if (tid < kLmMaxTokens) {
+        const int t = tid;
+        float bv = sv[0][t];
+        int bi = si[0][t];
+#pragma unroll
+        for (int w = 1; w < kLmFinalThreads / 64; ++w)
+            if (lm_better(sv[w][t], si[w][t], bv, bi)) {
+                bv = sv[w][t];
+                bi = si[w][t];
+            }
+        if (t < B) {
+            token_out[t] = (int64_t)bi;
+            if (book.next_input) book.next_input[t] = (int64_t)bi;
+            if (book.positions) book.positions[t] += 1;
+            if (book.history && book.step_idx) book.history[book.step_idx[0] * B + t] = (int64_t)bi;
+        }
     }
     if (book.step_idx) {
         __syncthreads();  // every token's history row index has been read
@@ -865,7 +906,9 @@ static int lm_head_greedy_impl(const uint16_t* h, const uint16_t* norm_weight, f
                                const LmStepBook& book, int B, int V, int K, void* stream) {
     if (B < 1 || B > kLmMaxTokens || V < 1 || K < 64 || (K % 64) != 0) return 1;
     if (!h || !norm_weight || !emb || !y_ws || !token_out || !part_val || !part_idx) return 2;
-    if ((((uintptr_t)h) | ((uintptr_t)norm_weight) | ((uintptr_t)emb) | ((uintptr_t)y_ws)) & 15u) return 1;
+    if ((((uintptr_t)h) | ((uintptr_t)norm_weight) | ((uintptr_t)emb) | ((uintptr_t)y_ws) | ((uintptr_t)part_val) |
+         ((uintptr_t)part_idx)) & 15u)
+        return 1;
     const size_t lds = (size_t)B * (2 * (size_t)K + kLmRowPad);
     if (lds > 96u * 1024u) return 1;
     static bool raised = false;  // more than 64 KiB of dynamic LDS has to be asked for, once per process

@@ -130,7 +130,8 @@ int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int 
  *   h bf16 [B, K]; norm_weight bf16 [K]; emb bf16 [V, K] row-major; y_ws bf16 [B, K] scratch;
  *   logits fp32 [B, V] or NULL (not written then); token_out int64 [B];
  *   part_val float / part_idx int [bitnet_lm_head_workgroups(V) * 16] scratch.
- * B <= 16, K % 64 == 0, B * (2 K + 32) <= 96 KiB; h, norm_weight, emb, y_ws 16-byte aligned.
+ * B <= 16, K % 64 == 0, B * (2 K + 32) <= 96 KiB; h, norm_weight, emb, y_ws, part_val, part_idx
+ * 16-byte aligned.
  * Three launches (norm; product with a best row per workgroup; reduction of those).
  * Returns 0, 1 (shape / alignment), 2 (null), 3 (launch).
  * Calls that share the scratch buffers must not overlap in time.
