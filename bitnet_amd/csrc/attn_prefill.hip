@@ -281,7 +281,9 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_kernel(
 // the slice at a time and does scores, softmax and P.V for the G query heads (columns c < G of the
 // 16-column tiles) entirely in registers; the waves' (maximum, sum, outputs) are combined through
 // LDS once.  No score buffer, no barrier between scores, softmax and P.V.
-constexpr int kDfRecFloats = kHeadDim + 2;  // record of one (sequence, kv head, split, head): 128 outputs, maximum, sum
+constexpr int kDfRecUnits = kHeadDim + 2;  // record of one (sequence, kv head, split, head): 128 outputs, maximum, sum,
+                                            // each an 8-byte unit (value, tag of the call that wrote it)
+constexpr int kDfSpinLimit = 1 << 16;       // polls of the merging workgroup before it gives up (never reached: see below)
 constexpr int kDfMaxSplits = 16;
 constexpr int kDfMaxWaves = 8;
 
@@ -300,7 +302,6 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
     __shared__ __attribute__((aligned(16))) float part_o[kDfMaxWaves][G][kHeadDim];
     __shared__ float part_m[kDfMaxWaves][G], part_l[kDfMaxWaves][G];
-    __shared__ int is_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -341,6 +342,10 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
             rsn[u] = rope_rows[(size_t)b * kHeadDim + kHeadDim / 2 + i];
         }
     }
+    // the tag of this call's records: one more than the epoch the last merge of this (sequence, kv head)
+    // left behind (an unconditional load: with one split there is no workspace and the value is unused)
+    const int* epochs = (const int*)(workspace + (size_t)gridDim.y * n_kv_heads * nsplit * G * kDfRecUnits * 2);
+    const int epoch = *(nsplit > 1 ? epochs + (b * n_kv_heads + kvh) : (const int*)positions);
     v4u kb[2][4], vb[8];
     auto load_rows = [&](int r0) {  // rows r0 .. r0 + 31 of the slice
 #pragma unroll
@@ -365,6 +370,12 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
 #pragma unroll
     for (int k = 1; k < kDfMaxSplits; ++k) nact += (k < nsplit && p >= k * span) ? 1 : 0;
     const bool active = sp < nact;
+    // The workgroup of the last active split merges the splits' records: workgroups start in the
+    // order of their index, so when it runs every other active split of this (sequence, kv head)
+    // has started and will deliver its record; and having a slice of its own to work through, it
+    // begins to poll about when the others finish (the last split of the grid, idle while the
+    // position is below its slice, polled from the start and its traffic slowed the others down).
+    const bool merger = nact > 1 && sp == nact - 1;
 
     // rope on adjacent pairs, fp32, rounded to bf16: q into LDS; the split that holds position p also
     // rotates k, keeps k and v of the new token in LDS and writes them to the cache
@@ -491,7 +502,13 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     __syncthreads();
 
     uint16_t* orow = out + (size_t)b * n_heads * kHeadDim + (size_t)(kvh * G) * kHeadDim;
-    float* rec = workspace + ((size_t)(b * n_kv_heads + kvh) * nsplit) * G * kDfRecFloats;
+    // Records are 8-byte units (value, tag) written with single device-coherent (write-through)
+    // stores: a reader that finds this call's tag in a unit has that unit's value, so nobody waits
+    // for the stores to be acknowledged and no arrival counter is needed -- the merging workgroup
+    // polls the units it needs until they carry the tag.  Against "stores, barrier until they are
+    // acknowledged, device-scope counter, loads" this saves one of the three trips across the chip.
+    unsigned long long* rec = (unsigned long long*)workspace + ((size_t)(b * n_kv_heads + kvh) * nsplit) * G * kDfRecUnits;
+    const unsigned long long tag = (unsigned long long)(unsigned)(epoch + 1) << 32;
     for (int hh = wave; hh < G; hh += nwaves) {
         float mx = -INFINITY;
         for (int k = 0; k < nwaves; ++k) mx = fmaxf(mx, part_m[k][hh]);
@@ -509,58 +526,66 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
             const float is = 1.0f / l;
             *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
         } else {
-            // device-coherent (write-through) stores: the record reaches the point where the other
-            // XCDs' loads see it without a writeback of this XCD's whole L2
-            float* r = rec + ((size_t)sp * G + hh) * kDfRecFloats;
-            __hip_atomic_store(r + 2 * lane, o0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(r + 2 * lane + 1, o1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned long long* r = rec + ((size_t)sp * G + hh) * kDfRecUnits;
+            __hip_atomic_store(r + 2 * lane, tag | __float_as_uint(o0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(r + 2 * lane + 1, tag | __float_as_uint(o1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (lane == 0) {
-                __hip_atomic_store(r + kHeadDim, mx * scale, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // in units of the scaled scores
-                __hip_atomic_store(r + kHeadDim + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(r + kHeadDim, tag | __float_as_uint(mx * scale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // in units of the scaled scores
+                __hip_atomic_store(r + kHeadDim + 1, tag | __float_as_uint(l), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
-    if (nact == 1) return;
+    if (!merger) return;
 
-    // The last split of this (sequence, kv head) to finish combines the records: the barrier waits
-    // until every thread's record stores have completed (write-through: completed = visible
-    // device-wide); then the arrival is counted with a device-scope atomic, and the last arrival
-    // reads the records with device-coherent loads.
-    __syncthreads();
-    if (tid == 0) {
-        const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = done == nact - 1;
-        if (is_last) __hip_atomic_store(&counters[b * n_kv_heads + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!is_last) return;
+    // The merge, eight splits at a time: all units of a batch are requested together and requested
+    // again while one of them still carries an older tag.  The poll ends: every split polled has
+    // started before this workgroup and writes its record without waiting for anything.  (The limit
+    // only keeps a wrongly initialised workspace from hanging the GPU.)
+    constexpr int kBatch = 8;
     for (int hh = wave; hh < G; hh += nwaves) {
-        float mk[kDfMaxSplits], lk[kDfMaxSplits], p0[kDfMaxSplits], p1[kDfMaxSplits];
+        float mx = -INFINITY, l = 0.0f, o0 = 0.0f, o1 = 0.0f;
+        for (int k0 = 0; k0 < nact; k0 += kBatch) {
+            unsigned long long um[kBatch], ul[kBatch], u0[kBatch], u1[kBatch];
+            for (int spin = 0; spin < kDfSpinLimit; ++spin) {
+                bool ok = true;
 #pragma unroll
-        for (int k = 0; k < kDfMaxSplits; ++k) {
-            const float* r = rec + ((size_t)(k < nact ? k : 0) * G + hh) * kDfRecFloats;
-            mk[k] = __hip_atomic_load(r + kHeadDim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            lk[k] = __hip_atomic_load(r + kHeadDim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            p0[k] = __hip_atomic_load(r + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            p1[k] = __hip_atomic_load(r + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        float mx = -INFINITY;
+                for (int k = 0; k < kBatch; ++k) {
+                    const unsigned long long* r = rec + ((size_t)((k0 + k) < nact ? (k0 + k) : k0) * G + hh) * kDfRecUnits;
+                    um[k] = __hip_atomic_load(r + kHeadDim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ul[k] = __hip_atomic_load(r + kHeadDim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    u0[k] = __hip_atomic_load(r + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    u1[k] = __hip_atomic_load(r + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
 #pragma unroll
-        for (int k = 0; k < kDfMaxSplits; ++k)
-            if (k < nact) mx = fmaxf(mx, mk[k]);
-        float l = 0.0f, o0 = 0.0f, o1 = 0.0f;
+                for (int k = 0; k < kBatch; ++k)
+                    ok = ok && ((um[k] & ul[k] & u0[k] & u1[k]) >> 32) == (tag >> 32) && ((um[k] | ul[k] | u0[k] | u1[k]) >> 32) == (tag >> 32);
+                if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+            }
+            float bm = mx;
 #pragma unroll
-        for (int k = 0; k < kDfMaxSplits; ++k) {
-            if (k < nact && lk[k] > 0.0f) {
-                const float w = __expf(mk[k] - mx);
-                l += lk[k] * w;
-                o0 += w * p0[k];
-                o1 += w * p1[k];
+            for (int k = 0; k < kBatch; ++k)
+                if (k0 + k < nact) bm = fmaxf(bm, __uint_as_float((unsigned)um[k]));
+            const float wold = l > 0.0f ? __expf(mx - bm) : 0.0f;
+            l *= wold;
+            o0 *= wold;
+            o1 *= wold;
+            mx = bm;
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k) {
+                const float lk = __uint_as_float((unsigned)ul[k]);
+                if (k0 + k < nact && lk > 0.0f) {
+                    const float w = __expf(__uint_as_float((unsigned)um[k]) - mx);
+                    l += lk * w;
+                    o0 += w * __uint_as_float((unsigned)u0[k]);
+                    o1 += w * __uint_as_float((unsigned)u1[k]);
+                }
             }
         }
         const float is = 1.0f / l;
         *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
     }
+    __syncthreads();  // every wave has read its records
+    if (tid == 0) ((int*)epochs)[b * n_kv_heads + kvh] = epoch + 1;
 }
 
 }  // namespace

@@ -816,7 +816,9 @@ extern "C" int bitnet_attn_decode_set_threads(int threads) {
 
 extern "C" int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits) {
     if (B < 1 || n_heads < 1 || n_kv_heads < 1 || n_splits < 1 || n_heads % n_kv_heads) return -1;
-    return B * n_kv_heads * n_splits * (n_heads / n_kv_heads) * kRecFloats;
+    // records of 8-byte units (value, tag) per (sequence, kv head, split, head), then one epoch per (sequence, kv head)
+    const long long n = (long long)B * n_kv_heads * n_splits * (n_heads / n_kv_heads) * kRecFloats * 2 + (long long)B * n_kv_heads;
+    return n < (1ll << 31) ? (int)n : -1;
 }
 
 static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
@@ -831,6 +833,7 @@ static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* ca
     if (n_splits < 1 || n_splits > (flash ? 16 : kMaxSplits)) return 1;
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
     if (n_splits > 1 && (!workspace || !counters)) return 2;
+    if (((uintptr_t)workspace) & 7u) return 1;
     if ((size_t)(S + 512) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;  // the kernel's 32-bit byte offsets into one sequence's cache
     const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // fixed slice of the cache per split
     // Eight waves take a slice of up to 128 rows in one round of loads (four waves: 64 rows; a

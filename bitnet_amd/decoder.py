@@ -67,15 +67,16 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
 
 
 class AttnWorkspace:
-    """Scratch of the split attention kernel: partial results of the splits and
-    one self-resetting arrival counter per (sequence, kv head).  One instance
+    """Scratch of the split attention kernel: tagged partial results of the
+    splits (zero before the first use) and one arrival counter per (sequence,
+    kv head) for the earlier kernel.  One instance
     serves all layers of a decoder (their kernels run one after the other)."""
 
     def __init__(self, batch: int, n_heads: int, n_kv_heads: int, n_splits: int, device):
         lib = _lib.load_library()
         self.n_splits = n_splits
         n = lib.bitnet_attn_decode_workspace_floats(batch, n_heads, n_kv_heads, n_splits)
-        self.partials = torch.empty(max(n, 1), dtype=torch.float32, device=device)
+        self.partials = torch.zeros(max(n, 1), dtype=torch.float32, device=device)  # zero once: see bitnet_attn_decode
         self.counters = torch.zeros(batch * n_kv_heads, dtype=torch.int32, device=device)
 
 

@@ -28,7 +28,9 @@ extern "C" {
  *            into that range by the kernel: no access leaves the buffers)
  *   cos/sin  fp32 [S, head_dim / 2]
  *   out      bf16 [B, n_heads * head_dim]
- *   workspace float [bitnet_attn_decode_workspace_floats(B, n_heads, n_kv_heads, n_splits)]
+ *   workspace float [bitnet_attn_decode_workspace_floats(B, n_heads, n_kv_heads, n_splits)], 8-byte
+ *            aligned and zero before the first call that uses it (the calls keep it consistent: every
+ *            split's record carries the tag of the call that wrote it, and the tag advances per call)
  *   counters  int [B * n_kv_heads], zero before the first call (every call leaves them zero)
  *   n_splits  1..16 (1..8 with kernel 1) workgroups share the S cache rows of one (sequence, kv head) in fixed slices;
  *             with 1, workspace and counters may be NULL.  Calls that share a workspace
