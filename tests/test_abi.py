@@ -82,3 +82,28 @@ def test_argument_checks_need_no_gpu(capfd):
     assert lib.bitlinear_quant_absmax(None, None, None, 1, 2560, 0, None) == 2
     assert lib.bitlinear_quant_absmax(None, None, None, 1, 2563, 0, None) == 1
     assert lib.bitlinear_int8xint2_acc_i32(None, None, None, None, None, None, 1, 2560, 100, None) == 1
+
+
+def test_decoder_entry_argument_checks_need_no_gpu():
+    """The decoder-side entry points refuse bad shapes (1) and null pointers (2)
+    before any HIP call."""
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built")
+    lib = _lib.load_library()
+    # bitnet_attn_decode: head_dim, group size, split count, nulls
+    assert lib.bitnet_attn_decode(None, None, None, None, None, None, None, None, None, 1, 1, 64, 4, 2, 64, None) == 1
+    assert lib.bitnet_attn_decode(None, None, None, None, None, None, None, None, None, 1, 1, 64, 6, 2, 128, None) == 1
+    assert lib.bitnet_attn_decode(None, None, None, None, None, None, None, None, None, 17, 1, 64, 4, 2, 128, None) == 1
+    assert lib.bitnet_attn_decode(None, None, None, None, None, None, None, None, None, 1, 1, 64, 4, 2, 128, None) == 2
+    assert lib.bitnet_attn_decode_rows(None, None, None, None, None, None, None, None, None, None, 1, 1, 64, 4, 2, 128, None) == 2
+    assert lib.bitnet_attn_decode_workspace_floats(1, 20, 5, 8) == 1 * 5 * 8 * 4 * 130 * 2 + 5
+    assert lib.bitnet_attn_decode_workspace_floats(1, 20, 6, 8) == -1
+    assert lib.bitnet_attn_decode_set_kernel(3) == 1 and lib.bitnet_attn_decode_set_kernel(0) == 0
+    # prompt side: start + T beyond the cache, head_dim, nulls
+    assert lib.bitnet_attn_prefill(None, None, None, None, 1, 40, 64, 30, 4, 2, 128, None) == 1
+    assert lib.bitnet_attn_prefill(None, None, None, None, 1, 40, 64, 0, 4, 2, 64, None) == 1
+    assert lib.bitnet_attn_prefill(None, None, None, None, 1, 40, 64, 0, 4, 2, 128, None) == 2
+    assert lib.bitnet_rope_cache_tokens(None, None, None, None, None, None, None, 1, 0, 64, 4, 2, 128, None) == 1
+    assert lib.bitnet_rope_cache_tokens(None, None, None, None, None, None, None, 1, 8, 64, 4, 2, 128, None) == 2
+    assert lib.bitnet_decode_step_begin(None, None, None, None, None, None, None, 1, 100, 250, 64, 128, None) == 1  # dim % 8
+    assert lib.bitnet_decode_step_begin(None, None, None, None, None, None, None, 1, 100, 256, 64, 128, None) == 2
