@@ -295,7 +295,7 @@ template <int G, bool ROWS>
 __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    const float* __restrict__ rope_rows, uint16_t* __restrict__ out, float* workspace, int* counters, int S, int span,
+    const float* __restrict__ rope_rows, uint16_t* __restrict__ out, float* workspace, int* counters, int S,
     int n_heads, int n_kv_heads) {
     __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
     __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
@@ -320,12 +320,18 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const int cache_bytes = (S - 1) * row_bytes + kHeadDim * 2;
     const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)ck, 0, cache_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cv, 0, cache_bytes, 0x00020000);
-    const int lo = sp * span;  // this split owns positions [lo, lo + span), span % 16 == 0
-    constexpr int kPastEnd = 0x7fff0000;
+    // The cache rows are dealt to the splits in blocks of 32: split sp owns blocks sp, sp + nsplit,
+    // sp + 2 nsplit, ... and within the split wave w takes the blocks sp + nsplit * (w + nwaves * round).
+    // Whatever the current position is, the visible rows are then spread evenly over all splits
+    // (contiguous slices of the cache capacity leave most splits idle while the position is far
+    // below the capacity), and the blocks of the first round can still be requested before the
+    // position is known.
+    const int blk0 = sp + nsplit * wave;
+    const int blk_stride = nsplit * nwaves;
 
     // Everything that depends on nothing is requested first: the token's q / k / v, the position,
-    // and the wave's first 32 K and V rows of the slice (rows outside the slice get an offset past
-    // the end of the descriptor, which costs no memory access).
+    // and the wave's first block of K and V rows (a block beyond the end of the cache lies beyond
+    // the descriptor: its requests cost no memory access and read as zero).
     constexpr int kItems = (G + 2) * (kHeadDim / 2);
     constexpr int kIters = (kItems + 255) / 256;
     uint32_t praw[kIters];
@@ -347,28 +353,24 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const int* epochs = (const int*)(workspace + (size_t)gridDim.y * n_kv_heads * nsplit * G * kDfRecUnits * 2);
     const int epoch = *(nsplit > 1 ? epochs + (b * n_kv_heads + kvh) : (const int*)positions);
     v4u kb[2][4], vb[8];
-    auto load_rows = [&](int r0) {  // rows r0 .. r0 + 31 of the slice
+    auto load_rows = [&](int blk) {  // cache rows 32 blk .. 32 blk + 31
+        const int base = blk * 32 * row_bytes;
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi) {
-            const int rel = r0 + bi * 16 + c;
-            const int off = rel < span ? (lo + rel) * row_bytes + g4 * 16 : kPastEnd;
+            const int off = base + (bi * 16 + c) * row_bytes + g4 * 16;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) kb[bi][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
         }
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            const int rel = r0 + (jj & 3) + (jj >> 2) * 16 + 4 * g4;
-            vb[jj] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, rel < span ? (lo + rel) * row_bytes + c * 16 : kPastEnd, 0, 0);
-        }
+        for (int jj = 0; jj < 8; ++jj)
+            vb[jj] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, base + ((jj & 3) + (jj >> 2) * 16 + 4 * g4) * row_bytes + c * 16, 0, 0);
     };
-    load_rows(wave * 32);
+    load_rows(blk0);
     const int64_t p_raw = positions[b];
     const int p = __builtin_amdgcn_readfirstlane(p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw));  // clamped into the cache
-    const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's visible positions are [lo, hi)
-    const bool owns_new = p >= lo && p < lo + span;
-    int nact = 1;  // splits whose slice starts at or below the position
-#pragma unroll
-    for (int k = 1; k < kDfMaxSplits; ++k) nact += (k < nsplit && p >= k * span) ? 1 : 0;
+    const int pblk = p >> 5;                        // the block of the new token's row
+    const bool owns_new = pblk % nsplit == sp;
+    const int nact = pblk + 1 < nsplit ? pblk + 1 : nsplit;  // splits that own a block with visible rows
     const bool active = sp < nact;
     // The workgroup of the last active split merges the splits' records: workgroups start in the
     // order of their index, so when it runs every other active split of this (sequence, kv head)
@@ -421,19 +423,19 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     float m_run = -INFINITY, l_run = 0.0f;
     const float scale = 0.08838834764831845f;           // 128^-0.5
     const float c2 = scale * 1.4426950408889634f;        // * log2(e): the softmax runs in base 2
-    for (int r0 = wave * 32; lo + r0 < hi; r0 += nwaves * 32) {
-        if (r0 != wave * 32) load_rows(r0);
+    for (int blk = blk0; blk <= pblk; blk += blk_stride) {
+        if (blk != blk0) load_rows(blk);
         // the new token's own row is not in the cache yet for this kernel's loads: it comes from LDS
-        if (owns_new && p - lo >= r0 && p - lo < r0 + 32) {
+        if (blk == pblk) {
 #pragma unroll
             for (int bi = 0; bi < 2; ++bi)
-                if (lo + r0 + bi * 16 + c == p) {
+                if (blk * 32 + bi * 16 + c == p) {
 #pragma unroll
                     for (int kk = 0; kk < 4; ++kk) kb[bi][kk] = *(const v4u*)(&knew[kk * 32 + g4 * 8]);
                 }
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj)
-                if (lo + r0 + (jj & 3) + (jj >> 2) * 16 + 4 * g4 == p) vb[jj] = *(const v4u*)(&vnew[c * 8]);
+                if (blk * 32 + (jj & 3) + (jj >> 2) * 16 + 4 * g4 == p) vb[jj] = *(const v4u*)(&vnew[c * 8]);
         }
         float sc[8];
 #pragma unroll
@@ -444,14 +446,14 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, kb[bi][kk]), qa[kk], acc, 0, 0, 0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int pos = lo + r0 + bi * 16 + 4 * g4 + j;
-                sc[bi * 4 + j] = pos < hi ? acc[j] : -INFINITY;
+                const int pos = blk * 32 + bi * 16 + 4 * g4 + j;
+                sc[bi * 4 + j] = pos <= p ? acc[j] : -INFINITY;
             }
         }
         float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
         mx = fmaxf(mx, xor_lane_f32(mx, lane, 16));
         mx = fmaxf(mx, xor_lane_f32(mx, lane, 32));
-        const float m_new = fmaxf(m_run, mx);  // finite: the step holds at least position lo + r0 < hi
+        const float m_new = fmaxf(m_run, mx);  // finite: the block's first row is visible (32 blk <= p)
         const float m2 = m_new * c2;
         float pr[8], psum = 0.0f;
 #pragma unroll
@@ -594,13 +596,13 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
 // the arguments.  rope_rows may be null: the rotation values then come from the tables.
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
                                     const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
-                                    float* workspace, int* counters, int n_splits, int span, int threads, int B, int S,
+                                    float* workspace, int* counters, int n_splits, int threads, int B, int S,
                                     int n_heads, int n_kv_heads, hipStream_t stream) {
     const int g = n_heads / n_kv_heads;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
 #define BITNET_DF_LAUNCH(GG, RR)                                                                                           \
     hipLaunchKernelGGL((attn_decode_flash_kernel<GG, RR>), grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, \
-                       sin_table, rope_rows, out, workspace, counters, S, span, n_heads, n_kv_heads)
+                       sin_table, rope_rows, out, workspace, counters, S, n_heads, n_kv_heads)
 #define BITNET_DF_LAUNCH_G(GG)     \
     if (rope_rows)                 \
         BITNET_DF_LAUNCH(GG, true); \

@@ -797,7 +797,7 @@ static int g_attn_kernel = 0;  // 0 = built-in choice, 1 = score buffer in LDS +
 // in attn_prefill.hip
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
                                     const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
-                                    float* workspace, int* counters, int n_splits, int span, int threads, int B, int S,
+                                    float* workspace, int* counters, int n_splits, int threads, int B, int S,
                                     int n_heads, int n_kv_heads, hipStream_t stream);
 
 /* tuning override for tests and measurements: which of the two decode-step attention kernels runs */
@@ -834,20 +834,22 @@ static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* ca
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
     if (n_splits > 1 && (!workspace || !counters)) return 2;
     if (((uintptr_t)workspace) & 7u) return 1;
-    if ((size_t)(S + 512) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;  // the kernel's 32-bit byte offsets into one sequence's cache
-    const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // fixed slice of the cache per split
+    // the kernels' 32-bit byte offsets into one sequence's cache (the first blocks requested may lie up to 4096 rows in)
+    if ((size_t)((S > 4096 ? S : 4096) + 512) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;
+    const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // a split's share of the cache capacity (kernel 1: its fixed slice)
     // Eight waves take a slice of up to 128 rows in one round of loads (four waves: 64 rows; a
     // second round exposes a full memory round trip, about 1 us).  Measured: that wins while every
     // workgroup has a CU of its own (up to 256 of them); beyond that two 512-thread workgroups
     // share a CU badly (12.9 -> 16.8 us at 320 workgroups) and 256 threads are the better choice.
     int threads = (span > 64 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
-    // the matrix-pipe kernel: a wave takes 32 rows per round, so four waves cover a slice of up to 128 rows
-    // in one round (measured at 96 rows: 6.85 us with four waves, 7.12 with eight; at 272 rows 8.77 / 8.46)
+    // the matrix-pipe kernel deals blocks of 32 rows to splits and waves: four waves cover a split's share of
+    // up to 128 rows of the capacity in one round (measured at 96 rows: 6.85 us with four waves, 7.12 with
+    // eight; at 272 rows 8.77 / 8.46)
     if (flash) threads = (span > 128 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
     if (g_attn_threads) threads = g_attn_threads;
     if (flash)
         return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, rope_rows, out, workspace,
-                                               counters, n_splits, span, threads, B, S, n_heads, n_kv_heads, (hipStream_t)stream);
+                                               counters, n_splits, threads, B, S, n_heads, n_kv_heads, (hipStream_t)stream);
     const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * 1024) * sizeof(float);  // scores + one 4 KB region per wave
     if (lds > 96u * 1024u) return 1;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);

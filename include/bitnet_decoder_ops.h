@@ -32,11 +32,12 @@ extern "C" {
  *            aligned and zero before the first call that uses it (the calls keep it consistent: every
  *            split's record carries the tag of the call that wrote it, and the tag advances per call)
  *   counters  int [B * n_kv_heads], zero before the first call (every call leaves them zero)
- *   n_splits  1..16 (1..8 with kernel 1) workgroups share the S cache rows of one (sequence, kv head) in fixed slices;
- *             with 1, workspace and counters may be NULL.  Calls that share a workspace
- *             must not overlap in time.  Fastest when B * n_kv_heads * n_splits <= 256 (one
- *             workgroup per CU: the kernel then runs eight waves per workgroup); splits whose
- *             slice starts beyond the current position cost almost nothing.
+ *   n_splits  1..16 (1..8 with kernel 1) workgroups share the cache rows of one (sequence, kv head): blocks of
+ *             32 rows dealt round-robin, so the rows up to the position are spread over all splits whatever
+ *             the capacity S is (kernel 1: fixed slices of S / n_splits rows, of which those beyond the
+ *             position cost almost nothing); with 1, workspace and counters may be NULL.  Calls that share
+ *             a workspace must not overlap in time.  Fastest when B * n_kv_heads * n_splits <= 256 (one
+ *             workgroup per CU: the kernel then runs eight waves per workgroup for long caches).
  * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8 (kernel 1 also needs
  * g * (S / n_splits + 16) * 4 bytes + 32 KiB <= 96 KiB of LDS for its scores).  Returns 0, or 1
  * (shape), 2 (null pointer), 3 (launch failed).  Scores and outputs on the bf16 matrix pipe with

@@ -197,6 +197,42 @@ def test_attention_decode_kernel_against_torch_fp32(B, S, nh, nkv, n_splits, whi
     assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance"
 
 
+@pytest.mark.parametrize("n_splits", [5, 16])
+@pytest.mark.parametrize("p", [0, 31, 32, 511, 600, 2047, 4099])
+def test_attention_decode_long_cache_any_position(p, n_splits):
+    """Cache capacity far beyond the position (4100 rows, up to 16 splits, eight
+    waves per workgroup): the rows are dealt to splits and waves in blocks of
+    32, so positions at block edges, inside the first round and in later rounds
+    are covered.  Same comparison and tolerance as above (matrix-pipe kernel)."""
+    B, S, nh, nkv, hd = 2, 4100, 8, 2, 128
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(77 + p)
+    att = decoder.Attention.__new__(decoder.Attention)
+    torch.nn.Module.__init__(att)
+    att.head_dim, att.n_heads, att.n_kv_heads = hd, nh, nkv
+    xqkv = torch.randn(B, (nh + 2 * nkv) * hd, generator=g, device=dev).to(torch.bfloat16)
+    ck = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    cv = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    pos = torch.tensor([p, max(0, p - 17)], device=dev)
+    cos, sin = decoder.rope_tables(hd, S, 500000.0, dev)
+    q, k, v = att.split_qkv(xqkv[:, None, :])
+    c, s_ = cos[pos][:, None, None, :], sin[pos][:, None, None, :]
+    q, k = decoder.apply_rope(q, c, s_), decoder.apply_rope(k, c, s_)
+    rk, rv = ck.clone(), cv.clone()
+    bidx = torch.arange(B, device=dev)
+    rk[bidx, pos] = k[:, 0]
+    rv[bidx, pos] = v[:, 0]
+    mask = torch.arange(S, device=dev)[None, None, :] <= pos[:, None, None]
+    want = att.attend(q, rk, rv, mask)[:, 0]
+    ws = decoder.AttnWorkspace(B, nh, nkv, n_splits, dev)
+    got = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
+    again = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(ck, rk) and torch.equal(cv, rv) and torch.equal(again, got)
+    bad = (_ulp(got, want) > 3) & ((got.float() - want.float()).abs() > 4e-3)
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance"
+
+
 def test_fused_decode_path_against_unfused():
     """Five-kernels-per-layer decode step vs the torch-glue step on the same
     model and cache: same cache rows for the first layer, logits within bf16
