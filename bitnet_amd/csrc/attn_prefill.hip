@@ -433,9 +433,14 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
 #pragma unroll
                     for (int kk = 0; kk < 4; ++kk) kb[bi][kk] = *(const v4u*)(&knew[kk * 32 + g4 * 8]);
                 }
+            // V rows behind the position are cleared: their probability is zero, but whatever the
+            // cache holds there (it may never have been written) must not reach the product as 0 x NaN
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj)
-                if (blk * 32 + (jj & 3) + (jj >> 2) * 16 + 4 * g4 == p) vb[jj] = *(const v4u*)(&vnew[c * 8]);
+            for (int jj = 0; jj < 8; ++jj) {
+                const int r = blk * 32 + (jj & 3) + (jj >> 2) * 16 + 4 * g4;
+                if (r == p) vb[jj] = *(const v4u*)(&vnew[c * 8]);
+                if (r > p) vb[jj] = v4u{0u, 0u, 0u, 0u};
+            }
         }
         float sc[8];
 #pragma unroll

@@ -233,6 +233,36 @@ def test_attention_decode_long_cache_any_position(p, n_splits):
     assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance"
 
 
+@pytest.mark.parametrize("which", [1, 2])
+@pytest.mark.parametrize("n_splits", [1, 8])
+def test_attention_decode_ignores_rows_behind_the_position(n_splits, which):
+    """Cache rows behind a sequence's position may never have been written:
+    with NaNs there the output has the bits it has with finite values there."""
+    B, S, nh, nkv, hd = 3, 300, 8, 2, 128
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(4242)
+    xqkv = torch.randn(B, (nh + 2 * nkv) * hd, generator=g, device=dev).to(torch.bfloat16)
+    ck = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    cv = torch.randn(B, S, nkv, hd, generator=g, device=dev).to(torch.bfloat16)
+    pos = torch.tensor([0, 37, 255], device=dev)
+    cos, sin = decoder.rope_tables(hd, S, 500000.0, dev)
+    ws = decoder.AttnWorkspace(B, nh, nkv, n_splits, dev) if n_splits > 1 else None
+    lib = _lib.load_library()
+    assert lib.bitnet_attn_decode_set_kernel(which) == 0
+    try:
+        want = decoder.attn_decode(xqkv, ck.clone(), cv.clone(), pos, cos, sin, nh, nkv, ws)
+        behind = torch.arange(S, device=dev)[None, :] > pos[:, None]
+        ck[behind] = float("nan")
+        cv[behind] = float("nan")
+        got = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitnet_attn_decode_set_kernel(0)
+    assert not torch.isnan(got.float()).any()
+    assert torch.equal(got, want)
+    assert torch.isnan(ck[behind].float()).all() and torch.isnan(cv[behind].float()).all()
+
+
 def test_fused_decode_path_against_unfused():
     """Five-kernels-per-layer decode step vs the torch-glue step on the same
     model and cache: same cache rows for the first layer, logits within bf16
