@@ -1398,6 +1398,7 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
         const int cand[9][2] = {{4, 10}, {5, 8}, {4, 8}, {5, 10}, {4, 5}, {5, 5}, {4, 16}, {5, 16}, {4, 4}};
         int best = -1, best_cost = 1 << 30;
         for (int i = 0; i < 9; ++i) {
+            if (cand[i][0] * pl.rb > kMaxWaves) continue;  // a workgroup has at most 16 waves
             const int per_round = cand[i][0] * cand[i][1];
             const int rounds = (units + per_round - 1) / per_round;
             const int waste = rounds * per_round - units;
@@ -1448,7 +1449,7 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
         need = (nvec + 64 * pl.rb * pl.s - 1) / (64 * pl.rb * pl.s);
     }
     pl.vmax = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : 8));
-    pl.ok = need <= 8;
+    pl.ok = need <= 8 && pl.rb * pl.s <= kMaxWaves;
     return pl;
 }
 

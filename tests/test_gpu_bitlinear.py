@@ -257,6 +257,32 @@ def test_many_row_blocks_launch_shape(n, k, m):
     assert np.array_equal(qd.cpu().numpy(), q)
 
 
+@pytest.mark.parametrize("m", [1, 4])
+@pytest.mark.parametrize("n,k", [(23088, 21504), (16384, 8192), (17600, 27648)])
+def test_many_row_blocks_with_long_rows(n, k, m):
+    """N >= 16384 together with K >= 8192: four row blocks per workgroup leave
+    room for four waves per block only (a plan with five asked for 1280 threads
+    and the launch failed).  Accumulators against the integer product computed
+    on the device in fp64 (exact: |acc| < 2^53), drop-in product and forward
+    against each other bit for bit."""
+    g = torch.Generator(device="cuda").manual_seed(n + k + m)
+    w = torch.randint(-1, 2, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+    pk = pack_weight.convert_weight_int8_to_int2(w, keep_device=True)
+    want = (a.double() @ w.double().t()).to(torch.int32)
+    assert torch.equal(bitlinear.bitnet_int8xint2_acc(a, pk), want)
+    x = torch.randn(m, k, generator=g, device="cuda").to(torch.bfloat16)
+    ws = torch.tensor([0.0161, 0.0, 0.0, 0.0], device="cuda").to(torch.bfloat16)
+    mod = bitlinear.BitLinearKernel(k, n).cuda()
+    mod.weight.data, mod.weight_scale.data = pk, ws
+    q, s = bitlinear.quant_input(x)
+    y = bitlinear.bitnet_int8xint2_linear(q, pk, s.reshape(-1), ws)
+    assert torch.equal(mod(x).view(torch.int16), y.view(torch.int16))
+    acc = (q.double() @ w.double().t()).float()
+    want_y = (acc / s.float() * ws[0].float()).to(torch.bfloat16)
+    assert torch.equal(y.view(torch.int16), want_y.view(torch.int16))
+
+
 def _random_shape_cases(count=36, seed=20240611):
     rng = np.random.default_rng(seed)
     cases = []
