@@ -390,7 +390,9 @@ constexpr int kPfPieces = kPfChunk / 16;        // 16-byte pieces per row and ch
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 template <int MT, int NT, int KS>
-__global__ __launch_bounds__(kPfWaves * 64 * KS) void gemm_i2_prefill_kernel(
+__global__ __launch_bounds__(kPfWaves * 64 * KS)
+__attribute__((amdgpu_waves_per_eu(MT == 2 && NT == 2 && KS == 1 ? 3 : 1)))
+void gemm_i2_prefill_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
     ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K, int band, int cseg) {
@@ -487,15 +489,17 @@ __global__ __launch_bounds__(kPfWaves * 64 * KS) void gemm_i2_prefill_kernel(
     for (int i = 0; i < PPT; ++i) rs[i] = 0;
 
     // Software pipeline over the 256-k chunks.  Two register sets by chunk parity
-    // for the activation pieces (aE / aO) and for the weight words (wE / wO):
-    // set j & 1 holds chunk j.  While chunk c is multiplied out of LDS, the
-    // pieces of chunk c+1 move from their registers into the other LDS buffer
-    // and the same registers are at once re-requested for chunk c+3; a weight
-    // word is re-requested for chunk c+2 right after the MFMAs that consumed it.
-    // Every load so has two whole multiply phases to land and no register is
-    // ever copied (a copy would wait for the load it copies).
+    // for the activation pieces (aE / aO): set j & 1 holds chunk j.  While chunk c
+    // is multiplied out of LDS, the pieces of chunk c+1 move from their registers
+    // into the other LDS buffer and the same registers are at once re-requested
+    // for chunk c+3; no register is ever copied (a copy would wait for the load it
+    // copies).  The weight words have one set: a word is re-requested for chunk
+    // c+1 right after the MFMAs that consumed it and has most of a chunk to land.
+    // (A second set, words requested two chunks ahead, measured the same at every
+    // size; without it the 64 x 256 tile fits three waves per SIMD instead of two:
+    // a layer's four GEMMs 1.67 -> 1.81 POP/s at M = 4096, 1.50 -> 1.54 at M = 2048.)
     v4i aE[PPT], aO[PPT];
-    uint32_t wE[kPfSteps][NT], wO[kPfSteps][NT];
+    uint32_t wW[kPfSteps][NT];
     const v4i zero4 = {0, 0, 0, 0};
     const int ones = 0x01010101;
     const int last_step_off = (ksteps - 1) * 128;  // byte offset of the last 32-k step inside a row block
@@ -522,13 +526,9 @@ __global__ __launch_bounds__(kPfWaves * 64 * KS) void gemm_i2_prefill_kernel(
 #pragma unroll
     for (int ks = 0; ks < kPfSteps; ++ks)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wE[ks][nt] = load_word(0, ks, nt);
+        for (int nt = 0; nt < NT; ++nt) wW[ks][nt] = load_word(0, ks, nt);
 #pragma unroll
     for (int i = 0; i < PPT; ++i) aO[i] = load_piece(1, i);
-#pragma unroll
-    for (int ks = 0; ks < kPfSteps; ++ks)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wO[ks][nt] = load_word(1, ks, nt);
 #pragma unroll
     for (int i = 0; i < PPT; ++i) stage_piece(0, i, aE[i], lds_a);
 #pragma unroll
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(kPfWaves * 64 * KS) void gemm_i2_prefill_kernel(
                 if (slot == SLOTS - 1) {
                     // the words of this step were expanded during the previous one: re-request them
 #pragma unroll
-                    for (int j = 0; j < NT; ++j) wuse[ks][j] = load_word(c + 2, ks, j);
+                    for (int j = 0; j < NT; ++j) wuse[ks][j] = load_word(c + 1, ks, j);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -603,8 +603,8 @@ __global__ __launch_bounds__(kPfWaves * 64 * KS) void gemm_i2_prefill_kernel(
         lds_barrier();
     };
     for (int c = 0; c < nchunks; c += 2) {
-        chunk_body(c, wE, aO);
-        if (c + 1 < nchunks) chunk_body(c + 1, wO, aE);
+        chunk_body(c, wW, aO);
+        if (c + 1 < nchunks) chunk_body(c + 1, wW, aE);
     }
 
     // row sums: the kPfPieces (= 16) threads of one DPP row staged the pieces of one activation row
