@@ -488,17 +488,17 @@ void gemm_i2_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < PPT; ++i) rs[i] = 0;
 
-    // Software pipeline over the 256-k chunks.  Two register sets by chunk parity
-    // for the activation pieces (aE / aO): set j & 1 holds chunk j.  While chunk c
-    // is multiplied out of LDS, the pieces of chunk c+1 move from their registers
-    // into the other LDS buffer and the same registers are at once re-requested
-    // for chunk c+3; no register is ever copied (a copy would wait for the load it
-    // copies).  The weight words have one set: a word is re-requested for chunk
-    // c+1 right after the MFMAs that consumed it and has most of a chunk to land.
-    // (A second set, words requested two chunks ahead, measured the same at every
-    // size; without it the 64 x 256 tile fits three waves per SIMD instead of two:
+    // Software pipeline over the 256-k chunks, one register set per operand.
+    // While chunk c is multiplied out of LDS, the activation pieces of chunk c+1
+    // move from their registers (aP) into the other LDS buffer and the same
+    // registers are at once re-requested for chunk c+2; no register is ever
+    // copied (a copy would wait for the load it copies).  A weight word is
+    // re-requested for chunk c+1 right after the MFMAs that consumed it.  Either
+    // load has most of a chunk to land.  (Second sets requested a chunk further
+    // ahead measured the same or 1 % slower at every size; without the second
+    // set of words the 64 x 256 tile fits three waves per SIMD instead of two:
     // a layer's four GEMMs 1.67 -> 1.81 POP/s at M = 4096, 1.50 -> 1.54 at M = 2048.)
-    v4i aE[PPT], aO[PPT];
+    v4i aP[PPT];
     uint32_t wW[kPfSteps][NT];
     const v4i zero4 = {0, 0, 0, 0};
     const int ones = 0x01010101;
@@ -522,22 +522,20 @@ void gemm_i2_prefill_kernel(
     };
 
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) aE[i] = load_piece(0, i);
+    for (int i = 0; i < PPT; ++i) aP[i] = load_piece(0, i);
 #pragma unroll
     for (int ks = 0; ks < kPfSteps; ++ks)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wW[ks][nt] = load_word(0, ks, nt);
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) aO[i] = load_piece(1, i);
+    for (int i = 0; i < PPT; ++i) stage_piece(0, i, aP[i], lds_a);
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) stage_piece(0, i, aE[i], lds_a);
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) aE[i] = load_piece(2, i);
+    for (int i = 0; i < PPT; ++i) aP[i] = load_piece(1, i);
     lds_barrier();
 
     // Per k-step, besides its MFMAs: one slice of the staging of chunk c+1 (LDS
-    // write + row-sum), the reload of that slice's registers for chunk c+3, the
-    // reload of this step's weight words for chunk c+2, and the LDS reads of the
+    // write + row-sum), the reload of that slice's registers for chunk c+2, the
+    // reload of this step's weight words for chunk c+1, and the LDS reads of the
     // next step's A operands.  Spread like this the memory work issues in the
     // shadow of the MFMAs instead of stopping all four waves at once.  Nothing is
     // conditional: pieces at k >= K (ragged last chunk, or a whole chunk past the
@@ -589,7 +587,7 @@ void gemm_i2_prefill_kernel(
 #pragma unroll
                     for (int i = ks * PPT / kPfSteps; i < (ks + 1) * PPT / kPfSteps; ++i) {
                         stage_piece(c + 1, i, astage[i], sbuf);
-                        astage[i] = load_piece(c + 3, i);
+                        astage[i] = load_piece(c + 2, i);
                     }
                 }
                 if (slot == SLOTS - 1) {
@@ -602,10 +600,7 @@ void gemm_i2_prefill_kernel(
         }
         lds_barrier();
     };
-    for (int c = 0; c < nchunks; c += 2) {
-        chunk_body(c, wW, aO);
-        if (c + 1 < nchunks) chunk_body(c + 1, wW, aE);
-    }
+    for (int c = 0; c < nchunks; ++c) chunk_body(c, wW, aP);
 
     // row sums: the kPfPieces (= 16) threads of one DPP row staged the pieces of one activation row
 #pragma unroll
