@@ -395,7 +395,7 @@ __attribute__((amdgpu_waves_per_eu(MT == 2 && NT == 2 && KS == 1 ? 3 : 1)))
 void gemm_i2_prefill_kernel(
     const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K, int band, int cseg) {
+    ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K, int nunits, int cseg_shift) {
     constexpr int TM = MT * 32;
     constexpr int NTHR = kPfWaves * 64;
     constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
@@ -422,18 +422,16 @@ void gemm_i2_prefill_kernel(
     // operands through the memory-side cache on its own.  Unless the number of
     // bands is a multiple of 8, the column tiles are cut into segments too, so
     // that every XCD gets the same number of (band, segment) units.
+    // The grid spells the mapping out so that no division stands between the
+    // kernel's entry and its first load: x = XCD + 8 * (row tile within the
+    // band), y = column tile within the segment, z = round of 8 units (the
+    // linear workgroup id, which picks the XCD, is x + 8 * band * (y + ...)).
     const int row_tiles = (M + TM - 1) / TM;
     const int col_tiles = (N + kPfWaves * NT * 32 - 1) / (kPfWaves * NT * 32);
-    const int xcd = blockIdx.x & 7;
-    const int seq = blockIdx.x >> 3;
-    const int nbands = (row_tiles + band - 1) / band;
-    const int seg_cols = (col_tiles + cseg - 1) / cseg;  // few bands: the columns are cut into cseg segments as well
-    const int per_unit = band * seg_cols;
-    const int unit = xcd + 8 * (seq / per_unit);         // unit = (band, column segment) -> XCD unit % 8
-    if (unit >= nbands * cseg) return;
-    const int within = seq % per_unit;
-    const int col_tile = (unit % cseg) * seg_cols + within / band;
-    const int row_tile = (unit / cseg) * band + within % band;
+    const int unit = (blockIdx.x & 7) + 8 * blockIdx.z;  // unit = (band, column segment) -> XCD unit % 8
+    if (unit >= nunits) return;
+    const int col_tile = (unit & ((1 << cseg_shift) - 1)) * gridDim.y + blockIdx.y;
+    const int row_tile = (unit >> cseg_shift) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     if (row_tile >= row_tiles || col_tile >= col_tiles) return;  // ragged last band / segment (uniform over the workgroup)
     const int m0 = row_tile * TM;
     const int n0 = (col_tile * kPfWaves + wave) * NT * 32;
@@ -471,11 +469,11 @@ void gemm_i2_prefill_kernel(
         n = n < N ? n : N - 1;
         w_off[nt] = ((n >> 4) * K + ((n & 15) >> 3) * 16 + kc * 8 + (n & 7)) * 4;
     }
-    if (threadIdx.x < TM) {
-        const float sv = bf16_to_f32(out ? s[(m0 + tid) < M ? (m0 + tid) : (M - 1)] : (uint16_t)0x3f80);
-        sval[tid] = sv;
-        rinv[tid] = 1.0f / sv;
-    }
+    // the tokens' scales: requested here, ahead of everything else, and used (a division) only
+    // once the loads of the first chunks are on their way; without output there are no scales
+    // (the accumulator-only entry): the request then goes to an address that exists
+    const int s_row = (m0 + (tid & (TM - 1))) < M ? (m0 + (tid & (TM - 1))) : (M - 1);
+    const uint16_t s_raw = *(out ? s + s_row : (const uint16_t*)wq);
 
     v16i acc[MT][NT];
 #pragma unroll
@@ -531,6 +529,11 @@ void gemm_i2_prefill_kernel(
     for (int i = 0; i < PPT; ++i) stage_piece(0, i, aP[i], lds_a);
 #pragma unroll
     for (int i = 0; i < PPT; ++i) aP[i] = load_piece(1, i);
+    if (threadIdx.x < TM) {
+        const float sv = out ? bf16_to_f32(s_raw) : 1.0f;
+        sval[tid] = sv;
+        rinv[tid] = 1.0f / sv;
+    }
     lds_barrier();
 
     // Per k-step, besides its MFMAs: one slice of the staging of chunk c+1 (LDS
@@ -1554,7 +1557,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     if (g_tune_path == 5 && g_tune_prefill_ks > 0) ks = (tile == 4 || (tile == 0 && g_tune_prefill_ks == 2)) ? g_tune_prefill_ks : 1;
     if (K <= kPfChunk * (ks - 1)) ks = 1;  // fewer chunks than groups
     const dim3 block(kPfWaves * 64 * ks, 1, 1);
-    // 1-D grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
+    // grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
     // tiles, fewer when there are not enough row tiles to give every XCD a band
     const int tm = tile == 1 ? 128 : (tile == 4 ? 32 : 64);
     const int tn = (tile == 0 || tile == 4) ? 128 : (tile == 3 ? 512 : 256);
@@ -1569,14 +1572,18 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // than M = 128)
     int g8 = nbands & 7;
     g8 = g8 == 0 ? 8 : (g8 & -g8);  // gcd(nbands, 8)
-    int cseg = 8 / g8;
-    cseg = cseg > col_tiles ? col_tiles : cseg;
+    int cseg_shift = g8 == 8 ? 0 : (g8 == 4 ? 1 : (g8 == 2 ? 2 : 3));  // 8 / g8 segments, a power of two
+    while ((1 << cseg_shift) > col_tiles) --cseg_shift;
+    const int cseg = 1 << cseg_shift;
     const int seg_cols = (col_tiles + cseg - 1) / cseg;
     const int units = nbands * cseg;
-    const dim3 grid(8 * ((units + 7) / 8) * band * seg_cols, 1, 1);
+    // x = XCD + 8 * (row tile within the band), y = column tile within the segment, z = round of 8
+    // units: the same order of workgroups as a linear grid, without divisions in the kernel
+    if (seg_cols > 65535 || (units + 7) / 8 > 65535) return BITLINEAR_ERR_SHAPE;
+    const dim3 grid(8 * band, seg_cols, (units + 7) / 8);
 #define BITLINEAR_LAUNCH_PF(MT_, NT_, KS_)                                                                          \
     hipLaunchKernelGGL((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
-                       act, wq, out, acc_out, s, ws, smap, residual, M, N, K, band, cseg)
+                       act, wq, out, acc_out, s, ws, smap, residual, M, N, K, units, cseg_shift)
     if (tile == 4) {
         if (ks == 4) {
             BITLINEAR_LAUNCH_PF(1, 1, 4);
