@@ -33,6 +33,9 @@ HIPCC_FLAGS = [
     "-ffp-contract=off",
     # packed fp32 VALU forms are kept out of all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the leading kernel arguments arrive in registers at wave start instead of through scalar loads
+    # (a memory round trip in front of every kernel's first useful instruction otherwise)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 

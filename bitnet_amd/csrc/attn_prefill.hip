@@ -293,10 +293,14 @@ constexpr int kDfMaxWaves = 8;
 // the rope.
 template <int G, bool ROWS>
 __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
+    // parameter order: what the loads at the kernel's entry need comes first, in the leading dwords
+    // that arrive in registers at wave start (kernel-argument preload); `heads` = n_heads | n_kv_heads << 16
+    // and `shape` = splits | threads << 16 repeat the launch geometry, which is not among those dwords
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
-    const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    const float* __restrict__ rope_rows, uint16_t* __restrict__ out, float* workspace, int* counters, int S,
-    int n_heads, int n_kv_heads) {
+    const int64_t* __restrict__ positions, const float* __restrict__ rope_rows, int S, int heads, int shape, int B,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, uint16_t* __restrict__ out, float* workspace,
+    int* counters) {
+    const int n_heads = heads & 0xffff, n_kv_heads = heads >> 16;
     __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
     __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
     __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
@@ -306,10 +310,10 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nthreads = blockDim.x;
+    const int nthreads = shape >> 16;
     const int nwaves = nthreads >> 6;
     const int kvh = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
-    const int nsplit = gridDim.z;
+    const int nsplit = shape & 0xffff;
     const int c = lane & 15, g4 = lane >> 4;
     const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
     const uint16_t* row = qkv + (size_t)b * row_elems;
@@ -350,7 +354,7 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     }
     // the tag of this call's records: one more than the epoch the last merge of this (sequence, kv head)
     // left behind (an unconditional load: with one split there is no workspace and the value is unused)
-    const int* epochs = (const int*)(workspace + (size_t)gridDim.y * n_kv_heads * nsplit * G * kDfRecUnits * 2);
+    const int* epochs = (const int*)(workspace + (size_t)B * n_kv_heads * nsplit * G * kDfRecUnits * 2);
     const int epoch = *(nsplit > 1 ? epochs + (b * n_kv_heads + kvh) : (const int*)positions);
     v4u kb[2][4], vb[8];
     auto load_rows = [&](int blk) {  // cache rows 32 blk .. 32 blk + 31
@@ -606,8 +610,9 @@ int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint
     const int g = n_heads / n_kv_heads;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
 #define BITNET_DF_LAUNCH(GG, RR)                                                                                           \
-    hipLaunchKernelGGL((attn_decode_flash_kernel<GG, RR>), grid, block, 0, stream, qkv, cache_k, cache_v, positions, cos_table, \
-                       sin_table, rope_rows, out, workspace, counters, S, n_heads, n_kv_heads)
+    hipLaunchKernelGGL((attn_decode_flash_kernel<GG, RR>), grid, block, 0, stream, qkv, cache_k, cache_v, positions,       \
+                       rope_rows, S, n_heads | (n_kv_heads << 16), n_splits | (threads << 16), B, cos_table, sin_table, out, \
+                       workspace, counters)
 #define BITNET_DF_LAUNCH_G(GG)     \
     if (rope_rows)                 \
         BITNET_DF_LAUNCH(GG, true); \

@@ -121,9 +121,9 @@ constexpr int kDecodeMaxLdsBytes = 48 * 1024;
 
 template <int R>
 __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
-    const int8_t* __restrict__ act, const v4u* __restrict__ wq, uint16_t* __restrict__ out,
+    const int8_t* __restrict__ act, const v4u* __restrict__ wq, int M, int N, int K, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, int M, int N, int K) {
+    ScaleMap smap) {
     __shared__ int red[kDecodeMaxWaves * 256];
     extern __shared__ __attribute__((aligned(16))) int8_t lds_act[];  // [M][K]
 
@@ -247,9 +247,9 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
 // ---------------------------------------------------------------------------
 template <int UPW>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
-    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, uint16_t* __restrict__ out,
     int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K) {
+    ScaleMap smap, const uint16_t* __restrict__ residual) {
     __shared__ int red[kMaxWaves * 256];
 
     const int lane = threadIdx.x & 63;
@@ -393,9 +393,11 @@ template <int MT, int NT, int KS>
 __global__ __launch_bounds__(kPfWaves * 64 * KS)
 __attribute__((amdgpu_waves_per_eu(MT == 2 && NT == 2 && KS == 1 ? 3 : 1)))
 void gemm_i2_prefill_kernel(
-    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
-    int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, const uint16_t* __restrict__ residual, int M, int N, int K, int nunits, int cseg_shift) {
+    // parameter order: what the first loads need comes first (kernel-argument preload)
+    // (band and seg_cols repeat gridDim.x / 8 and gridDim.y: the grid's own size is not among the preloaded dwords)
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int nunits, int cseg_shift,
+    int band, int seg_cols, const uint16_t* __restrict__ s, uint16_t* __restrict__ out, int32_t* __restrict__ acc_out,
+    const uint16_t* __restrict__ ws, ScaleMap smap, const uint16_t* __restrict__ residual) {
     constexpr int TM = MT * 32;
     constexpr int NTHR = kPfWaves * 64;
     constexpr int PPT = TM * kPfPieces / NTHR;  // pieces of a chunk per thread
@@ -430,8 +432,8 @@ void gemm_i2_prefill_kernel(
     const int col_tiles = (N + kPfWaves * NT * 32 - 1) / (kPfWaves * NT * 32);
     const int unit = (blockIdx.x & 7) + 8 * blockIdx.z;  // unit = (band, column segment) -> XCD unit % 8
     if (unit >= nunits) return;
-    const int col_tile = (unit & ((1 << cseg_shift) - 1)) * gridDim.y + blockIdx.y;
-    const int row_tile = (unit >> cseg_shift) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int col_tile = (unit & ((1 << cseg_shift) - 1)) * seg_cols + blockIdx.y;
+    const int row_tile = (unit >> cseg_shift) * band + (blockIdx.x >> 3);
     if (row_tile >= row_tiles || col_tile >= col_tiles) return;  // ragged last band / segment (uniform over the workgroup)
     const int m0 = row_tile * TM;
     const int n0 = (col_tile * kPfWaves + wave) * NT * 32;
@@ -1005,9 +1007,13 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
 // its own, because loads under a runtime branch would make the compiler wait conservatively later)
 template <int UPW, int VMAX, int PRO, bool RES>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
-    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, uint16_t* __restrict__ out,
+    // parameter order: what stands between the kernel's entry and its first loads comes first, in
+    // the leading dwords that are handed over in registers at wave start (kernel-argument preload)
+    // (aux: the second thing the prologue loads -- ex.norm_weight for PRO 1 and 2, ex.act_scale for PRO 3)
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, int mode,
+    float inv_vec_per_row, const uint16_t* __restrict__ aux, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
-    FusedExtras ex, int M, int N, int K, int RB, int S, int mode, float inv_vec_per_row) {
+    FusedExtras ex) {
     extern __shared__ __attribute__((aligned(16))) int8_t lds_q[];  // [M][K + pad]
     __shared__ int red[kFusedMaxRB * 256];
     __shared__ uint32_t amax_bits[kFusedMaxTokens];
@@ -1075,10 +1081,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         } else {
             xv[v] = *(const uint4*)(x + idx * 8);                            // rows are contiguous
         }
-        if (PRO == 1 || PRO == 2) gv[v] = *(const uint4*)(ex.norm_weight + col * 8);
+        if (PRO == 1 || PRO == 2) gv[v] = *(const uint4*)(aux + col * 8);
     }
     // PRO 3: the scale of token row tid, raw bits; any other variant re-reads a weight scale and ignores it
-    const uint16_t* asp = PRO == 3 ? ex.act_scale : ws;
+    const uint16_t* asp = PRO == 3 ? aux : ws;
     const uint16_t e_as = asp[PRO == 3 ? (tid < M ? tid : M - 1) : 0];
     // weight words of the first round
     uint32_t w[UPW];
@@ -1323,7 +1329,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     const dim3 block(waves * 64, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
 #define BITLINEAR_LAUNCH(U)                                                                                  \
-    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, out, acc_out, s, ws, smap, residual, M, N, K)
+    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, M, N, K, out, acc_out, s, ws, smap, residual)
     switch (upw) {
         case 1: BITLINEAR_LAUNCH(1); break;
         case 2: BITLINEAR_LAUNCH(2); break;
@@ -1345,7 +1351,7 @@ int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     const size_t lds = (size_t)M * K;
     const v4u* wq = (const v4u*)packed;
 #define BITLINEAR_LAUNCH(R)                                                                                     \
-    hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, out, acc_out, s, ws, smap, M, N, K)
+    hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, M, N, K, out, acc_out, s, ws, smap)
     // R steps (1 KB each per wave) per round, two rounds in flight
     if (steps <= 4) BITLINEAR_LAUNCH(2);
     else if (steps <= 10) BITLINEAR_LAUNCH(5);
@@ -1475,8 +1481,9 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     const int pro = ex.act_scale ? 3 : (ex.norm_weight ? (ex.glu ? 2 : 1) : 0);
     if (pro == 0 && ex.residual) return BITLINEAR_ERR_ARG;  // the plain forward has no residual epilogue
 #define BITLINEAR_LAUNCH_UVPR(U, V, P, R)                                                                            \
-    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P, R>), grid, block, lds, stream, x, wq, out, ws, smap, q_out, \
-                       s_out, ex, M, N, K, pl.rb, pl.s, mode, 1.0f / (float)(K / (pro == 3 ? 16 : 8)))
+    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P, R>), grid, block, lds, stream, x, wq, M, N, K, pl.rb, pl.s,  \
+                       mode, 1.0f / (float)(K / (pro == 3 ? 16 : 8)), pro == 3 ? ex.act_scale : ex.norm_weight, out, ws, \
+                       smap, q_out, s_out, ex)
 #define BITLINEAR_LAUNCH_UVP(U, V, P)              \
     if (ex.residual)                               \
         BITLINEAR_LAUNCH_UVPR(U, V, P, true);      \
@@ -1583,7 +1590,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const dim3 grid(8 * band, seg_cols, (units + 7) / 8);
 #define BITLINEAR_LAUNCH_PF(MT_, NT_, KS_)                                                                          \
     hipLaunchKernelGGL((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
-                       act, wq, out, acc_out, s, ws, smap, residual, M, N, K, units, cseg_shift)
+                       act, wq, M, N, K, units, cseg_shift, band, seg_cols, s, out, acc_out, ws, smap, residual)
     if (tile == 4) {
         if (ks == 4) {
             BITLINEAR_LAUNCH_PF(1, 1, 4);
