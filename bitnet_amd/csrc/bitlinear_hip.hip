@@ -121,15 +121,14 @@ constexpr int kDecodeMaxLdsBytes = 48 * 1024;
 
 template <int R>
 __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
-    const int8_t* __restrict__ act, const v4u* __restrict__ wq, int M, int N, int K, uint16_t* __restrict__ out,
-    int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap) {
+    const int8_t* __restrict__ act, const v4u* __restrict__ wq, int M, int N, int K, int nwaves,
+    uint16_t* __restrict__ out, int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s,
+    const uint16_t* __restrict__ ws, ScaleMap smap) {
     __shared__ int red[kDecodeMaxWaves * 256];
     extern __shared__ __attribute__((aligned(16))) int8_t lds_act[];  // [M][K]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int nwaves = blockDim.x >> 6;
     const int rb = blockIdx.x * nwaves + wave;  // 16-row block of this wave
     const bool rows_ok = rb < (N >> 4);
     const int g = lane >> 4;
@@ -202,7 +201,7 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
     {
         // activations -> LDS while the weight loads are in flight
         const int nvec = (M * K) >> 4;
-        for (int i = threadIdx.x; i < nvec; i += blockDim.x)
+        for (int i = threadIdx.x; i < nvec; i += nwaves * 64)
             *(v4i*)(lds_act + (size_t)i * 16) = *(const v4i*)(act + (size_t)i * 16);
         lds_barrier();
     }
@@ -247,14 +246,13 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
 // ---------------------------------------------------------------------------
 template <int UPW>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
-    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, uint16_t* __restrict__ out,
-    int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws,
-    ScaleMap smap, const uint16_t* __restrict__ residual) {
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int nwaves,
+    uint16_t* __restrict__ out, int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s,
+    const uint16_t* __restrict__ ws, ScaleMap smap, const uint16_t* __restrict__ residual) {
     __shared__ int red[kMaxWaves * 256];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int nwaves = blockDim.x >> 6;
     const int g = lane >> 4;  // which 16 of the step's 64 k
     const int p = lane & 15;  // weight row (A operand) / token (B operand)
     const int nb = blockIdx.x;
@@ -266,20 +264,6 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     const uint32_t* wrow = wq + (size_t)nb * K + lane_word;
     const bool tok_ok = (m0 + p) < M;
     const int8_t* arow = act + (size_t)(tok_ok ? (m0 + p) : 0) * K + g * 16;
-
-    // The thread that will finish output (row, token) fetches its two scales
-    // now, as raw bits with nothing depending on them until the epilogue, so
-    // their latency overlaps the weight stream instead of preceding or
-    // following it.  Indices are clamped so every thread may load.
-    const int e_lane = threadIdx.x & 63;
-    const int e_m = m0 + (e_lane & 15);
-    const int e_n = nb * 16 + 4 * (e_lane >> 4) + ((threadIdx.x >> 6) & 3);
-    uint16_t e_sb = 0, e_wsb = 0, e_res = 0;
-    if (out) {
-        e_sb = s[e_m < M ? e_m : M - 1];
-        e_wsb = ws[scale_slot(smap, e_n)];
-        if (residual) e_res = residual[(size_t)(e_m < M ? e_m : M - 1) * N + e_n];
-    }
 
     v4i acc_q = {0, 0, 0, 0};
     v4i acc_b = {0, 0, 0, 0};
@@ -317,6 +301,22 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     const int base0 = wave * UPW;
     load_round(w0, b0, base0);
     if (base0 + stride < units) load_round(w1, b1, base0 + stride);
+
+    // The thread that will finish output (row, token) fetches its two scales
+    // now -- behind the first weight requests, which need nothing but
+    // arguments that arrive in registers, while the scale map and these
+    // pointers come through a scalar load -- as raw bits with nothing
+    // depending on them until the epilogue, so their latency overlaps the
+    // weight stream.  Indices are clamped so every thread may load.
+    const int e_lane = threadIdx.x & 63;
+    const int e_m = m0 + (e_lane & 15);
+    const int e_n = nb * 16 + 4 * (e_lane >> 4) + ((threadIdx.x >> 6) & 3);
+    uint16_t e_sb = 0, e_wsb = 0, e_res = 0;
+    if (out) {
+        e_sb = s[e_m < M ? e_m : M - 1];
+        e_wsb = ws[scale_slot(smap, e_n)];
+        if (residual) e_res = residual[(size_t)(e_m < M ? e_m : M - 1) * N + e_n];
+    }
     for (int base = base0; base < units; base += 2 * stride) {
         use_round(w0, b0, base);
         if (base + 2 * stride < units) load_round(w0, b0, base + 2 * stride);
@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
     my[192] = acc_q.w + acc_b.w;
     __syncthreads();
 
-    if (blockDim.x >= 256) {
+    if (nwaves >= 4) {
         if (threadIdx.x < 256 && e_m < M) {
             int part[kMaxWaves];  // independent LDS reads, one wait
 #pragma unroll
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_mfma_kernel(
         return;
     }
     // fewer than four waves: every thread finishes several outputs
-    for (int t = threadIdx.x; t < 256; t += blockDim.x) {
+    for (int t = threadIdx.x; t < 256; t += nwaves * 64) {
         const int l = t & 63;
         const int m = m0 + (l & 15);
         if (m >= M) continue;
@@ -432,6 +432,8 @@ void gemm_i2_prefill_kernel(
     const int col_tiles = (N + kPfWaves * NT * 32 - 1) / (kPfWaves * NT * 32);
     const int unit = (blockIdx.x & 7) + 8 * blockIdx.z;  // unit = (band, column segment) -> XCD unit % 8
     if (unit >= nunits) return;
+    const bool has_out = (cseg_shift >> 8) != 0;  // bit 8 repeats out != nullptr (out itself is not among the preloaded dwords)
+    cseg_shift &= 0xff;
     const int col_tile = (unit & ((1 << cseg_shift) - 1)) * seg_cols + blockIdx.y;
     const int row_tile = (unit >> cseg_shift) * band + (blockIdx.x >> 3);
     if (row_tile >= row_tiles || col_tile >= col_tiles) return;  // ragged last band / segment (uniform over the workgroup)
@@ -475,7 +477,7 @@ void gemm_i2_prefill_kernel(
     // once the loads of the first chunks are on their way; without output there are no scales
     // (the accumulator-only entry): the request then goes to an address that exists
     const int s_row = (m0 + (tid & (TM - 1))) < M ? (m0 + (tid & (TM - 1))) : (M - 1);
-    const uint16_t s_raw = *(out ? s + s_row : (const uint16_t*)wq);
+    const uint16_t s_raw = *(has_out ? s + s_row : (const uint16_t*)wq);
 
     v16i acc[MT][NT];
 #pragma unroll
@@ -532,7 +534,7 @@ void gemm_i2_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < PPT; ++i) aP[i] = load_piece(1, i);
     if (threadIdx.x < TM) {
-        const float sv = out ? bf16_to_f32(s_raw) : 1.0f;
+        const float sv = has_out ? bf16_to_f32(s_raw) : 1.0f;
         sval[tid] = sv;
         rinv[tid] = 1.0f / sv;
     }
@@ -1027,7 +1029,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
     // in front of the first load is kept short: wave-uniform values on the scalar unit, no integer
     // division, no 64-bit address arithmetic.
     const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
+    // = blockDim.x; where the prologue needs it early (more than one vector per thread) it is taken
+    // from arguments that arrive in registers instead of from the hidden arguments (a scalar load)
+    const int nthreads = VMAX == 1 ? (int)blockDim.x : 64 * RB * S;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int rbl = (wave >= S ? 1 : 0) + (wave >= 2 * S ? 1 : 0) + (wave >= 3 * S ? 1 : 0);  // wave / S, RB <= 4
@@ -1329,7 +1333,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     const dim3 block(waves * 64, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
 #define BITLINEAR_LAUNCH(U)                                                                                  \
-    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, M, N, K, out, acc_out, s, ws, smap, residual)
+    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, M, N, K, waves, out, acc_out, s, ws, smap, residual)
     switch (upw) {
         case 1: BITLINEAR_LAUNCH(1); break;
         case 2: BITLINEAR_LAUNCH(2); break;
@@ -1351,7 +1355,7 @@ int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     const size_t lds = (size_t)M * K;
     const v4u* wq = (const v4u*)packed;
 #define BITLINEAR_LAUNCH(R)                                                                                     \
-    hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, M, N, K, out, acc_out, s, ws, smap)
+    hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, M, N, K, waves, out, acc_out, s, ws, smap)
     // R steps (1 KB each per wave) per round, two rounds in flight
     if (steps <= 4) BITLINEAR_LAUNCH(2);
     else if (steps <= 10) BITLINEAR_LAUNCH(5);
@@ -1590,7 +1594,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const dim3 grid(8 * band, seg_cols, (units + 7) / 8);
 #define BITLINEAR_LAUNCH_PF(MT_, NT_, KS_)                                                                          \
     hipLaunchKernelGGL((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
-                       act, wq, M, N, K, units, cseg_shift, band, seg_cols, s, out, acc_out, ws, smap, residual)
+                       act, wq, M, N, K, units, cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual)
     if (tile == 4) {
         if (ks == 4) {
             BITLINEAR_LAUNCH_PF(1, 1, 4);
