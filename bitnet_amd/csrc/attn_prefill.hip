@@ -294,13 +294,14 @@ constexpr int kDfMaxWaves = 8;
 template <int G, bool ROWS>
 __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     // parameter order: what the loads at the kernel's entry need comes first, in the leading dwords
-    // that arrive in registers at wave start (kernel-argument preload); `heads` = n_heads | n_kv_heads << 16
-    // and `shape` = splits | threads << 16 repeat the launch geometry, which is not among those dwords
+    // that arrive in registers at wave start (kernel-argument preload).  `epochs` is the epoch array
+    // inside the workspace (any readable address with one split); `shape` = n_heads | n_kv_heads << 8 |
+    // splits << 16 | waves << 24 repeats the launch geometry, which is not among those dwords
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
-    const int64_t* __restrict__ positions, const float* __restrict__ rope_rows, int S, int heads, int shape, int B,
+    const int64_t* __restrict__ positions, const float* __restrict__ rope_rows, int* epochs, int S, int shape,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, uint16_t* __restrict__ out, float* workspace,
     int* counters) {
-    const int n_heads = heads & 0xffff, n_kv_heads = heads >> 16;
+    const int n_heads = shape & 0xff, n_kv_heads = (shape >> 8) & 0xff;
     __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
     __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
     __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
@@ -310,10 +311,15 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nthreads = shape >> 16;
-    const int nwaves = nthreads >> 6;
+    const int nwaves = (shape >> 24) & 0xff;
+    const int nthreads = nwaves * 64;
     const int kvh = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
-    const int nsplit = shape & 0xffff;
+    const int nsplit = (shape >> 16) & 0xff;
+    // two scalar requests from preloaded pointers, under way before anything else: the position, and
+    // the tag of this call's records -- one more than the epoch the last merge of this (sequence, kv
+    // head) left behind (with one split the value is unused)
+    const int64_t p_raw = positions[b];
+    const int epoch = epochs[nsplit > 1 ? b * n_kv_heads + kvh : 0];
     const int c = lane & 15, g4 = lane >> 4;
     const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
     const uint16_t* row = qkv + (size_t)b * row_elems;
@@ -352,10 +358,6 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
             rsn[u] = rope_rows[(size_t)b * kHeadDim + kHeadDim / 2 + i];
         }
     }
-    // the tag of this call's records: one more than the epoch the last merge of this (sequence, kv head)
-    // left behind (an unconditional load: with one split there is no workspace and the value is unused)
-    const int* epochs = (const int*)(workspace + (size_t)B * n_kv_heads * nsplit * G * kDfRecUnits * 2);
-    const int epoch = *(nsplit > 1 ? epochs + (b * n_kv_heads + kvh) : (const int*)positions);
     v4u kb[2][4], vb[8];
     auto load_rows = [&](int blk) {  // cache rows 32 blk .. 32 blk + 31
         const int base = blk * 32 * row_bytes;
@@ -370,7 +372,6 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
             vb[jj] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, base + ((jj & 3) + (jj >> 2) * 16 + 4 * g4) * row_bytes + c * 16, 0, 0);
     };
     load_rows(blk0);
-    const int64_t p_raw = positions[b];
     const int p = __builtin_amdgcn_readfirstlane(p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw));  // clamped into the cache
     const int pblk = p >> 5;                        // the block of the new token's row
     const bool owns_new = pblk % nsplit == sp;
@@ -596,7 +597,7 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
         *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
     }
     __syncthreads();  // every wave has read its records
-    if (tid == 0) ((int*)epochs)[b * n_kv_heads + kvh] = epoch + 1;
+    if (tid == 0) epochs[b * n_kv_heads + kvh] = epoch + 1;
 }
 
 }  // namespace
@@ -608,11 +609,14 @@ int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint
                                     float* workspace, int* counters, int n_splits, int threads, int B, int S,
                                     int n_heads, int n_kv_heads, hipStream_t stream) {
     const int g = n_heads / n_kv_heads;
+    if (n_heads > 255 || n_splits > 255 || threads > 64 * 255) return 1;  // packed into one kernel argument
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
+    // the epoch array follows the splits' records in the workspace
+    int* epochs = n_splits > 1 ? (int*)(workspace + (size_t)B * n_kv_heads * n_splits * g * kDfRecUnits * 2) : (int*)positions;
 #define BITNET_DF_LAUNCH(GG, RR)                                                                                           \
     hipLaunchKernelGGL((attn_decode_flash_kernel<GG, RR>), grid, block, 0, stream, qkv, cache_k, cache_v, positions,       \
-                       rope_rows, S, n_heads | (n_kv_heads << 16), n_splits | (threads << 16), B, cos_table, sin_table, out, \
-                       workspace, counters)
+                       rope_rows, epochs, S, n_heads | (n_kv_heads << 8) | (n_splits << 16) | ((threads / 64) << 24),        \
+                       cos_table, sin_table, out, workspace, counters)
 #define BITNET_DF_LAUNCH_G(GG)     \
     if (rope_rows)                 \
         BITNET_DF_LAUNCH(GG, true); \
