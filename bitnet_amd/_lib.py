@@ -18,6 +18,11 @@ SIGNATURES = {
     "bitlinear_last_status": (_c_int, []),
     "bitlinear_status_string": (ctypes.c_char_p, [_c_int]),
     "bitlinear_ws_num": (_c_int, [_c_int, _c_int]),
+    "bitlinear_last_kernel": (ctypes.c_char_p, []),
+    "bitlinear_forward_bf16_acc_i32": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "bitlinear_int8xint2_acc_i32": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -51,6 +56,8 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
     "bitnet_attn_decode_workspace_floats": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
+    "bitnet_attn_decode_error_index": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
+    "bitnet_attn_decode_set_spin_limit": (_c_int, [_c_int]),
     "bitnet_attn_prefill": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],

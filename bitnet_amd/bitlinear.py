@@ -69,6 +69,8 @@ def bitnet_int8xint2_linear(input0, input1, s, ws, out=None):
         raise ValueError("weight_scale has fewer slots than this shape uses")
     if out is None:
         out = torch.empty(*out_shape, dtype=torch.bfloat16, device=input0.device)
+    elif out.dtype != torch.bfloat16 or out.numel() != M * N or not out.is_contiguous() or not out.is_cuda:
+        raise ValueError("out must be a contiguous bfloat16 GPU tensor of M x N elements")
     if M == 0:
         return out  # no token rows: nothing to launch
     lib.bitlinear_int8xint2(_ptr(input0), _ptr(input1), _ptr(out), _ptr(s), _ptr(ws), M, N, K, _stream_ptr())
@@ -79,9 +81,13 @@ def bitnet_int8xint2_linear(input0, input1, s, ws, out=None):
 def bitnet_int8xint2_acc(input0, input1):
     """Raw int32 accumulators [..., N] of the same product (test/debug)."""
     _check_device(input0, input1)
+    if input0.dtype != torch.int8 or input1.dtype != torch.int8:
+        raise TypeError("input0 and input1 must be int8")
     M = _flat_rows(input0)
     N = input1.shape[0]
     K = input1.shape[1] * 4
+    if input0.shape[-1] != K:
+        raise ValueError(f"activation width {input0.shape[-1]} does not match packed weight K={K}")
     acc = torch.empty(*input0.shape[:-1], N, dtype=torch.int32, device=input0.device)
     if M == 0:
         return acc
@@ -91,16 +97,60 @@ def bitnet_int8xint2_acc(input0, input1):
     return acc
 
 
+def bitlinear_forward_acc(input, weight, weight_scale, mode: int = QUANT_COMPILED):
+    """BitLinearKernel.forward through bitlinear_forward_bf16_acc_i32: the bf16
+    output [..., N] together with the int32 accumulators of its product (test/debug)."""
+    _check_device(input, weight, weight_scale)
+    if input.dtype != torch.bfloat16 or weight.dtype != torch.int8 or weight_scale.dtype != torch.bfloat16:
+        raise TypeError("expected bfloat16 activations, int8 packed weight, bfloat16 weight scales")
+    M = _flat_rows(input)
+    N = weight.shape[0]
+    K = weight.shape[1] * 4
+    if input.shape[-1] != K:
+        raise ValueError(f"activation width {input.shape[-1]} does not match packed weight K={K}")
+    lib = _lib.load_library()
+    if weight_scale.numel() < lib.bitlinear_ws_num(N, K):
+        raise ValueError("weight_scale has fewer slots than this shape uses")
+    out = torch.empty(*input.shape[:-1], N, dtype=torch.bfloat16, device=input.device)
+    acc = torch.empty(*input.shape[:-1], N, dtype=torch.int32, device=input.device)
+    if M == 0:
+        return out, acc
+    q = torch.empty(M, K, dtype=torch.int8, device=input.device)
+    s = torch.empty(M, dtype=torch.bfloat16, device=input.device)
+    st = lib.bitlinear_forward_bf16_acc_i32(
+        _ptr(input), _ptr(weight), _ptr(acc), _ptr(out), _ptr(weight_scale), _ptr(q), _ptr(s), M, N, K, mode, _stream_ptr()
+    )
+    _lib.check(st, f"bitlinear_forward_bf16_acc_i32(M={M}, N={N}, K={K})")
+    return out, acc
+
+
+def last_kernel() -> str:
+    """Name of the product kernel the calling thread's last library call launched."""
+    return _lib.load_library().bitlinear_last_kernel().decode()
+
+
 def bitnet_int8xint2_linear_seg(input0, input1, s, ws, seg_ends, out=None):
     """Like bitnet_int8xint2_linear but row n takes ws[j] of the segment
     [seg_ends[j-1], seg_ends[j]) it lies in -- the scale layout
     gpu/convert_checkpoint.py:42-77 writes for fused wqkv / w13."""
     _check_device(input0, input1, s, ws)
+    if input0.dtype != torch.int8 or input1.dtype != torch.int8:
+        raise TypeError("input0 and input1 must be int8")
+    if s.dtype != torch.bfloat16 or ws.dtype != torch.bfloat16:
+        raise TypeError("s and ws must be bfloat16")
     M = _flat_rows(input0)
     N = input1.shape[0]
     K = input1.shape[1] * 4
+    if input0.shape[-1] != K:
+        raise ValueError(f"activation width {input0.shape[-1]} does not match packed weight K={K}")
+    if s.numel() < M:
+        raise ValueError(f"need one activation scale per row: {s.numel()} < {M}")
+    if ws.numel() < len(seg_ends):
+        raise ValueError("weight_scale has fewer slots than there are segments")
     if out is None:
         out = torch.empty(*input0.shape[:-1], N, dtype=torch.bfloat16, device=input0.device)
+    elif out.dtype != torch.bfloat16 or out.numel() != M * N or not out.is_contiguous() or not out.is_cuda:
+        raise ValueError("out must be a contiguous bfloat16 GPU tensor of M x N elements")
     if M == 0:
         return out
     ends = (ctypes.c_int * len(seg_ends))(*[int(e) for e in seg_ends])
@@ -155,6 +205,12 @@ class BitLinearKernel(nn.Module):
 
     def forward(self, input):
         _check_device(input, self.weight, self.weight_scale)
+        if input.dtype != torch.bfloat16:
+            raise TypeError("BitLinearKernel.forward expects bfloat16 activations")
+        if input.shape[-1] != self.in_features:
+            raise ValueError(f"activation width {input.shape[-1]} does not match in_features={self.in_features}")
+        if self.weight.shape != (self.out_features, self.in_features // 4) or self.weight.dtype != torch.int8:
+            raise ValueError("weight must be int8 [out_features, in_features // 4] (the packed layout)")
         M = _flat_rows(input)
         N, K = self.out_features, self.in_features
         q = torch.empty(input.shape, dtype=torch.int8, device=input.device)

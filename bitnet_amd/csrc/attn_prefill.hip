@@ -283,7 +283,7 @@ __global__ __launch_bounds__(64 * G) void attn_prefill_kernel(
 // LDS once.  No score buffer, no barrier between scores, softmax and P.V.
 constexpr int kDfRecUnits = kHeadDim + 2;  // record of one (sequence, kv head, split, head): 128 outputs, maximum, sum,
                                             // each an 8-byte unit (value, tag of the call that wrote it)
-constexpr int kDfSpinLimit = 1 << 16;       // polls of the merging workgroup before it gives up (never reached: see below)
+constexpr int kDfSpinLimit = 1 << 16;       // polls of the merging workgroup before it gives up (see the merge below)
 constexpr int kDfMaxSplits = 16;
 constexpr int kDfMaxWaves = 8;
 
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
     const int64_t* __restrict__ positions, const float* __restrict__ rope_rows, int* epochs, int S, int shape,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, uint16_t* __restrict__ out, float* workspace,
-    int* counters) {
+    int* err_word, int spin_limit) {
     const int n_heads = shape & 0xff, n_kv_heads = (shape >> 8) & 0xff;
     __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
     __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
@@ -550,15 +550,23 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
     if (!merger) return;
 
     // The merge, eight splits at a time: all units of a batch are requested together and requested
-    // again while one of them still carries an older tag.  The poll ends: every split polled has
-    // started before this workgroup and writes its record without waiting for anything.  (The limit
-    // only keeps a wrongly initialised workspace from hanging the GPU.)
+    // again while one of them still carries an older tag.  Every split polled was dispatched before
+    // this workgroup and writes its record without waiting for anything, so the poll is expected to
+    // end after a few rounds; that order of dispatch is observed behaviour, not something the
+    // hardware promises, and a workspace that was not zero before its first use breaks the tags.  The
+    // poll is therefore bounded, and a poll that runs out is not papered over: the head's output row
+    // becomes NaN and the workspace's error word is set (it stays set; the host reads it, see
+    // bitnet_attn_decode_error_index).
     constexpr int kBatch = 8;
     for (int hh = wave; hh < G; hh += nwaves) {
         float mx = -INFINITY, l = 0.0f, o0 = 0.0f, o1 = 0.0f;
+        bool gave_up = false;
         for (int k0 = 0; k0 < nact; k0 += kBatch) {
             unsigned long long um[kBatch], ul[kBatch], u0[kBatch], u1[kBatch];
-            for (int spin = 0; spin < kDfSpinLimit; ++spin) {
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k) um[k] = ul[k] = u0[k] = u1[k] = 0ull;
+            bool complete = false;
+            for (int spin = 0; spin < spin_limit; ++spin) {
                 bool ok = true;
 #pragma unroll
                 for (int k = 0; k < kBatch; ++k) {
@@ -571,8 +579,12 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
 #pragma unroll
                 for (int k = 0; k < kBatch; ++k)
                     ok = ok && ((um[k] & ul[k] & u0[k] & u1[k]) >> 32) == (tag >> 32) && ((um[k] | ul[k] | u0[k] | u1[k]) >> 32) == (tag >> 32);
-                if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+                if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+                    complete = true;
+                    break;
+                }
             }
+            gave_up = gave_up || !complete;
             float bm = mx;
 #pragma unroll
             for (int k = 0; k < kBatch; ++k)
@@ -593,8 +605,9 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
                 }
             }
         }
-        const float is = 1.0f / l;
+        const float is = gave_up ? __builtin_nanf("") : 1.0f / l;
         *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
+        if (gave_up && lane == 0) __hip_atomic_store(err_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();  // every wave has read its records
     if (tid == 0) epochs[b * n_kv_heads + kvh] = epoch + 1;
@@ -607,16 +620,20 @@ __global__ __launch_bounds__(kDfMaxWaves * 64) void attn_decode_flash_kernel(
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
                                     const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
                                     float* workspace, int* counters, int n_splits, int threads, int B, int S,
-                                    int n_heads, int n_kv_heads, hipStream_t stream) {
+                                    int n_heads, int n_kv_heads, int spin_limit, hipStream_t stream) {
+    (void)counters;  // the arrival counters belong to the other kernel
     const int g = n_heads / n_kv_heads;
     if (n_heads > 255 || n_splits > 255 || threads > 64 * 255) return 1;  // packed into one kernel argument
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
     // the epoch array follows the splits' records in the workspace
     int* epochs = n_splits > 1 ? (int*)(workspace + (size_t)B * n_kv_heads * n_splits * g * kDfRecUnits * 2) : (int*)positions;
+    // the error word follows the epochs (with one split nothing is merged and nothing can fail)
+    int* err_word = n_splits > 1 ? epochs + (size_t)B * n_kv_heads : nullptr;
+    if (spin_limit < 0) spin_limit = kDfSpinLimit;
 #define BITNET_DF_LAUNCH(GG, RR)                                                                                           \
     hipLaunchKernelGGL((attn_decode_flash_kernel<GG, RR>), grid, block, 0, stream, qkv, cache_k, cache_v, positions,       \
                        rope_rows, epochs, S, n_heads | (n_kv_heads << 8) | (n_splits << 16) | ((threads / 64) << 24),        \
-                       cos_table, sin_table, out, workspace, counters)
+                       cos_table, sin_table, out, workspace, err_word, spin_limit)
 #define BITNET_DF_LAUNCH_G(GG)     \
     if (rope_rows)                 \
         BITNET_DF_LAUNCH(GG, true); \

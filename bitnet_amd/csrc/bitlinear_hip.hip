@@ -21,11 +21,13 @@
 // epilogue (gpu/bitnet_kernels/bitnet_kernels.h:79-82) is applied.
 
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <type_traits>
 #include <stdint.h>
 #include <stdio.h>
 
 #include "bitlinear_hip.h"
+#include "host_util.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
@@ -860,6 +862,7 @@ struct FusedExtras {
     float eps;
     int glu;                      // 1: x is [M, 2K] = (x1 | x3); h = bf16(bf16(relu(x1)^2) * x3) feeds the norm
     const uint16_t* act_scale;    // PRO 3 only: bf16 [M], the scales of the int8 rows handed in as x
+    int32_t* acc_out;             // int32 [M, N] or nullptr: the raw accumulators (parity tests)
 };
 
 __device__ __forceinline__ double dpp_sum_f64_row(double v) {
@@ -1263,13 +1266,15 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
         if (m < M && n < N) {
             uint16_t wsb = wsb_first;
             if (slot_first != slot_last) wsb = ws[scale_slot(smap, n)];  // uniform branch, rare
-            const float a = (float)(red[t] - 2 * qsum[m]);
+            const int acc_i = red[t] - 2 * qsum[m];
+            if (ex.acc_out) ex.acc_out[(size_t)m * N + n] = acc_i;  // uniform branch: parity tests only
+            const float a = (float)acc_i;
             const float sv = sval[m], ri = rinv[m];
             const float q0 = a * ri;
             const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
             uint16_t o = f32_to_bf16_rne(q * bf16_to_f32(wsb));
             if (kHasRes) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
-            out[(size_t)m * N + n] = o;
+            if (out) out[(size_t)m * N + n] = o;  // uniform: the accumulator-only call has no output
         }
     }
 }
@@ -1278,15 +1283,33 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
 // host side
 // ---------------------------------------------------------------------------
 thread_local int g_status = BITLINEAR_OK;
-int g_tune_waves = 0;
-int g_tune_upw = 0;
-int g_tune_decode_waves = 0;
-int g_tune_path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse
-int g_tune_fused[3] = {1, 10, 4};
-int g_tune_prefill_big = 0;
-int g_tune_prefill_band = 0;  // row tiles per band of the prefill GEMM's tile order, 0 = built-in choice
-int g_tune_prefill_ks = 0;    // groups of waves splitting K in the small prefill tiles, 0 = built-in choice
-int g_tune_staged = 0;  // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
+// name of the product kernel the calling thread's most recent call launched (tests and the smoke
+// check report which kernel they exercised)
+thread_local const char* g_last_kernel = "none";
+// Launch-shape overrides (bitlinear_set_tuning).  The process-wide copy is guarded by a mutex; every
+// entry point takes one snapshot of it into the calling thread's own copy before it plans a launch,
+// so a call never sees half of another thread's update.
+struct Tuning {
+    int waves = 0;
+    int upw = 0;
+    int decode_waves = 0;
+    int path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse, 5 = GEMM tile
+    int fused[3] = {1, 10, 4};
+    int prefill_big = 0;
+    int prefill_band = 0;  // row tiles per band of the prefill GEMM's tile order, 0 = built-in choice
+    int prefill_ks = 0;    // groups of waves splitting K in the small prefill tiles, 0 = built-in choice
+    int staged = 0;        // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
+    int stream = 0;        // product through the streaming kernel: 0 = built-in choice, 1 = whenever it applies, 2 = never
+};
+std::mutex g_tuning_mutex;
+Tuning g_tuning_shared;
+thread_local Tuning t_tune;
+void refresh_tuning() {
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);
+    t_tune = g_tuning_shared;
+}
+
+using bitnet_host::OncePerDevice;
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 constexpr int kPrefillFewTiles = 330;   // up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles
 constexpr int kPrefillSplit2Tiles = 320;  // up to this many 32 x 128 tiles two groups of waves split a tile's K,
@@ -1316,9 +1339,9 @@ void pick_launch(int K, int* waves, int* upw) {
     if (u < 4 && units >= 4 * 4) u = 4;  // keep a few loads in flight per wave
     int w = (units + u - 1) / u;
     if (w > kMaxWaves) w = kMaxWaves;
-    if (g_tune_waves > 0) {
-        w = g_tune_waves;
-        u = g_tune_upw;
+    if (t_tune.waves > 0) {
+        w = t_tune.waves;
+        u = t_tune.upw;
     }
     *waves = w;
     *upw = u;
@@ -1329,6 +1352,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
                   const uint16_t* residual = nullptr) {
     int waves, upw;
     pick_launch(K, &waves, &upw);
+    g_last_kernel = "gemv_i2_mfma_kernel";
     const dim3 grid(N / 16, (M + 15) / 16, 1);
     const dim3 block(waves * 64, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
@@ -1348,7 +1372,8 @@ int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
                   const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
     const int steps = (K + 255) / 256;
     int waves = 4;
-    if (g_tune_decode_waves > 0) waves = g_tune_decode_waves;
+    g_last_kernel = "gemv_i2_decode_kernel";
+    if (t_tune.decode_waves > 0) waves = t_tune.decode_waves;
     const int blocks16 = N / 16;
     const dim3 grid((blocks16 + waves - 1) / waves, 1, 1);
     const dim3 block(waves * 64, 1, 1);
@@ -1390,10 +1415,10 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
     if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31) return pl;  // the kernel addresses the weights with 32-bit byte offsets
     if ((size_t)M * (K + kFusedRowPad) > (pro == 3 ? kFusedLdsRaised : kFusedLdsPlain)) return pl;
     const int units = K / 64;
-    if (g_tune_path == 3) {
-        pl.rb = g_tune_fused[0];
-        pl.s = g_tune_fused[1];
-        pl.upw = g_tune_fused[2];
+    if (t_tune.path == 3) {
+        pl.rb = t_tune.fused[0];
+        pl.s = t_tune.fused[1];
+        pl.upw = t_tune.fused[2];
     } else if (N / 16 >= 1024 && M <= 4) {
         // Many row blocks (N >= 16384) and few tokens: the matrix is large enough to be bandwidth-bound, and what
         // measured best there is many small workgroups (four or five waves per row block, several
@@ -1442,7 +1467,7 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
     }
     const int nvec = M * (K / (pro == 3 ? 16 : 8));
     int need = (nvec + 64 * pl.rb * pl.s - 1) / (64 * pl.rb * pl.s);
-    if (need > 8 && g_tune_path != 3) {
+    if (need > 8 && t_tune.path != 3) {
         // a large activation block: as many waves as a workgroup may have, so that every
         // thread quantizes at most 8 vectors
         pl.s = kMaxWaves / pl.rb;
@@ -1465,13 +1490,12 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
 // may hold up to 16 rows of 6912 and more, so its limit is raised once per
 // instance (a host-side attribute, no stream work).
 template <int U, int V, bool R>
-void raise_fused_lds() {
-    static bool done = false;
-    if (!done) {
-        (void)hipFuncSetAttribute((const void*)bitlinear_fused_kernel<U, V, 3, R>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)(kFusedLdsRaised + kFusedTailPad));
-        done = true;
-    }
+hipError_t raise_fused_lds() {
+    static OncePerDevice once;
+    return once.run([] {
+        return hipFuncSetAttribute((const void*)bitlinear_fused_kernel<U, V, 3, R>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)(kFusedLdsRaised + kFusedTailPad));
+    });
 }
 
 int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const uint16_t* ws, const ScaleMap& smap,
@@ -1484,6 +1508,9 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
     const uint32_t* wq = (const uint32_t*)packed;
     const int pro = ex.act_scale ? 3 : (ex.norm_weight ? (ex.glu ? 2 : 1) : 0);
     if (pro == 0 && ex.residual) return BITLINEAR_ERR_ARG;  // the plain forward has no residual epilogue
+    static const char* const kFusedNames[4] = {"bitlinear_fused_kernel<quantizer>", "bitlinear_fused_kernel<norm>",
+                                               "bitlinear_fused_kernel<gate+norm>", "bitlinear_fused_kernel<staged int8>"};
+    g_last_kernel = kFusedNames[pro];
 #define BITLINEAR_LAUNCH_UVPR(U, V, P, R)                                                                            \
     hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P, R>), grid, block, lds, stream, x, wq, M, N, K, pl.rb, pl.s,  \
                        mode, 1.0f / (float)(K / (pro == 3 ? 16 : 8)), pro == 3 ? ex.act_scale : ex.norm_weight, out, ws, \
@@ -1500,10 +1527,8 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
         case 2: BITLINEAR_LAUNCH_UVP(U, V, 2); break;               \
         default:                                                    \
             if (lds > 48u * 1024u) {                                \
-                if (ex.residual)                                    \
-                    raise_fused_lds<U, V, true>();                  \
-                else                                                \
-                    raise_fused_lds<U, V, false>();                 \
+                const hipError_t e = ex.residual ? raise_fused_lds<U, V, true>() : raise_fused_lds<U, V, false>(); \
+                if (e != hipSuccess) return BITLINEAR_ERR_LAUNCH;   \
             }                                                       \
             BITLINEAR_LAUNCH_UVP(U, V, 3);                          \
             break;                                                  \
@@ -1535,18 +1560,22 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const uint32_t* wq = (const uint32_t*)packed;
     // the kernel addresses the packed weights through a buffer descriptor with 32-bit offsets
     if ((long long)N * K / 4 >= (1ll << 31)) return BITLINEAR_ERR_SHAPE;
+    g_last_kernel = "gemm_i2_prefill_kernel";
     // the large tile double-buffers 2 x 128 rows x 272 bytes = 68 KiB of LDS (so do four groups of the
     // small one): above the 64 KiB a kernel gets without asking (a host-side attribute, set once per process)
-    static bool lds_limit_raised = false;
-    if (!lds_limit_raised) {
-        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<4, 2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  2 * 128 * kPfRowBytes);
-        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<1, 1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  4 * 2 * 32 * kPfRowBytes);
-        (void)hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<2, 1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  2 * 2 * 64 * kPfRowBytes);
-        lds_limit_raised = true;
-    }
+    static OncePerDevice lds_limit_raised;
+    const hipError_t lds_err = lds_limit_raised.run([] {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<4, 2, 1>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 128 * kPfRowBytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<1, 1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    4 * 2 * 32 * kPfRowBytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<2, 1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    2 * 2 * 64 * kPfRowBytes);
+        return e;
+    });
+    if (lds_err != hipSuccess) return BITLINEAR_ERR_LAUNCH;
     // tile (rows x columns of the output per workgroup): 0 = 64 x 128, 1 = 128 x 256, 2 = 64 x 256,
     // 3 = 64 x 512, 4 = 32 x 128.  Measured: the wide tile pays once there are many tiles (about four
     // per CU of the narrow kind); with few tiles (up to about 1.3 per CU) half-height tiles put twice as
@@ -1554,7 +1583,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // us at 3840 x 2560, 21.5 -> 16.4 at 2560 x 6912).
     const long long narrow_tiles = (long long)((N + 127) / 128) * ((M + 63) / 64);
     int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : (narrow_tiles <= kPrefillFewTiles ? 4 : 0);
-    if (g_tune_path == 5) tile = g_tune_prefill_big;
+    if (t_tune.path == 5) tile = t_tune.prefill_big;
     // groups of waves that split a tile's K between them (small tiles only): while the small tiles
     // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
     // instruction stream, and more groups shorten it
@@ -1565,7 +1594,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // 11.6 -> 13.6 us)
     if (tile == 4 && small_tiles <= kPrefillSplit2Tiles)
         ks = (small_tiles <= kPrefillSplit4Tiles && K >= kPrefillSplit4MinK) ? 4 : 2;
-    if (g_tune_path == 5 && g_tune_prefill_ks > 0) ks = (tile == 4 || (tile == 0 && g_tune_prefill_ks == 2)) ? g_tune_prefill_ks : 1;
+    if (t_tune.path == 5 && t_tune.prefill_ks > 0) ks = (tile == 4 || (tile == 0 && t_tune.prefill_ks == 2)) ? t_tune.prefill_ks : 1;
     if (K <= kPfChunk * (ks - 1)) ks = 1;  // fewer chunks than groups
     const dim3 block(kPfWaves * 64 * ks, 1, 1);
     // grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
@@ -1575,7 +1604,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     const int row_tiles = (M + tm - 1) / tm, col_tiles = (N + tn - 1) / tn;
     int band = row_tiles / 8;
     band = band < 1 ? 1 : (band > 8 ? 8 : band);
-    if (g_tune_path == 5 && g_tune_prefill_band > 0) band = g_tune_prefill_band;
+    if (t_tune.path == 5 && t_tune.prefill_band > 0) band = t_tune.prefill_band;
     const int nbands = (row_tiles + band - 1) / band;
     // the columns are cut into segments as well, as many as it takes for the number of (band,
     // segment) units to be a multiple of the 8 XCDs: every XCD then gets the same number of units
@@ -1623,13 +1652,13 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
                 const uint16_t* residual = nullptr) {
     // vector loads: 16-byte groups of both operands must be 16-byte aligned
     if ((((uintptr_t)act) | ((uintptr_t)packed)) & 15u) return BITLINEAR_ERR_ARG;
-    if (M > kPrefillMinTokens && g_tune_path != 2) {
+    if (M > kPrefillMinTokens && t_tune.path != 2) {
         // A few dozen tokens on a narrow matrix leave most CUs without a GEMM tile, and a tile's
         // chain of 256-k chunks is then pure latency (about 0.64 us each).  There the split-K kernel,
         // run once per 16 tokens and re-reading the weights from L2 (about 1.45 TB/s measured),
         // finishes earlier.  Both estimates in microseconds, fitted to measurements at the 2B shapes.
         bool gemm = true;
-        if (M <= 256 && g_tune_path == 0) {
+        if (M <= 256 && t_tune.path == 0) {
             const double groups = (M + 15) / 16;
             const double splitk_us = 3.5 + groups * ((double)N * K / 4.0) / 1.45e6;
             const double tiles = ((N + 127) / 128) * (double)((M + 63) / 64);
@@ -1647,21 +1676,25 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // The kernel that stages the int8 rows in LDS once per workgroup and shares
     // them between several row blocks: fewer activation bytes through L2 than
     // the kernels below, which read their B operands straight from global.
-    if (out && !acc_out && g_tune_staged != 2 && g_tune_path != 1 && g_tune_path != 2) {
+    // (The accumulator export takes the same kernel choice as the drop-in call, so what the parity
+    // tests read is what the drop-in entry computes.  Without an output there are no scales: the
+    // kernel's unconditional scale requests then go to an address that exists.)
+    if (t_tune.staged != 2 && t_tune.path != 1 && t_tune.path != 2) {
         const FusedPlan pl = plan_fused(M, N, K, 3);
         // measured: up to 4 tokens staging always wins (2.8-4.5 us against 3.1-5.1 at the 2B shapes);
         // beyond, it pays once a workgroup shares the rows between two or more row blocks
-        const bool wanted = g_tune_staged == 1 || M <= kDecodeMaxTokens || (N / 16) >= 432;
+        const bool wanted = t_tune.staged == 1 || M <= kDecodeMaxTokens || (N / 16) >= 432;
         if (pl.ok && wanted)
-            return launch_fused((const uint16_t*)act, packed, out, ws, smap, nullptr, nullptr,
-                                FusedExtras{nullptr, residual, 0.0f, 0, s}, M, N, K, 0, pl, stream);
+            return launch_fused((const uint16_t*)act, packed, out, out ? ws : (const uint16_t*)packed, smap, nullptr,
+                                nullptr, FusedExtras{nullptr, residual, 0.0f, 0, out ? s : (const uint16_t*)packed, acc_out},
+                                M, N, K, 0, pl, stream);
     }
     if (residual) return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
     const bool decode_fits = M <= kDecodeMaxTokens && (size_t)M * K <= (size_t)kDecodeMaxLdsBytes;
     // The one-wave-per-row-block kernel pays off once there are enough row
     // blocks to fill every SIMD; below that, splitting K across waves wins.
     const bool many_rows = (N / 16) >= 512;
-    if (decode_fits && g_tune_path != 2 && (many_rows || g_tune_path == 1)) return launch_decode(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+    if (decode_fits && t_tune.path != 2 && (many_rows || t_tune.path == 1)) return launch_decode(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
     return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
 }
 
@@ -1678,6 +1711,8 @@ ScaleMap equal_slots(int N, int ws_num) {
 extern "C" {
 
 int bitlinear_last_status(void) { return g_status; }
+
+const char* bitlinear_last_kernel(void) { return g_last_kernel; }
 
 const char* bitlinear_status_string(int status) {
     switch (status) {
@@ -1697,53 +1732,60 @@ int bitlinear_ws_num(int N, int K) {
 }
 
 int bitlinear_set_tuning(int kernel, int a, int b, int c) {
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);
+    Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g_tune_path = g_tune_waves = g_tune_upw = g_tune_decode_waves = g_tune_staged = 0;
+        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
         if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
-        g_tune_staged = a;
+        g.staged = a;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 7) {
+        if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
+        g.stream = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 1) {
         if (a < 1 || a > kDecodeMaxWaves) return set_status(BITLINEAR_ERR_ARG);
-        g_tune_path = 1;
-        g_tune_decode_waves = a;
+        g.path = 1;
+        g.decode_waves = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 2) {
         if (a == 0 && b == 0) {  // split-K kernel always, launch shape left to the library
-            g_tune_path = 2;
-            g_tune_waves = g_tune_upw = 0;
+            g.path = 2;
+            g.waves = g.upw = 0;
             return set_status(BITLINEAR_OK);
         }
         if (a < 1 || a > kMaxWaves || !(b == 1 || b == 2 || b == 4 || b == 8))
             return set_status(BITLINEAR_ERR_ARG);
-        g_tune_path = 2;
-        g_tune_waves = a;
-        g_tune_upw = b;
+        g.path = 2;
+        g.waves = a;
+        g.upw = b;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 3) {
         const bool upw_ok = c == 4 || c == 5 || c == 8 || c == 10 || c == 16;
         if (a < 1 || a > kFusedMaxRB || b < 1 || a * b > kMaxWaves || !upw_ok) return set_status(BITLINEAR_ERR_ARG);
-        g_tune_path = 3;
-        g_tune_fused[0] = a;
-        g_tune_fused[1] = b;
-        g_tune_fused[2] = c;
+        g.path = 3;
+        g.fused[0] = a;
+        g.fused[1] = b;
+        g.fused[2] = c;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 4) {
-        g_tune_path = 4;
+        g.path = 4;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
         if (a < 0 || a > 4 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
-        g_tune_path = 5;
-        g_tune_prefill_big = a;
-        g_tune_prefill_band = b;
-        g_tune_prefill_ks = c;
+        g.path = 5;
+        g.prefill_big = a;
+        g.prefill_band = b;
+        g.prefill_ks = c;
         return set_status(BITLINEAR_OK);
     }
     return set_status(BITLINEAR_ERR_ARG);
@@ -1751,6 +1793,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
 
 int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1, int32_t* acc_out, uint16_t* output0,
                                 const uint16_t* s, const uint16_t* ws, int M, int N, int K, void* stream) {
+    refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!input0 || !input1 || (!acc_out && !output0) || (output0 && (!s || !ws))) return set_status(BITLINEAR_ERR_NULL);
     return set_status(launch_gemv(input0, input1, output0, acc_out, s, ws, equal_slots(N, bitlinear_ws_num(N, K)), M,
@@ -1759,6 +1802,7 @@ int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1, int3
 
 void bitlinear_int8xint2(int8_t* input0, int8_t* input1, uint16_t* output0, uint16_t* s, uint16_t* ws, int M, int N,
                          int K, void* stream) {
+    refresh_tuning();
     if (!shape_ok(M, N, K)) {
         // same line the reference prints for a shape it has no kernel for (bitnet_kernels.cu:35)
         printf("required ladder gemm kernel: M %d, N %d, K %d\n", M, N, K);
@@ -1776,6 +1820,7 @@ void bitlinear_int8xint2(int8_t* input0, int8_t* input1, uint16_t* output0, uint
 
 int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1, uint16_t* output0, const uint16_t* s,
                             const uint16_t* ws, const int* seg_ends, int nseg, int M, int N, int K, void* stream) {
+    refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!input0 || !input1 || !output0 || !s || !ws || !seg_ends) return set_status(BITLINEAR_ERR_NULL);
     if (nseg < 1 || nseg > kMaxSeg) return set_status(BITLINEAR_ERR_ARG);
@@ -1809,8 +1854,9 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s, int M, int
     return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
 }
 
-int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
-                           int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+static int forward_impl(const uint16_t* x, const int8_t* packed, uint16_t* output0, int32_t* acc_out, const uint16_t* ws,
+                        int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+    refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !packed || !output0 || !ws) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
@@ -1819,21 +1865,34 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* ou
     const FusedPlan pl = plan_fused(M, N, K);
     // one kernel while the activation block is small enough for every workgroup to quantize it
     // again (or when the caller gave no workspaces for the two-kernel path)
-    const bool small = (long long)M * K <= kFuseMaxElems || g_tune_path == 3 || !q_ws || !s_ws;
-    if (pl.ok && small && g_tune_path != 4)
+    const bool small = (long long)M * K <= kFuseMaxElems || t_tune.path == 3 || !q_ws || !s_ws;
+    if (pl.ok && small && t_tune.path != 4)
         return set_status(launch_fused(x, packed, output0, ws, sm, q_ws, s_ws,
-                                       FusedExtras{nullptr, nullptr, 0.0f, 0, nullptr}, M, N, K, mode, pl,
+                                       FusedExtras{nullptr, nullptr, 0.0f, 0, nullptr, acc_out}, M, N, K, mode, pl,
                                        (hipStream_t)stream));
     // larger blocks: the quantizer once, in a kernel of its own, then the product
     if (!q_ws || !s_ws) return set_status(BITLINEAR_ERR_NULL);
     const int st = bitlinear_quant_absmax(x, q_ws, s_ws, M, K, mode, stream);
     if (st != BITLINEAR_OK) return st;
-    return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream));
+    return set_status(launch_gemv(q_ws, packed, output0, acc_out, s_ws, ws, sm, M, N, K, (hipStream_t)stream));
+}
+
+int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
+                           int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+    return forward_impl(x, packed, output0, nullptr, ws, q_ws, s_ws, M, N, K, mode, stream);
+}
+
+int bitlinear_forward_bf16_acc_i32(const uint16_t* x, const int8_t* packed, int32_t* acc_out, uint16_t* output0,
+                                   const uint16_t* ws, int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode,
+                                   void* stream) {
+    if (!acc_out) return set_status(BITLINEAR_ERR_NULL);
+    return forward_impl(x, packed, output0, acc_out, ws, q_ws, s_ws, M, N, K, mode, stream);
 }
 
 int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu,
                                 const int8_t* packed, const uint16_t* ws, const uint16_t* residual, uint16_t* output0,
                                 int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+    refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !norm_weight || !packed || !ws || !output0) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
@@ -1841,9 +1900,9 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, 
         return set_status(BITLINEAR_ERR_ARG);
     const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
     const FusedPlan pl = plan_fused(M, N, K, glu ? 2 : 1);
-    const bool small = (long long)M * K <= kFuseMaxElemsNorm || g_tune_path == 3 || !q_ws || !s_ws;
-    if (pl.ok && small && g_tune_path != 4) {
-        const FusedExtras ex = {norm_weight, residual, eps, glu ? 1 : 0, nullptr};
+    const bool small = (long long)M * K <= kFuseMaxElemsNorm || t_tune.path == 3 || !q_ws || !s_ws;
+    if (pl.ok && small && t_tune.path != 4) {
+        const FusedExtras ex = {norm_weight, residual, eps, glu ? 1 : 0, nullptr, nullptr};
         return set_status(launch_fused(x, packed, output0, ws, sm, nullptr, nullptr, ex, M, N, K, mode, pl,
                                        (hipStream_t)stream));
     }

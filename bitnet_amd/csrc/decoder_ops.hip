@@ -19,7 +19,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "bitnet_decoder_ops.h"
+#include "host_util.h"
 
 namespace {
 
@@ -344,6 +347,9 @@ __global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
     // completed = visible device-wide); only then is the arrival counted, with a device-scope
     // atomic, and the last arrival reads the records with device-coherent loads.  No L2-wide
     // writeback or invalidate is involved.
+    // (the wait is spelled out: the arrival below must not be counted before this thread's
+    // write-through record stores are acknowledged)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
         const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -791,14 +797,23 @@ __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const fl
 
 }  // namespace
 
-static int g_attn_threads = 0;
-static int g_attn_kernel = 0;  // 0 = built-in choice, 1 = score buffer in LDS + vector-pipe P.V, 2 = everything on the matrix pipe
+static std::atomic<int> g_attn_threads{0};
+static std::atomic<int> g_attn_kernel{0};  // 0 = built-in choice, 1 = score buffer in LDS + vector-pipe P.V, 2 = everything on the matrix pipe
 
 // in attn_prefill.hip
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
                                     const float* cos_table, const float* sin_table, const float* rope_rows, uint16_t* out,
                                     float* workspace, int* counters, int n_splits, int threads, int B, int S,
-                                    int n_heads, int n_kv_heads, hipStream_t stream);
+                                    int n_heads, int n_kv_heads, int spin_limit, hipStream_t stream);
+
+static std::atomic<int> g_attn_spin_limit{-1};  // polls of the merging workgroup; < 0 = the kernel's own limit
+
+/* test hook: the bound of the merging workgroup's poll (< 0 restores the built-in bound; 0 makes every
+   merge of more than one split give up at once, which is how the failure path is tested) */
+extern "C" int bitnet_attn_decode_set_spin_limit(int polls) {
+    g_attn_spin_limit = polls < 0 ? -1 : polls;
+    return 0;
+}
 
 /* tuning override for tests and measurements: which of the two decode-step attention kernels runs */
 extern "C" int bitnet_attn_decode_set_kernel(int which) {
@@ -814,11 +829,22 @@ extern "C" int bitnet_attn_decode_set_threads(int threads) {
     return 0;
 }
 
+// records of 8-byte units (value, tag) per (sequence, kv head, split, head), then one epoch per
+// (sequence, kv head), then the error word and a word of padding
+static long long attn_ws_error_index(int B, int n_heads, int n_kv_heads, int n_splits) {
+    return (long long)B * n_kv_heads * n_splits * (n_heads / n_kv_heads) * kRecFloats * 2 + (long long)B * n_kv_heads;
+}
+
 extern "C" int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits) {
     if (B < 1 || n_heads < 1 || n_kv_heads < 1 || n_splits < 1 || n_heads % n_kv_heads) return -1;
-    // records of 8-byte units (value, tag) per (sequence, kv head, split, head), then one epoch per (sequence, kv head)
-    const long long n = (long long)B * n_kv_heads * n_splits * (n_heads / n_kv_heads) * kRecFloats * 2 + (long long)B * n_kv_heads;
+    const long long n = attn_ws_error_index(B, n_heads, n_kv_heads, n_splits) + 2;
     return n < (1ll << 31) ? (int)n : -1;
+}
+
+extern "C" int bitnet_attn_decode_error_index(int B, int n_heads, int n_kv_heads, int n_splits) {
+    if (B < 1 || n_heads < 1 || n_kv_heads < 1 || n_splits < 1 || n_heads % n_kv_heads) return -1;
+    const long long n = attn_ws_error_index(B, n_heads, n_kv_heads, n_splits);
+    return n + 2 < (1ll << 31) ? (int)n : -1;
 }
 
 static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
@@ -846,21 +872,22 @@ static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* ca
     // up to 128 rows of the capacity in one round (measured at 96 rows: 6.85 us with four waves, 7.12 with
     // eight; at 272 rows 8.77 / 8.46)
     if (flash) threads = (span > 128 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
-    if (g_attn_threads) threads = g_attn_threads;
+    if (const int forced = g_attn_threads.load()) threads = forced;
     if (flash)
         return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, rope_rows, out, workspace,
-                                               counters, n_splits, threads, B, S, n_heads, n_kv_heads, (hipStream_t)stream);
+                                               counters, n_splits, threads, B, S, n_heads, n_kv_heads, g_attn_spin_limit.load(),
+                                               (hipStream_t)stream);
     const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * 1024) * sizeof(float);  // scores + one 4 KB region per wave
     if (lds > 96u * 1024u) return 1;
     const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
 #define BITNET_ATTN_LAUNCH(GG)                                                                                        \
     {                                                                                                                 \
-        static bool raised = false; /* more than 64 KiB of dynamic LDS has to be asked for, once per process */     \
-        if (!raised) {                                                                                                \
-            (void)hipFuncSetAttribute((const void*)attn_decode_kernel<GG>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                      96 * 1024);                                                                     \
-            raised = true;                                                                                            \
-        }                                                                                                             \
+        static bitnet_host::OncePerDevice raised; /* more than 64 KiB of dynamic LDS has to be asked for */          \
+        if (raised.run([] {                                                                                           \
+                return hipFuncSetAttribute((const void*)attn_decode_kernel<GG>,                                       \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);                    \
+            }) != hipSuccess)                                                                                         \
+            return 3;                                                                                                 \
         hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, block, lds, (hipStream_t)stream, qkv, cache_k, cache_v,      \
                            positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads);       \
     }
@@ -891,7 +918,7 @@ extern "C" int bitnet_attn_decode_rows(const uint16_t* qkv, uint16_t* cache_k, u
                             n_splits, B, S, n_heads, n_kv_heads, head_dim, stream);
 }
 
-static int g_lm_kernel = 0;  // 0 = built-in choice, 1 = matrix-pipe kernel, 2 = streaming kernel where it applies
+static std::atomic<int> g_lm_kernel{0};  // 0 = built-in choice, 1 = matrix-pipe kernel, 2 = streaming kernel where it applies
 
 /* tuning override for tests and measurements; results differ only in the order of fp32 additions */
 extern "C" int bitnet_lm_head_set_kernel(int which) {
@@ -916,11 +943,11 @@ static int lm_head_greedy_impl(const uint16_t* h, const uint16_t* norm_weight, f
         return 1;
     const size_t lds = (size_t)B * (2 * (size_t)K + kLmRowPad);
     if (lds > 96u * 1024u) return 1;
-    static bool raised = false;  // more than 64 KiB of dynamic LDS has to be asked for, once per process
-    if (!raised) {
-        (void)hipFuncSetAttribute((const void*)lm_head_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        raised = true;
-    }
+    static bitnet_host::OncePerDevice raised;  // more than 64 KiB of dynamic LDS has to be asked for
+    if (raised.run([] {
+            return hipFuncSetAttribute((const void*)lm_head_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        }) != hipSuccess)
+        return 3;
     hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(B), dim3(kNormThreads), 0, (hipStream_t)stream, h, norm_weight, eps, y_ws, K);
     int nparts = 0;
     const bool stream_ok = B <= 8 && (K % 512) == 0 && (size_t)B * 2 * K <= 60u * 1024u;

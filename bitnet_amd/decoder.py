@@ -74,10 +74,29 @@ class AttnWorkspace:
 
     def __init__(self, batch: int, n_heads: int, n_kv_heads: int, n_splits: int, device):
         lib = _lib.load_library()
+        self.batch = batch
+        self.n_heads = n_heads
+        self.n_kv_heads = n_kv_heads
         self.n_splits = n_splits
         n = lib.bitnet_attn_decode_workspace_floats(batch, n_heads, n_kv_heads, n_splits)
-        self.partials = torch.zeros(max(n, 1), dtype=torch.float32, device=device)  # zero once: see bitnet_attn_decode
+        if n < 0:
+            raise ValueError("AttnWorkspace: bad batch / head counts / number of splits")
+        self.error_index = lib.bitnet_attn_decode_error_index(batch, n_heads, n_kv_heads, n_splits)
+        self.partials = torch.zeros(n, dtype=torch.float32, device=device)  # zero once: see bitnet_attn_decode
         self.counters = torch.zeros(batch * n_kv_heads, dtype=torch.int32, device=device)
+
+    def error(self) -> int:
+        """The workspace's error word (synchronises): non-zero once a merge of
+        the splits' records gave up, which also left NaN rows in that call's
+        output (bitnet_attn_decode_error_index)."""
+        return int(self.partials[self.error_index : self.error_index + 1].view(torch.int32).item())
+
+    def check(self) -> None:
+        if self.error():
+            raise _lib.BitLinearLibraryError(
+                "attention decode: a merge of the split records gave up (workspace not zeroed before its first use, "
+                "or shared between overlapping calls); the affected output rows are NaN"
+            )
 
 
 def decode_step_begin(tokens, positions, emb_weight, cos, sin):
@@ -105,6 +124,21 @@ def attn_decode(xqkv, cache_k, cache_v, positions, cos, sin, n_heads, n_kv_heads
     B = xqkv.shape[0]
     S = cache_k.shape[1]
     hd = cache_k.shape[-1]
+    # the kernels index every buffer with these sizes: check them here, before any launch
+    if xqkv.dtype != torch.bfloat16 or cache_k.dtype != torch.bfloat16 or cache_v.dtype != torch.bfloat16:
+        raise TypeError("attn_decode: xqkv and the caches must be bfloat16")
+    if xqkv.shape != (B, (n_heads + 2 * n_kv_heads) * hd):
+        raise ValueError(f"attn_decode: xqkv has shape {tuple(xqkv.shape)}, expected {(B, (n_heads + 2 * n_kv_heads) * hd)}")
+    if cache_k.shape != (B, S, n_kv_heads, hd) or cache_v.shape != cache_k.shape:
+        raise ValueError("attn_decode: the caches must be [batch, max_seq, n_kv_heads, head_dim] with the batch of xqkv")
+    if positions.dtype != torch.int64 or positions.numel() != B:
+        raise ValueError("attn_decode: positions must be int64 [batch]")
+    if cos.shape[0] < S or sin.shape[0] < S:
+        raise ValueError("attn_decode: the rope tables have fewer rows than the cache has positions")
+    if workspace is not None and (workspace.batch != B or workspace.n_heads != n_heads or workspace.n_kv_heads != n_kv_heads):
+        raise ValueError("attn_decode: the workspace was sized for another batch or head count")
+    if rope_rows is not None and (rope_rows.dtype != torch.float32 or rope_rows.shape != (B, hd)):
+        raise ValueError("attn_decode: rope_rows must be float32 [batch, head_dim]")
     out = torch.empty(B, n_heads * hd, dtype=torch.bfloat16, device=xqkv.device)
     ns = workspace.n_splits if workspace is not None else 1
     lib = _lib.load_library()
@@ -195,6 +229,15 @@ def norm_bitlinear(x, norm: "RMSNorm", lin: BitLinearKernel, glu: bool = False, 
     [M, K] (or [M, 2K] with glu)."""
     M = x.shape[0]
     K = lin.in_features
+    if x.dtype != torch.bfloat16 or not x.is_cuda or not x.is_contiguous():
+        raise ValueError("norm_bitlinear: x must be a contiguous bfloat16 GPU tensor")
+    if x.dim() != 2 or x.shape[1] != (2 * K if glu else K):
+        raise ValueError(f"norm_bitlinear: x has shape {tuple(x.shape)}, expected [M, {2 * K if glu else K}]")
+    if norm.weight.dtype != torch.bfloat16 or norm.weight.numel() != K:
+        raise ValueError("norm_bitlinear: the norm weight must be bfloat16 [K]")
+    if residual is not None and (residual.dtype != torch.bfloat16 or residual.shape != (M, lin.out_features)
+                                 or not residual.is_contiguous()):
+        raise ValueError("norm_bitlinear: residual must be contiguous bfloat16 [M, N]")
     out = torch.empty(M, lin.out_features, dtype=torch.bfloat16, device=x.device)
     q_ws = torch.empty(M, K, dtype=torch.int8, device=x.device)
     s_ws = torch.empty(M, dtype=torch.bfloat16, device=x.device)
@@ -484,6 +527,10 @@ class Generator:
         tokens greedily.  Returns [steps, B]."""
         if steps > self.history.shape[0]:
             raise ValueError("more steps than the generator was sized for")
+        if start_pos < 0 or start_pos + steps > self.max_seq:
+            raise ValueError(
+                f"decode: positions {start_pos}..{start_pos + steps - 1} do not fit a cache of {self.max_seq} rows"
+            )
         self.tok.copy_(first.view(-1, 1))
         self.pos.fill_(start_pos)
         if self.use_graph and self.graph is None:
@@ -502,4 +549,7 @@ class Generator:
                 self.graph.replay()
             else:
                 self._step()
-        return self.history[:steps].clone()
+        out = self.history[:steps].clone()
+        if self.fused:
+            self.attn_ws.check()  # one small copy to the host per decode() call
+        return out

@@ -76,6 +76,15 @@ int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1,
                                 int M, int N, int K, void* stream);
 
 /*
+ * Name of the product kernel that the calling host thread's most recent call
+ * launched ("none" before the first).  M <= 16 takes the same kernel whether
+ * or not acc_out is asked for, so a parity test of the accumulators reads what
+ * the drop-in entry computes; tests and the smoke check report the name.  The
+ * reference has one kernel and nothing to report (bitnet_kernels.cu:3-37).
+ */
+const char* bitlinear_last_kernel(void);
+
+/*
  * Variant with explicit weight-scale segments: row n uses ws[j] for the first
  * j with n < seg_ends[j]  (seg_ends ascending, seg_ends[nseg-1] == N,
  * 1 <= nseg <= 8, host array).  This is the scale layout
@@ -120,6 +129,17 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
                            uint16_t* output0, const uint16_t* ws,
                            int8_t* q_ws, uint16_t* s_ws,
                            int M, int N, int K, int mode, void* stream);
+
+/*
+ * bitlinear_forward_bf16 that also stores the int32 accumulators of the product
+ * (bitnet_kernels.h:74-78) to acc_out [M, N]: the same kernels, launch shapes
+ * and results.  Exists so tests can prove the accumulators of the one-kernel
+ * forward bit-exact.
+ */
+int bitlinear_forward_bf16_acc_i32(const uint16_t* x, const int8_t* packed,
+                                   int32_t* acc_out, uint16_t* output0,
+                                   const uint16_t* ws, int8_t* q_ws, uint16_t* s_ws,
+                                   int M, int N, int K, int mode, void* stream);
 
 /*
  * bitlinear_forward_bf16 with the operations that surround a BitLinear in the

@@ -125,6 +125,22 @@ int bitnet_attn_decode_set_kernel(int which);
 int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits);
 
 /*
+ * Index (in floats) of the workspace's error word, an int that is zero in a healthy workspace.
+ * With more than one split, the workgroup that merges the splits' records polls for them a bounded
+ * number of times.  If a poll ever runs out (a workspace that was not zero before its first use, or
+ * splits that did not start in the order the kernel counts on), the affected heads' output rows are
+ * written as NaN and this word is set to 1; it stays set until the host clears the workspace.  No
+ * entry point reads it back (none synchronises): the caller copies the word to the host when it
+ * next synchronises anyway, e.g. at the end of a generation.  -1 for bad arguments.
+ */
+int bitnet_attn_decode_error_index(int B, int n_heads, int n_kv_heads, int n_splits);
+
+/* Test hook: bound of that poll (< 0 restores the built-in bound of 65536 rounds; 0 makes every
+ * merge of more than one split give up at once -- every kernel still runs to its end -- which is
+ * how the failure path above is tested).  Returns 0. */
+int bitnet_attn_decode_set_spin_limit(int polls);
+
+/*
  * The tail of a greedy decode step (Transformer.forward's `self.output(self.norm(h))`,
  * gpu/model.py:280-281, and the argmax of the generation loop, gpu/generate.py:264-288):
  *   y      = RMSNorm(h) with norm_weight (same rounding points as bitlinear_norm_forward_bf16)

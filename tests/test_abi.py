@@ -64,7 +64,9 @@ def test_host_only_entry_points():
     assert lib.bitlinear_set_tuning(5, 1, 0, 0) == 0
     assert lib.bitlinear_set_tuning(6, 1, 0, 0) == 0
     assert lib.bitlinear_set_tuning(6, 3, 0, 0) != 0
-    assert lib.bitlinear_set_tuning(7, 0, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(7, 1, 0, 0) == 0
+    assert lib.bitlinear_set_tuning(7, 3, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(8, 0, 0, 0) != 0
     assert lib.bitlinear_set_tuning(0, 0, 0, 0) == 0
 
 
@@ -96,7 +98,11 @@ def test_decoder_entry_argument_checks_need_no_gpu():
     assert lib.bitnet_attn_decode(None, None, None, None, None, None, None, None, None, 17, 1, 64, 4, 2, 128, None) == 1
     assert lib.bitnet_attn_decode(None, None, None, None, None, None, None, None, None, 1, 1, 64, 4, 2, 128, None) == 2
     assert lib.bitnet_attn_decode_rows(None, None, None, None, None, None, None, None, None, None, 1, 1, 64, 4, 2, 128, None) == 2
-    assert lib.bitnet_attn_decode_workspace_floats(1, 20, 5, 8) == 1 * 5 * 8 * 4 * 130 * 2 + 5
+    assert lib.bitnet_attn_decode_workspace_floats(1, 20, 5, 8) == 1 * 5 * 8 * 4 * 130 * 2 + 5 + 2
+    assert lib.bitnet_attn_decode_error_index(1, 20, 5, 8) == 1 * 5 * 8 * 4 * 130 * 2 + 5
+    assert lib.bitnet_attn_decode_error_index(1, 20, 6, 8) == -1
+    assert lib.bitnet_attn_decode_set_spin_limit(5) == 0 and lib.bitnet_attn_decode_set_spin_limit(-1) == 0
+    assert lib.bitlinear_last_kernel() in (b"none", b"gemv_i2_mfma_kernel")
     assert lib.bitnet_attn_decode_workspace_floats(1, 20, 6, 8) == -1
     assert lib.bitnet_attn_decode_set_kernel(3) == 1 and lib.bitnet_attn_decode_set_kernel(0) == 0
     # prompt side: start + T beyond the cache, head_dim, nulls

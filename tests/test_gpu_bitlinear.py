@@ -97,7 +97,7 @@ def test_acc_single_nonzero_weight_picks_the_activation():
 
 
 @pytest.mark.parametrize("shape_id", [0, 1, 2, 3])
-@pytest.mark.parametrize("m", [1, 4, 16])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16])
 def test_scaled_output_at_2b_shapes(shape_id, m):
     """Configs 0-2: seeded N(0,1) activations, quantized per token, real
     weight scales in the slots this shape uses."""
@@ -115,6 +115,81 @@ def test_scaled_output_at_2b_shapes(shape_id, m):
     mod.weight_scale.data = dev_bf16(ws_bits)
     out2 = mod(dev_bf16(xb))
     _assert_bits_equal(host_bits(out2), want, f"{sh.name} forward M={m}")
+
+
+@pytest.mark.parametrize("shape_id", [0, 1, 2, 3])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16])
+def test_default_path_accumulators_bit_exact_at_2b_shapes(shape_id, m):
+    """in_thread_C_local after the reduction (gpu/bitnet_kernels/bitnet_kernels.h:74-78),
+    read from the kernels the library picks by itself: the accumulator export of
+    the drop-in entry must run the kernel the drop-in entry runs, and the
+    one-kernel forward (quantizer inside) exports its own.  Seeded workload data."""
+    lib = _lib.load_library()
+    sh = workload.shapes_2b()[shape_id]
+    w = workload.ternary_weight(sh.K, sh.N, shape_id)
+    ws_bits = workload.weight_scales(sh.K, sh.N, shape_id, sh.parts)
+    xb = workload.activations_bf16(m, sh.K, shape_id)
+    q, s_bits = o.quant_input(xb, o.QUANT_COMPILED)
+    acc_want, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    pk, qd = _packed_dev(w), dev_i8(q)
+    out = bitlinear.bitnet_int8xint2_linear(qd, pk, dev_bf16(s_bits), dev_bf16(ws_bits))
+    k_dropin = bitlinear.last_kernel()
+    acc = bitlinear.bitnet_int8xint2_acc(qd, pk)
+    k_acc = bitlinear.last_kernel()
+    assert k_acc == k_dropin, (k_acc, k_dropin)
+    if m <= 4:
+        assert k_dropin == "bitlinear_fused_kernel<staged int8>"  # what bench.py's product-only figure times
+    assert np.array_equal(acc.cpu().numpy(), acc_want), k_acc
+    _assert_bits_equal(host_bits(out), want, f"{sh.name} M={m} ({k_dropin})")
+    # accumulators and output in ONE call of the export (s and ws given)
+    import ctypes
+
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    acc2 = torch.empty(m, sh.N, dtype=torch.int32, device="cuda")
+    out2 = torch.empty(m, sh.N, dtype=torch.bfloat16, device="cuda")
+    sd, wsd = dev_bf16(s_bits), dev_bf16(ws_bits)
+    assert lib.bitlinear_int8xint2_acc_i32(P(qd), P(pk), P(acc2), P(out2), P(sd), P(wsd), m, sh.N, sh.K, None) == 0
+    assert np.array_equal(acc2.cpu().numpy(), acc_want)
+    _assert_bits_equal(host_bits(out2), want, "acc export with output")
+    # the whole forward: quantizer + product in one kernel while the block is small
+    out3, acc3 = bitlinear.bitlinear_forward_acc(dev_bf16(xb), pk, dev_bf16(ws_bits))
+    k_fwd = bitlinear.last_kernel()
+    if m * sh.K <= 16384:
+        assert k_fwd == "bitlinear_fused_kernel<quantizer>"  # what bench.py's headline times at M = 1
+    assert np.array_equal(acc3.cpu().numpy(), acc_want), k_fwd
+    _assert_bits_equal(host_bits(out3), want, f"{sh.name} forward M={m} ({k_fwd})")
+
+
+@pytest.mark.parametrize("rb,s_,upw", [(1, 8, 5), (2, 5, 8), (4, 4, 10), (2, 8, 5), (1, 16, 4), (3, 5, 8)])
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_fused_kernel_accumulators_for_every_launch_shape(rb, s_, upw, m):
+    """The LDS-atomic reduction and the -2 * sum(q) correction of the fused kernel
+    with one to four row blocks per workgroup, read as raw int32 (quantizer
+    inside, and int8 rows staged)."""
+    lib = _lib.load_library()
+    n, k = 2560, 2560
+    rng = np.random.default_rng(rb * 100 + s_ * 10 + m)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    xb = o.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0, 0, 0], dtype=np.float32))
+    q, s_bits = o.quant_input(xb, 0)
+    acc_want, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    pk = _packed_dev(w)
+    try:
+        assert lib.bitlinear_set_tuning(3, rb, s_, upw) == 0
+        out, acc = bitlinear.bitlinear_forward_acc(dev_bf16(xb), pk, dev_bf16(ws_bits))
+        # (a thread of the one-kernel forward quantizes at most 8 vectors of 8 values: 16 tokens do not fit 512 threads)
+        if m * k // 8 <= 8 * 64 * rb * s_:
+            assert bitlinear.last_kernel() == "bitlinear_fused_kernel<quantizer>"
+        assert lib.bitlinear_set_tuning(6, 1, 0, 0) == 0
+        acc_staged = bitlinear.bitnet_int8xint2_acc(dev_i8(q), pk)
+        assert bitlinear.last_kernel() == "bitlinear_fused_kernel<staged int8>"
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    assert np.array_equal(acc_staged.cpu().numpy(), acc_want)
+    _assert_bits_equal(host_bits(out), want, "forward")
 
 
 def test_qkv_scale_slots_follow_the_reference_rule_and_seg_variant():
@@ -456,21 +531,85 @@ def test_prefill_extreme_values_and_split_k_agreement():
     assert np.array_equal(acc_gemm, acc_splitk)
 
 
-@pytest.mark.parametrize("shape_id,m", [(0, 128), (1, 2048), (2, 128), (3, 512)])
+@pytest.mark.parametrize("shape_id", [0, 1, 2, 3])
+@pytest.mark.parametrize("m", [128, 512, 2048])
 def test_prefill_scaled_output_with_outliers(shape_id, m):
-    """Config 3: N(0,1) activations with 1% of entries x20, quantized per token
-    (two-kernel forward: the block is too large for the fused kernel)."""
+    """Config 3, all twelve (shape, M) pairs: N(0,1) activations with 1% of
+    entries x20, quantized per token, through BitLinearKernel.forward (quantizer
+    kernel + int8 MFMA GEMM) and through the accumulator export of the drop-in
+    entry: quantized rows, scales, int32 accumulators and bf16 outputs of every
+    row against the oracle, bit for bit."""
     sh = workload.shapes_2b()[shape_id]
     w = workload.ternary_weight(sh.K, sh.N, shape_id)
     ws_bits = workload.weight_scales(sh.K, sh.N, shape_id, sh.parts)
     xb = workload.activations_bf16(m, sh.K, shape_id, outliers=True)
     q, s_bits = o.quant_input(xb, o.QUANT_COMPILED)
-    _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    acc_want, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
     mod = bitlinear.BitLinearKernel(sh.K, sh.N).cuda()
     mod.weight.data = _packed_dev(w)
     mod.weight_scale.data = dev_bf16(ws_bits)
     out = mod(dev_bf16(xb))
+    assert bitlinear.last_kernel() == "gemm_i2_prefill_kernel"
     _assert_bits_equal(host_bits(out), want, f"{sh.name} prefill M={m}")
+    qd, sd = mod.quant_input(dev_bf16(xb))
+    assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(host_bits(sd).reshape(-1), s_bits)
+    acc = bitlinear.bitnet_int8xint2_acc(qd, mod.weight.data)
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+
+
+@pytest.mark.parametrize("shape_id", [0, 1, 2, 3])
+@pytest.mark.parametrize("m", [128, 512, 2048])
+def test_fp_path_agrees_with_the_int8_path(shape_id, m):
+    """The reference runs every M > 1 through its fp module (gpu/model.py:77-85,
+    chosen at gpu/generate.py:56-57): fake-quantized bf16 activations times
+    dequantised bf16 weights (gpu/convert_checkpoint.py:29-32), a bf16 GEMM with
+    fp32 accumulation.  The int8 path computes the same products exactly.  With
+    a = q / s the fake-quantized activation and w * ws the dequantised weight,
+    the fp result is  sum_k bf16(q_k / s) * bf16(w_k * ws)  and the int8 result
+    bf16(acc / s * ws):
+      * bf16(w * ws) = +-ws or 0 exactly (ws is a bf16 value), so the weight side adds no error;
+      * bf16(q / s) carries a relative rounding error of at most 2^-9 per element
+        (the reference rounds the fake-quantized activation to bf16), so the fp
+        sum differs from acc / s * ws by at most 2^-9 * sum_k |q_k w_k| / s * ws,
+        plus fp32 accumulation error (K * 2^-24 relative to the same sum, below
+        2^-11 here) and the final bf16 roundings of both results (2^-9 each,
+        relative to the result).
+    Asserted per element:  |fp - int8| <= 2^-8 * (sum_k |q_k w_k|) / s * ws + 2^-7 * |int8|.
+    The fp module quantizes in eager bf16 arithmetic, so the int8 side runs the
+    quantizer mode that is bit-identical to that (mode 1) and both sides see the
+    same integers q (asserted).  Config-3 data (1% outliers), every (shape, M) pair."""
+    sh = workload.shapes_2b()[shape_id]
+    w = workload.ternary_weight(sh.K, sh.N, shape_id)
+    ws_bits = workload.weight_scales(sh.K, sh.N, shape_id, sh.parts)
+    xb = workload.activations_bf16(m, sh.K, shape_id, outliers=True)
+    x = dev_bf16(xb)
+    wd = torch.from_numpy(w).cuda()
+    ws = dev_bf16(ws_bits)
+    # quantizer mode 1 = torch eager on bf16 tensors, which is how the fp module quantizes
+    mod = bitlinear.BitLinearKernel(sh.K, sh.N, quant_mode=bitlinear.QUANT_EAGER_BF16).cuda()
+    mod.weight.data = _packed_dev(w)
+    mod.weight_scale.data = ws
+    y_int8 = mod(x).float()
+    # the fp module with the weights its converter writes: per sub-tensor (w * scale) in bf16
+    # (equal slots here, as the int8 kernel indexes them: bitnet_kernels.h:80)
+    ws_num = _lib.load_library().bitlinear_ws_num(sh.N, sh.K)
+    slot = torch.arange(sh.N, device="cuda") // (sh.N // ws_num)
+    w_fp = (wd.to(torch.bfloat16) * ws[slot][:, None]).to(torch.bfloat16)
+    fp = bitlinear.BitLinear(sh.K, sh.N, bias=False, device="cuda", dtype=torch.bfloat16)
+    fp.weight.data = w_fp
+    with torch.no_grad():
+        y_fp = fp(x).float()
+    q, s = mod.quant_input(x)
+    # both paths multiply the same integers: the fake-quantized activation is bf16(q / s)
+    with torch.no_grad():
+        assert torch.equal(fp.quant_input(x), q.to(torch.bfloat16) / s)
+    mag = (q.double().abs() @ wd.double().abs().t()).float() / s.float() * ws[slot].float()[None, :]
+    bound = mag * 2.0 ** -8 + y_int8.abs() * 2.0 ** -7
+    excess = (y_fp - y_int8).abs() - bound
+    assert float(excess.max()) <= 0.0, f"fp vs int8: worst excess {float(excess.max())} at {sh.name} M={m}"
+    # and the bound is not vacuous: typical relative difference is far below one percent
+    rel = float((y_fp - y_int8).norm() / y_int8.norm())
+    assert rel < 4e-3, rel
 
 
 @pytest.mark.parametrize("m", [17, 24, 48, 100, 130, 250])
