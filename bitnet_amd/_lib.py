@@ -36,6 +36,10 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
+    "bitlinear_forward_bf16_static": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "bitlinear_norm_forward_bf16": (
         _c_int,
         [_c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,

@@ -32,6 +32,16 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
+// Scratch of bitlinear_forward_bf16_static: the quantized activations and their scales travel from
+// the quantizer kernel to the product kernel through this array instead of through workspaces that
+// a caller allocates.  Every GPU the library runs on holds its own copy, at its own address, until
+// the process ends.  Layout: bf16 scales of up to kStaticMaxTokens tokens, then the int8 rows.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+constexpr int kStaticMaxTokens = 16384;
+constexpr size_t kStaticScaleBytes = (size_t)kStaticMaxTokens * 2;
+constexpr size_t kStaticMaxElems = kStaticScratchBytes - kStaticScaleBytes;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 constexpr int kMaxSeg = 8;
@@ -1721,6 +1731,8 @@ const char* bitlinear_status_string(int status) {
         case BITLINEAR_ERR_NULL: return "null pointer";
         case BITLINEAR_ERR_LAUNCH: return "kernel launch failed";
         case BITLINEAR_ERR_ARG: return "invalid argument";
+        case BITLINEAR_ERR_SCRATCH:
+            return "activation block beyond the static scratch (need M <= 16384 and M * K <= 16744448)";
         default: return "unknown status";
     }
 }
@@ -1880,6 +1892,40 @@ static int forward_impl(const uint16_t* x, const int8_t* packed, uint16_t* outpu
 int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
                            int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
     return forward_impl(x, packed, output0, nullptr, ws, q_ws, s_ws, M, N, K, mode, stream);
+}
+
+// The array's name is only a handle on the host: its device address is looked up once per device
+// (each GPU has its own copy) and kept.
+static unsigned char* static_scratch_ptr(hipError_t* err) {
+    static std::once_flag flags[bitnet_host::kMaxDevices];
+    static unsigned char* ptrs[bitnet_host::kMaxDevices];
+    static hipError_t results[bitnet_host::kMaxDevices];
+    int dev = 0;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= bitnet_host::kMaxDevices) {
+        *err = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    std::call_once(flags[dev], [dev] {
+        void* p = nullptr;
+        results[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        ptrs[dev] = results[dev] == hipSuccess ? (unsigned char*)p : nullptr;
+    });
+    *err = results[dev];
+    return ptrs[dev];
+}
+
+int bitlinear_forward_bf16_static(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws, int M,
+                                  int N, int K, int mode, void* stream) {
+    if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
+    if (M > kStaticMaxTokens || (size_t)M * (size_t)K > kStaticMaxElems) return set_status(BITLINEAR_ERR_SCRATCH);
+    if (!x || !packed || !output0 || !ws) return set_status(BITLINEAR_ERR_NULL);
+    hipError_t err = hipSuccess;
+    unsigned char* base = static_scratch_ptr(&err);
+    if (err != hipSuccess || !base) return set_status(BITLINEAR_ERR_LAUNCH);
+    return forward_impl(x, packed, output0, nullptr, ws, (int8_t*)(base + kStaticScaleBytes), (uint16_t*)base, M, N, K, mode,
+                        stream);
 }
 
 int bitlinear_forward_bf16_acc_i32(const uint16_t* x, const int8_t* packed, int32_t* acc_out, uint16_t* output0,

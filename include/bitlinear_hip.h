@@ -30,6 +30,8 @@ extern "C" {
 #define BITLINEAR_ERR_LAUNCH 3  /* the HIP runtime refused the launch       */
 #define BITLINEAR_ERR_ARG 4     /* bad mode / segment list / tuning value, or
                                    an operand not 16-byte aligned           */
+#define BITLINEAR_ERR_SCRATCH 5 /* bitlinear_forward_bf16_static: the
+                                   activation block exceeds the static scratch */
 
 /*
  * Drop-in replacement for the reference's only exported symbol
@@ -129,6 +131,28 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
                            uint16_t* output0, const uint16_t* ws,
                            int8_t* q_ws, uint16_t* s_ws,
                            int M, int N, int K, int mode, void* stream);
+
+/*
+ * bitlinear_forward_bf16 without workspace arguments, for callers that cannot
+ * allocate device memory at all (code under graph capture that owns no
+ * buffers of its own, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference, whose host shim allocates per call
+ * (gpu/model.py:33).  The quantized rows and their scales, which
+ * bitlinear_forward_bf16 keeps in q_ws / s_ws, live in a 16 MiB array inside
+ * the library's device image (one copy per GPU, held until the process ends).
+ * Limits: M <= 16384 tokens and M * K <= 16744448 activation elements (the
+ * largest prompt block of the 2B shapes, 2048 x 6912, fits); beyond them the
+ * call launches nothing and returns BITLINEAR_ERR_SCRATCH.  Same kernels and
+ * the same bits as bitlinear_forward_bf16.  Allocates nothing and frees
+ * nothing; the first call on a device looks the array's address up (a host
+ * call, not stream work).  All calls on one GPU share the array: two of them
+ * must not overlap in time (same stream, or ordered by events), or they race
+ * on the quantized rows.  Nothing in the array needs clearing between calls:
+ * every element the product reads was written by the same call's quantizer.
+ */
+int bitlinear_forward_bf16_static(const uint16_t* x, const int8_t* packed,
+                                  uint16_t* output0, const uint16_t* ws,
+                                  int M, int N, int K, int mode, void* stream);
 
 /*
  * bitlinear_forward_bf16 that also stores the int32 accumulators of the product

@@ -84,6 +84,10 @@ def test_argument_checks_need_no_gpu(capfd):
     assert lib.bitlinear_quant_absmax(None, None, None, 1, 2560, 0, None) == 2
     assert lib.bitlinear_quant_absmax(None, None, None, 1, 2563, 0, None) == 1
     assert lib.bitlinear_int8xint2_acc_i32(None, None, None, None, None, None, 1, 2560, 100, None) == 1
+    # the allocation-free forward: sizes beyond its static scratch, then nulls, before any HIP call
+    assert lib.bitlinear_forward_bf16_static(None, None, None, None, 16385, 2560, 64, 0, None) == 5
+    assert lib.bitlinear_forward_bf16_static(None, None, None, None, 4096, 2560, 4160, 0, None) == 5
+    assert lib.bitlinear_forward_bf16_static(None, None, None, None, 2048, 2560, 6912, 0, None) == 2
 
 
 def test_decoder_entry_argument_checks_need_no_gpu():
