@@ -84,7 +84,26 @@ SIGNATURES = {
     "bitnet_lm_head_workgroups": (_c_int, [_c_int]),
     "bitnet_lm_head_set_kernel": (_c_int, [_c_int]),
     "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
+    "bitlinear_int8xint2_grouped": (_c_int, [_c_ptr, _c_int, _c_ptr]),
+    # include/bitlinear_probes.h
+    "bitlinear_probe_empty": (_c_int, [_c_int, _c_int, _c_ptr]),
+    "bitlinear_probe_weight_stream": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
 }
+
+
+class Problem(ctypes.Structure):
+    """struct bitlinear_problem of include/bitlinear_hip.h."""
+
+    _fields_ = [
+        ("input0", _c_ptr),
+        ("input1", _c_ptr),
+        ("output0", _c_ptr),
+        ("s", _c_ptr),
+        ("ws", _c_ptr),
+        ("M", _c_int),
+        ("N", _c_int),
+        ("K", _c_int),
+    ]
 
 _lib = None
 

@@ -27,6 +27,7 @@
 #include <stdio.h>
 
 #include "bitlinear_hip.h"
+#include "bitlinear_probes.h"
 #include "host_util.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -251,6 +252,214 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
         if (acc_out) acc_out[(size_t)e_m * N + e_n] = sum;
         if (out) out[(size_t)e_m * N + e_n] = f32_to_bf16_rne((float)sum / bf16_to_f32(e_sb) * bf16_to_f32(e_wsb));
     }
+}
+
+// ---------------------------------------------------------------------------
+// Streaming kernel (M <= 4 tokens): waves that own whole 16-row blocks and never meet
+// ---------------------------------------------------------------------------
+// For matrices (or groups of matrices) large enough to be bandwidth-bound.  A work item is one
+// 16-row block of one problem: 4 * K contiguous bytes.  A workgroup of four waves belongs to one
+// problem; each of its waves takes a run of consecutive row blocks and walks them with ONE software
+// pipeline that does not stop at item boundaries: a ring of D 16-byte weight loads per lane (D KB per
+// wave, the lanes of one load covering 1 KB = 16 rows x 256 k), each slot re-requested for the next
+// round of k-steps -- or for the first round of the wave's next row block -- right after the MFMAs
+// that consumed it.  The operand scheme is the decode kernel's: the four words of a lane's 16 bytes
+// are rows 4q..4q+3 of one 16-k chunk and feed four MFMAs whose B operand carries token m's chunk at
+// column 4 * sigma + m, so only the diagonal blocks of the results are read.  The problem's int8
+// activation rows are copied into LDS once per workgroup (requested before the weights, so that they
+// are not queued behind them: loads return in the order of their requests), with sum(a) per token
+// taken on the way (it removes the +2 of the stored codes); after that single barrier no wave waits
+// for another, and the only other LDS traffic is each wave's own 1 KB transposition of its diagonal
+// results.  Several problems of one shape (a grouped launch) are the grid's second dimension.
+constexpr int kStreamMaxProblems = 48;  // the operands of a grouped launch travel as kernel arguments
+constexpr int kStreamMaxTokens = 4;
+constexpr int kStreamMaxActBytes = 32768;  // M * K: at most 8 16-byte pieces per thread of the staging pass
+constexpr int kStreamRowPad = 64;          // bytes between token rows in LDS beyond K: the 4 tokens of a read hit different banks
+struct StreamProblem {
+    const int8_t* act;     // int8 [M, K]
+    const int8_t* packed;  // packed weight [N, K/4]
+    uint16_t* out;         // bf16 [M, N] or nullptr
+    const uint16_t* s;     // bf16 [M]
+    const uint16_t* ws;    // bf16 weight scales
+};
+struct StreamArgs {
+    int M, N, K;
+    int blocks16;     // N / 16: items per problem
+    int ipw;          // consecutive items per wave
+    int rounds;       // rounds of D 256-k steps per item
+    int steps;        // ceil(K / 256)
+    int pad_;
+    int32_t* acc_out;  // int32 [M, N] of problem 0, or nullptr
+    ScaleMap smap;     // every boundary a multiple of 16
+    StreamProblem p[kStreamMaxProblems];
+};
+
+template <int D, bool COMPUTE>
+__global__ __launch_bounds__(256) void gemv_i2_stream_kernel(const StreamArgs a, uint32_t* __restrict__ sink) {
+    extern __shared__ __attribute__((aligned(16))) int8_t lds_act[];  // [M][K + pad] + tail
+    __shared__ __attribute__((aligned(16))) int red[4][256];         // per wave: [G][token][row]
+    __shared__ int wave_part[4][kStreamMaxTokens];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int pid = blockIdx.y;
+    int rb = (blockIdx.x * 4 + wave) * a.ipw;
+    const int rb_end = (rb + a.ipw) < a.blocks16 ? (rb + a.ipw) : a.blocks16;
+    const bool have_items = rb < rb_end;  // uniform over the wave
+    const int g = lane >> 4;
+    const int sg = (lane >> 2) & 3;
+    const int q = lane & 3;
+    const int chunk = 4 * g + sg;  // 16-k chunk inside a 256-k step
+    // 16-byte group of (row quad q, chunk) inside the step's 1 KB: tile chunk / 2, k-half chunk & 1
+    const int w_voff = ((chunk >> 1) * 8 + (q >> 1) * 4 + (chunk & 1) * 2 + (q & 1)) * 16;
+    const int tokB = q < a.M ? q : a.M - 1;  // columns of tokens >= M are never read
+    const int kp = a.K + kStreamRowPad;
+    const int wbytes = a.K * 4;  // one 16-row block
+    const StreamProblem prob = a.p[pid];
+
+    // Descriptors span exactly one row block: a k-step past the end of K is out of range and reads as
+    // zero weights (which contribute nothing, whatever the B operand holds), and the requests of a
+    // wave that has run out of row blocks go to an empty descriptor: no memory access.
+    auto w_desc = [&](int rb_, bool valid) {
+        return __builtin_amdgcn_make_buffer_rsrc((void*)(prob.packed + (size_t)rb_ * (size_t)wbytes), 0, valid ? wbytes : 0,
+                                                 0x00020000);
+    };
+
+    // the activation block first (it comes from cache and must not queue behind the weights) ...
+    constexpr int kPieces = kStreamMaxActBytes / 16 / 256;  // 16-byte pieces per thread
+    v4i piece[kPieces];
+    int prow[kPieces], pdst[kPieces];
+    uint16_t e_sb = 0, e_wb = 0;
+    if (COMPUTE) {
+        const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)prob.act, 0, a.M * a.K, 0x00020000);
+        const int kp16 = a.K >> 4;
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+            const int pc = tid + i * 256;
+            const int row = (pc >= kp16 ? 1 : 0) + (pc >= 2 * kp16 ? 1 : 0) + (pc >= 3 * kp16 ? 1 : 0);
+            prow[i] = pc < a.M * kp16 ? row : -1;
+            pdst[i] = row * kp + (pc - row * kp16) * 16;
+            piece[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, pc * 16, 0, 0));  // past the end: zeros
+        }
+        // (unconditional: a call without output hands in addresses that exist; a load under a branch would
+        // be waited for inside the branch, in front of the weight requests)
+        e_sb = prob.s[tokB];
+        e_wb = prob.ws[(lane & 7) < a.smap.nseg ? (lane & 7) : 0];
+    }
+    // ... then the first round of weight words
+    v4u w[D];
+    __amdgpu_buffer_rsrc_t cw = w_desc(have_items ? rb : 0, have_items);
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        w[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(cw, w_voff, j * 1024, 2 /* nt */));
+        __builtin_amdgcn_sched_barrier(0);  // requested in the order in which the slots are consumed
+    }
+    int rowsum2_tok = 0;  // twice the sum of the int8 row of this lane's token (lane & 3)
+    float e_sf = 1.0f;    // that token's activation scale
+    uint32_t e_wsv = 0;   // lane j < nseg: weight scale of slot j, as fp32 bits
+    if (COMPUTE) {
+        int part[kStreamMaxTokens] = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+            if (prow[i] >= 0) *(v4i*)(lds_act + pdst[i]) = piece[i];
+            const int ones = 0x01010101;
+            int d = __builtin_amdgcn_sdot4(piece[i].x, ones, 0, false);
+            d = __builtin_amdgcn_sdot4(piece[i].y, ones, d, false);
+            d = __builtin_amdgcn_sdot4(piece[i].z, ones, d, false);
+            d = __builtin_amdgcn_sdot4(piece[i].w, ones, d, false);
+#pragma unroll
+            for (int m = 0; m < kStreamMaxTokens; ++m) part[m] += prow[i] == m ? d : 0;
+        }
+#pragma unroll
+        for (int m = 0; m < kStreamMaxTokens; ++m) {
+            const int tot = wave_sum_i32(part[m]);
+            if (lane == 0) wave_part[wave][m] = tot;
+        }
+        e_sf = bf16_to_f32(e_sb);
+        e_wsv = ((uint32_t)e_wb) << 16;
+        lds_barrier();  // LDS only: the weight words stay in flight
+        rowsum2_tok = 2 * (wave_part[0][q] + wave_part[1][q] + wave_part[2][q] + wave_part[3][q]);
+    }
+    if (!have_items) return;  // behind the only barrier
+
+    const int8_t* bp = lds_act + tokB * kp + chunk * 16;
+    uint32_t x_acc = 0;  // load-only variant: something that depends on every byte
+    for (; rb < rb_end; ++rb) {
+        const bool nvalid = (rb + 1) < rb_end;
+        const __amdgpu_buffer_rsrc_t nw = w_desc(nvalid ? rb + 1 : rb, nvalid);
+        v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0}, acc3 = {0, 0, 0, 0};
+        for (int sub = 0; sub < a.rounds; ++sub) {
+            // what the ring requests while this round is multiplied: the row block's next round, or the
+            // first round of the wave's next row block
+            const bool last = (sub + 1) == a.rounds;
+            const __amdgpu_buffer_rsrc_t rw = last ? nw : cw;
+            const int so = last ? 0 : (sub + 1) * D;
+            const int st0 = sub * D;
+            v4i bcur;
+            if (COMPUTE) bcur = *(const v4i*)(bp + (st0 < a.steps ? st0 : a.steps - 1) * 256);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < D; ++j) {
+                const uint32_t wd[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
+                if (COMPUTE) {
+                    // the next step's B operand is read while this step is multiplied (a step past the
+                    // end re-reads the last one: its weights are zero)
+                    const int stn = st0 + j + 1;
+                    const v4i bnext = *(const v4i*)(bp + (stn < a.steps ? stn : a.steps - 1) * 256);
+                    v4i e[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        e[i].x = (int)(wd[i] & 0x03030303u);
+                        e[i].y = (int)((wd[i] >> 2) & 0x03030303u);
+                        e[i].z = (int)((wd[i] >> 4) & 0x03030303u);
+                        e[i].w = (int)((wd[i] >> 6) & 0x03030303u);
+                    }
+                    w[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, (so + j) * 1024, 2 /* nt */));
+                    acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(e[0], bcur, acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(e[1], bcur, acc1, 0, 0, 0);
+                    acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(e[2], bcur, acc2, 0, 0, 0);
+                    acc3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(e[3], bcur, acc3, 0, 0, 0);
+                    bcur = bnext;
+                } else {
+                    x_acc ^= wd[0] ^ wd[1] ^ wd[2] ^ wd[3];
+                    w[j] = __builtin_bit_cast(v4u, __builtin_amdgcn_raw_buffer_load_b128(rw, w_voff, (so + j) * 1024, 2 /* nt */));
+                }
+                __builtin_amdgcn_sched_barrier(0);  // the slot's re-request stays where it is written: right behind its use
+            }
+        }
+        if (COMPUTE) {
+            // result lane 16 G + p' holds A-rows 4 G + r (r = register); the diagonal blocks (sigma' == G) sit in
+            // the lanes with g == sg, token q; register r of MFMA i is weight row 4 r + i
+            int* my = red[wave];
+            if (sg == g) {
+                int* dst = my + (g * 4 + q) * 16;
+                *(v4i*)(dst + 0) = v4i{acc0.x, acc1.x, acc2.x, acc3.x};
+                *(v4i*)(dst + 4) = v4i{acc0.y, acc1.y, acc2.y, acc3.y};
+                *(v4i*)(dst + 8) = v4i{acc0.z, acc1.z, acc2.z, acc3.z};
+                *(v4i*)(dst + 12) = v4i{acc0.w, acc1.w, acc2.w, acc3.w};
+            }
+            // the same wave wrote and reads: LDS operations of a wave complete in order
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int row = lane >> 2;  // token = q
+            const int sum = my[(0 * 4 + q) * 16 + row] + my[(1 * 4 + q) * 16 + row] + my[(2 * 4 + q) * 16 + row] +
+                            my[(3 * 4 + q) * 16 + row] - rowsum2_tok;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int n = rb * 16 + row;
+            const int slot = scale_slot_uniform(a.smap, rb * 16);
+            const float wsf = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)e_wsv, slot));
+            if (q < a.M) {
+                const size_t o = (size_t)q * a.N + n;
+                if (a.acc_out && pid == 0) a.acc_out[o] = sum;
+                if (prob.out) prob.out[o] = f32_to_bf16_rne((float)sum / e_sf * wsf);
+            }
+        }
+        cw = nw;
+    }
+    if (!COMPUTE && x_acc == 0x9e3779b9u && sink) sink[0] = x_acc;  // keeps the loads alive; practically never taken
 }
 
 // ---------------------------------------------------------------------------
@@ -1310,6 +1519,8 @@ struct Tuning {
     int prefill_ks = 0;    // groups of waves splitting K in the small prefill tiles, 0 = built-in choice
     int staged = 0;        // product through the LDS-staged kernel: 0 = built-in choice, 1 = whenever it fits, 2 = never
     int stream = 0;        // product through the streaming kernel: 0 = built-in choice, 1 = whenever it applies, 2 = never
+    int stream_depth = 0;  // its ring depth (0 = built-in choice)
+    int stream_waves = 0;  // its waves per CU (0 = built-in choice)
 };
 std::mutex g_tuning_mutex;
 Tuning g_tuning_shared;
@@ -1320,6 +1531,11 @@ void refresh_tuning() {
 }
 
 using bitnet_host::OncePerDevice;
+// Row blocks from which ONE call goes through the streaming kernel (measured at M = 1: 55296 x 5120, 3456
+// row blocks: 12.7 us against 13.3 with the LDS-staged kernel's many small workgroups, at 4 tokens 13.0
+// against 15.4; 20480 x 3200, 1280 row blocks: 6.5 against 5.0 -- with few row blocks per CU the waves
+// that split K finish earlier).  Grouped calls take it from two problems on.
+constexpr int kStreamMinBlocks = 2048;
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 constexpr int kPrefillFewTiles = 330;   // up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles
 constexpr int kPrefillSplit2Tiles = 320;  // up to this many 32 x 128 tiles two groups of waves split a tile's K,
@@ -1657,6 +1873,71 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
+// Streaming kernel: applicability and launch.  D (loads in flight per lane) is chosen so that the
+// rounds of D steps cover the ceil(K / 256) steps of a row block with the fewest idle steps.
+bool stream_applicable(int M, int N, int K, const ScaleMap& smap) {
+    if (M < 1 || M > kStreamMaxTokens) return false;
+    if ((long long)M * K > kStreamMaxActBytes) return false;  // the activation block lives in LDS
+    for (int j = 0; j < smap.nseg; ++j)
+        if (smap.ends[j] % 16) return false;  // the kernel takes one scale slot per 16-row block
+    (void)N;
+    return true;
+}
+
+int launch_stream(const StreamProblem* probs, int nprob, int M, int N, int K, const ScaleMap& smap, int32_t* acc_out,
+                  hipStream_t stream, bool compute = true, uint32_t* sink = nullptr) {
+    if (nprob < 1 || nprob > kStreamMaxProblems) return BITLINEAR_ERR_ARG;
+    const int steps = (K + 255) / 256;
+    // D (loads in flight per lane): the rounds of D steps should cover the steps of a row block with few
+    // idle steps; among equals the first of this list
+    const int depths[6] = {5, 6, 7, 4, 8, 10};
+    int depth = 5, best = 1 << 30;
+    for (int i = 0; i < 6; ++i) {
+        const int rounds = (steps + depths[i] - 1) / depths[i];
+        const int waste = rounds * depths[i] - steps;
+        if (waste < best) {
+            best = waste;
+            depth = depths[i];
+        }
+    }
+    if (t_tune.stream_depth > 0) depth = t_tune.stream_depth;
+    StreamArgs a;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.blocks16 = N / 16;
+    a.steps = steps;
+    a.pad_ = 0;
+    // waves the launch is sized for, over all problems: a run of row blocks per wave
+    const int waves_per_cu = t_tune.stream_waves > 0 ? t_tune.stream_waves : 8;
+    const long long total_items = (long long)nprob * a.blocks16;
+    const int max_waves = 256 * waves_per_cu;
+    a.ipw = (int)((total_items + max_waves - 1) / max_waves);
+    a.rounds = (steps + depth - 1) / depth;
+    a.acc_out = acc_out;
+    a.smap = smap;
+    for (int i = 0; i < kStreamMaxProblems; ++i) a.p[i] = probs[i < nprob ? i : 0];
+    const int waves = (a.blocks16 + a.ipw - 1) / a.ipw;  // per problem
+    const dim3 grid((waves + 3) / 4, nprob, 1), block(256, 1, 1);
+    const size_t lds = compute ? (size_t)M * (K + kStreamRowPad) + 256 : 0;
+    g_last_kernel = "gemv_i2_stream_kernel";
+#define BITLINEAR_LAUNCH_STREAM(DD)                                                                      \
+    if (compute)                                                                                         \
+        hipLaunchKernelGGL((gemv_i2_stream_kernel<DD, true>), grid, block, lds, stream, a, sink);        \
+    else                                                                                                 \
+        hipLaunchKernelGGL((gemv_i2_stream_kernel<DD, false>), grid, block, lds, stream, a, sink)
+    switch (depth) {
+        case 4: BITLINEAR_LAUNCH_STREAM(4); break;
+        case 6: BITLINEAR_LAUNCH_STREAM(6); break;
+        case 7: BITLINEAR_LAUNCH_STREAM(7); break;
+        case 8: BITLINEAR_LAUNCH_STREAM(8); break;
+        case 10: BITLINEAR_LAUNCH_STREAM(10); break;
+        default: BITLINEAR_LAUNCH_STREAM(5); break;
+    }
+#undef BITLINEAR_LAUNCH_STREAM
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
 int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                 const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream,
                 const uint16_t* residual = nullptr) {
@@ -1686,6 +1967,14 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // The kernel that stages the int8 rows in LDS once per workgroup and shares
     // them between several row blocks: fewer activation bytes through L2 than
     // the kernels below, which read their B operands straight from global.
+    // Bandwidth-bound sizes at up to four tokens: waves that stream whole row blocks
+    if (t_tune.stream != 2 && t_tune.path == 0 && !residual && stream_applicable(M, N, K, smap)) {
+        const bool wanted = t_tune.stream == 1 || (N / 16) >= kStreamMinBlocks;
+        if (wanted) {
+            const StreamProblem one = {act, packed, out, out ? s : (const uint16_t*)packed, out ? ws : (const uint16_t*)packed};
+            return launch_stream(&one, 1, M, N, K, smap, acc_out, stream);
+        }
+    }
     // (The accumulator export takes the same kernel choice as the drop-in call, so what the parity
     // tests read is what the drop-in entry computes.  Without an output there are no scales: the
     // kernel's unconditional scale requests then go to an address that exists.)
@@ -1720,6 +2009,35 @@ ScaleMap equal_slots(int N, int ws_num) {
 
 extern "C" {
 
+// Measurement probes (declared in include/bitlinear_probes.h): what a launch costs when the kernel does
+// nothing, and when it only requests a matrix's bytes with the streaming kernel's access pattern.
+__global__ void probe_empty_kernel() {}
+
+int bitlinear_probe_empty(int blocks, int threads, void* stream) {
+    if (blocks < 1 || threads < 1 || threads > 1024) return BITLINEAR_ERR_ARG;
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream);
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+int bitlinear_probe_weight_stream(const int8_t* const* packed, int count, int N, int K, uint32_t* sink, void* stream) {
+    refresh_tuning();
+    if (!shape_ok(1, N, K)) return BITLINEAR_ERR_SHAPE;
+    if (!packed || count < 1 || count > kStreamMaxProblems) return BITLINEAR_ERR_ARG;
+    StreamProblem sp[kStreamMaxProblems];
+    for (int i = 0; i < count; ++i) {
+        if (!packed[i] || (((uintptr_t)packed[i]) & 15u)) return BITLINEAR_ERR_ARG;
+        sp[i] = StreamProblem{packed[i], packed[i], nullptr, nullptr, nullptr};
+    }
+    // Nothing is multiplied, so a row block need not be a real one: with few row blocks the same bytes are
+    // read as more, shorter pieces (a row block cut into 2, 4, ... runs of k), so that the probe stands for
+    // the fastest way of requesting these bytes, not for one kernel's decomposition.
+    while ((long long)count * (N / 16) < 2048 && (K % 128) == 0 && K >= 2048) {
+        N *= 2;
+        K /= 2;
+    }
+    return launch_stream(sp, count, 1, N, K, equal_slots(N, 1), nullptr, (hipStream_t)stream, false, sink);
+}
+
 int bitlinear_last_status(void) { return g_status; }
 
 const char* bitlinear_last_kernel(void) { return g_last_kernel; }
@@ -1747,7 +2065,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = 0;
+        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -1756,8 +2074,11 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 7) {
-        if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
+        const bool depth_ok = b == 0 || b == 4 || b == 5 || b == 6 || b == 7 || b == 8 || b == 10;
+        if (a < 0 || a > 2 || !depth_ok || c < 0 || c > 32) return set_status(BITLINEAR_ERR_ARG);
         g.stream = a;
+        g.stream_depth = b;
+        g.stream_waves = c;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 1) {
@@ -1828,6 +2149,48 @@ void bitlinear_int8xint2(int8_t* input0, int8_t* input1, uint16_t* output0, uint
     }
     set_status(launch_gemv(input0, input1, output0, nullptr, s, ws, equal_slots(N, bitlinear_ws_num(N, K)), M, N, K,
                            (hipStream_t)stream));
+}
+
+int bitlinear_int8xint2_grouped(const bitlinear_problem* problems, int count, void* stream) {
+    refresh_tuning();
+    if (count < 0) return set_status(BITLINEAR_ERR_ARG);
+    if (count == 0) return set_status(BITLINEAR_OK);
+    if (!problems) return set_status(BITLINEAR_ERR_NULL);
+    // everything is checked before anything is launched
+    for (int i = 0; i < count; ++i) {
+        const bitlinear_problem& p = problems[i];
+        if (!shape_ok(p.M, p.N, p.K)) return set_status(BITLINEAR_ERR_SHAPE);
+        if (!p.input0 || !p.input1 || !p.output0 || !p.s || !p.ws) return set_status(BITLINEAR_ERR_NULL);
+        if ((((uintptr_t)p.input0) | ((uintptr_t)p.input1)) & 15u) return set_status(BITLINEAR_ERR_ARG);
+    }
+    int i = 0;
+    while (i < count) {
+        const bitlinear_problem& p0 = problems[i];
+        const ScaleMap sm = equal_slots(p0.N, bitlinear_ws_num(p0.N, p0.K));
+        // a run of problems of one shape is one launch of the streaming kernel (one flat list of row blocks)
+        int j = i + 1;
+        while (j < count && j - i < kStreamMaxProblems && problems[j].M == p0.M && problems[j].N == p0.N &&
+               problems[j].K == p0.K)
+            ++j;
+        const bool grouped = t_tune.stream != 2 && t_tune.path == 0 && stream_applicable(p0.M, p0.N, p0.K, sm) &&
+                             (j - i > 1 || t_tune.stream == 1 || (p0.N / 16) >= kStreamMinBlocks);
+        if (grouped) {
+            StreamProblem sp[kStreamMaxProblems];
+            for (int k = i; k < j; ++k)
+                sp[k - i] = StreamProblem{problems[k].input0, problems[k].input1, problems[k].output0, problems[k].s, problems[k].ws};
+            const int st = launch_stream(sp, j - i, p0.M, p0.N, p0.K, sm, nullptr, (hipStream_t)stream);
+            if (st != BITLINEAR_OK) return set_status(st);
+        } else {
+            for (int k = i; k < j; ++k) {
+                const bitlinear_problem& p = problems[k];
+                const int st = launch_gemv(p.input0, p.input1, p.output0, nullptr, p.s, p.ws, sm, p.M, p.N, p.K,
+                                           (hipStream_t)stream);
+                if (st != BITLINEAR_OK) return set_status(st);
+            }
+        }
+        i = j;
+    }
+    return set_status(BITLINEAR_OK);
 }
 
 int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1, uint16_t* output0, const uint16_t* s,

@@ -87,6 +87,28 @@ int bitlinear_int8xint2_acc_i32(const int8_t* input0, const int8_t* input1,
 const char* bitlinear_last_kernel(void);
 
 /*
+ * Several products in one call.  Each element is one bitlinear_int8xint2 call
+ * (same operands, same meaning, same results bit for bit); consecutive
+ * elements of equal (M, N, K) with M <= 4 are executed by ONE kernel launch
+ * whose waves walk the row blocks of all of them as one list (up to 48
+ * problems per launch; longer runs take several), other elements are launched
+ * one by one.  The problems of a call must be independent of each other: no
+ * output0 may be an input of another element.  The reference has no such
+ * entry: it launches one kernel per BitLinear (gpu/model.py:128, 160, 193,
+ * 196), each far smaller than what MI355X must have in flight to use its HBM.
+ * `problems` is a host array, read during the call only.
+ */
+typedef struct bitlinear_problem {
+    const int8_t* input0;   /* int8 [M, K] */
+    const int8_t* input1;   /* packed ternary weight [N, K/4] */
+    uint16_t* output0;      /* bf16 [M, N] */
+    const uint16_t* s;      /* bf16 [M] */
+    const uint16_t* ws;     /* bf16, at least bitlinear_ws_num(N, K) entries */
+    int M, N, K;
+} bitlinear_problem;
+int bitlinear_int8xint2_grouped(const bitlinear_problem* problems, int count, void* stream);
+
+/*
  * Variant with explicit weight-scale segments: row n uses ws[j] for the first
  * j with n < seg_ends[j]  (seg_ends ascending, seg_ends[nseg-1] == N,
  * 1 <= nseg <= 8, host array).  This is the scale layout
@@ -211,6 +233,12 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *   kernel 6: product of int8 rows (M <= 16) through the kernel that stages
  *             them in LDS: a = 0 built-in choice (M > 4 and N >= 6912), 1 whenever it
  *             fits, 2 never.  Independent of kernels 1..5; kernel 0 resets it.
+ *   kernel 7: product of int8 rows (M <= 4) through the streaming kernel (one
+ *             wave per 16-row block, no staging): a = 0 built-in choice, 1
+ *             whenever it applies, 2 never (also in grouped calls); b = loads in
+ *             flight per lane (0 = built-in choice, or 4, 5, 6, 7, 8, 10); c = waves
+ *             per CU the launch is sized for (0 = built-in choice, up to 32).
+ *             Applies with kernel 0 only; kernel 0 resets it.
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 

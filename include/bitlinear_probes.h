@@ -1,0 +1,36 @@
+/*
+ * Measurement probes of libbitlinear_hip.so.  Not part of the drop-in interface
+ * (the reference has no counterpart): bench.py uses them to measure, in the same
+ * run and launch style as its headline, what a kernel launch costs on this
+ * machine when the kernel does nothing and when it only requests a matrix's
+ * bytes.  Same conventions as include/bitlinear_hip.h: device pointers owned by
+ * the caller, no allocation, no synchronisation, launches on the given stream.
+ */
+#ifndef BITLINEAR_PROBES_H
+#define BITLINEAR_PROBES_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* One launch of a kernel with an empty body: `blocks` workgroups of `threads`
+ * threads (1..1024).  Returns 0, 3 (launch failed) or 4 (bad argument). */
+int bitlinear_probe_empty(int blocks, int threads, void* stream);
+
+/*
+ * One launch that requests every byte of `count` (1..48) packed weights of
+ * shape [N, K/4] (host array of device pointers) with the streaming product
+ * kernel's own grid, access pattern and software pipeline, and does nothing
+ * with them beyond an exclusive-or that keeps the requests alive: no
+ * activation operand, no decode, no MFMA, no output.  sink: one device word
+ * that is practically never written (may be NULL).  Returns a BITLINEAR_* code.
+ */
+int bitlinear_probe_weight_stream(const int8_t* const* packed, int count, int N, int K,
+                                  uint32_t* sink, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITLINEAR_PROBES_H */

@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def _declared_functions():
     names = []
-    for header in ("bitlinear_hip.h", "bitnet_decoder_ops.h"):
+    for header in ("bitlinear_hip.h", "bitnet_decoder_ops.h", "bitlinear_probes.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names += re.findall(r"\b(bit(?:linear|net)_[a-z0-9_]+)\s*\(", text)

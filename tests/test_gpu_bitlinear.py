@@ -774,6 +774,162 @@ def test_product_through_the_lds_staged_kernel(n, k, m, staged):
     _assert_bits_equal(host_bits(out), want, f"staged={staged} M={m}")
 
 
+@pytest.mark.parametrize("depth,waves", [(0, 0), (4, 3), (7, 16), (10, 1)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("n,k", [(16, 64), (48, 192), (32, 3200), (1040, 256), (3840, 2560), (2560, 6912), (20480, 3200)])
+def test_streaming_kernel_bit_exact(n, k, m, depth, waves):
+    """The streaming kernel (one wave per 16-row block, activations in LDS, a
+    ring of weight loads that runs across row blocks) forced for shapes it would
+    not be chosen for: a single row block, a K of one partial step, 12.5 steps,
+    runs of one to several row blocks per wave, every ring depth; three scale
+    slots at 3840 x 2560.  Accumulators and scaled outputs bit for bit."""
+    if (n, k) in ((3840, 2560), (2560, 6912), (20480, 3200)) and (depth, waves) not in ((0, 0), (7, 16)):
+        pytest.skip("large shapes: two launch shapes are enough")
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=n + 3 * k + m)
+    s_bits = o.f32_to_bf16_bits(np.linspace(3.0, 90.0, m).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    acc_want, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    pk, ad = _packed_dev(w), dev_i8(a)
+    try:
+        assert lib.bitlinear_set_tuning(7, 1, depth, waves) == 0
+        out = bitlinear.bitnet_int8xint2_linear(ad, pk, dev_bf16(s_bits), dev_bf16(ws_bits))
+        assert bitlinear.last_kernel() == "gemv_i2_stream_kernel"
+        acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
+        assert bitlinear.last_kernel() == "gemv_i2_stream_kernel"
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    _assert_bits_equal(host_bits(out), want, f"stream N={n} K={k} M={m}")
+
+
+def test_streaming_kernel_is_the_choice_for_the_largest_shape_and_respects_segments():
+    """55296 x 5120 (bitnet_kernels.cu:32) at up to four tokens goes through the
+    streaming kernel by itself; five tokens do not.  Checked against the integer
+    product computed on the device in fp64 (exact).  Scale segments that are not
+    multiples of 16 rows keep the call away from it (it takes one slot per row block)."""
+    lib = _lib.load_library()
+    n, k = 55296, 5120
+    g = torch.Generator(device="cuda").manual_seed(55296)
+    w = torch.randint(-1, 2, (n, k), generator=g, device="cuda", dtype=torch.int8)
+    pk = pack_weight.convert_weight_int8_to_int2(w, keep_device=True)
+    ws = torch.tensor([0.0161, 0.0, 0.0, 0.0], device="cuda").to(torch.bfloat16)
+    for m, want_kernel in ((1, "gemv_i2_stream_kernel"), (4, "gemv_i2_stream_kernel"), (5, None)):
+        a = torch.randint(-128, 128, (m, k), generator=g, device="cuda", dtype=torch.int8)
+        s = (torch.rand(m, generator=g, device="cuda") * 50 + 2).to(torch.bfloat16)
+        acc_want = (a.double() @ w.double().t())
+        y = bitlinear.bitnet_int8xint2_linear(a, pk, s, ws)
+        if want_kernel:
+            assert bitlinear.last_kernel() == want_kernel
+        else:
+            assert bitlinear.last_kernel() != "gemv_i2_stream_kernel"
+        assert torch.equal(bitlinear.bitnet_int8xint2_acc(a, pk), acc_want.to(torch.int32))
+        want_y = (acc_want.float() / s.float()[:, None] * ws[0].float()).to(torch.bfloat16)
+        assert torch.equal(y.view(torch.int16), want_y.view(torch.int16))
+    # segments
+    n2, k2 = 3840, 2560
+    w2, a2 = _rand_case(n2, k2, 2, seed=11)
+    s_bits = o.f32_to_bf16_bits(np.array([3.25, 17.5], dtype=np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.011, 0.023, 0.037, 0.0], dtype=np.float32))
+    pk2 = _packed_dev(w2)
+    try:
+        assert lib.bitlinear_set_tuning(7, 1, 0, 0) == 0
+        for ends, streams in (([2560, 3200, 3840], True), ([1000, 3001, 3840], False)):
+            _, want_seg = o.bitlinear_int8xint2_seg(a2, w2, s_bits, ws_bits, ends)
+            out_seg = bitlinear.bitnet_int8xint2_linear_seg(dev_i8(a2), pk2, dev_bf16(s_bits), dev_bf16(ws_bits), ends)
+            assert (bitlinear.last_kernel() == "gemv_i2_stream_kernel") == streams
+            _assert_bits_equal(host_bits(out_seg), want_seg, f"segments {ends}")
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+
+
+def _grouped_call(lib, problems):
+    """problems: list of (a, packed, out, s, ws, M, N, K) device tensors / ints."""
+    import ctypes
+
+    arr = (_lib.Problem * max(1, len(problems)))()
+    for i, (a, pk, out, s, ws, m, n, k) in enumerate(problems):
+        arr[i] = _lib.Problem(a.data_ptr(), pk.data_ptr(), out.data_ptr(), s.data_ptr(), ws.data_ptr(), m, n, k)
+    return lib.bitlinear_int8xint2_grouped(arr, len(problems), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+
+@pytest.mark.parametrize("shape_id", [0, 1, 2, 3])
+@pytest.mark.parametrize("m", [1, 4])
+def test_grouped_launch_at_2b_shapes(shape_id, m):
+    """bitlinear_int8xint2_grouped over the weights of five layers of one 2B shape
+    (distinct weights, activations and scales per problem): one launch of the
+    streaming kernel, every problem's output equal to the oracle's bit for bit."""
+    lib = _lib.load_library()
+    sh = workload.shapes_2b()[shape_id]
+    ws_bits = workload.weight_scales(sh.K, sh.N, shape_id, sh.parts)
+    problems, wants = [], []
+    for layer in range(5):
+        w = workload.ternary_weight(sh.K, sh.N, shape_id, layer)
+        rng = np.random.default_rng(1000 * shape_id + 10 * layer + m)
+        xb = o.f32_to_bf16_bits(rng.standard_normal((m, sh.K)).astype(np.float32) * (1.0 + layer))
+        q, s_bits = o.quant_input(xb, o.QUANT_COMPILED)
+        _, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+        wants.append(want)
+        out = torch.full((m, sh.N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        problems.append((dev_i8(q), _packed_dev(w), out, dev_bf16(s_bits), dev_bf16(ws_bits), m, sh.N, sh.K))
+    assert _grouped_call(lib, problems) == 0
+    assert bitlinear.last_kernel() == "gemv_i2_stream_kernel"
+    torch.cuda.synchronize()
+    for i, (p, want) in enumerate(zip(problems, wants)):
+        _assert_bits_equal(host_bits(p[2]), want, f"{sh.name} problem {i}")
+
+
+def test_grouped_launch_mixed_shapes_long_runs_and_errors():
+    """Runs of equal shape become one launch each, more than 48 equal problems
+    several, M > 4 and lone problems go through the ordinary choice of kernel;
+    an empty list is fine; a bad element is refused before anything is launched."""
+    lib = _lib.load_library()
+    rng = np.random.default_rng(77)
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    wsd = dev_bf16(ws_bits)
+    spec = [(3840, 2560, 1), (3840, 2560, 1), (2560, 2560, 2), (2560, 6912, 8), (2560, 6912, 8), (2560, 2560, 2), (48, 192, 3)]
+    spec += [(64, 256, 1)] * 53
+    problems, wants = [], []
+    for (n, k, m) in spec:
+        w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+        a = rng.integers(-128, 128, size=(m, k), dtype=np.int8)
+        s_bits = o.f32_to_bf16_bits((2.0 + 50.0 * rng.random(m)).astype(np.float32))
+        _, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+        wants.append(want)
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        problems.append((dev_i8(a), _packed_dev(w), out, dev_bf16(s_bits), wsd, m, n, k))
+    assert _grouped_call(lib, problems) == 0
+    torch.cuda.synchronize()
+    for i, (p, want) in enumerate(zip(problems, wants)):
+        _assert_bits_equal(host_bits(p[2]), want, f"problem {i} {spec[i]}")
+    assert _grouped_call(lib, []) == 0
+    # a bad shape in the middle: status 1, and the outputs in front of it stay untouched
+    for p in problems[:3]:
+        p[2].fill_(float("nan"))
+    bad = list(problems[:3])
+    bad[2] = bad[2][:5] + (2, 100, 2560)
+    assert _grouped_call(lib, bad) == 1
+    torch.cuda.synchronize()
+    assert torch.isnan(problems[0][2].float()).all()
+    # in a captured graph, replayed
+    good = problems[:2]
+    for p in good:
+        p[2].zero_()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        assert _grouped_call(lib, good) == 0
+    for _ in range(3):
+        for p in good:
+            p[2].zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for p, want in zip(good, wants[:2]):
+            _assert_bits_equal(host_bits(p[2]), want, "grouped graph replay")
+
+
 def test_3d_input_and_out_argument():
     n, k = 2560, 2560
     w, a = _rand_case(n, k, 6, seed=3)
