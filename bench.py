@@ -289,18 +289,166 @@ def large_shapes(lib, dev, budget_bytes=1 << 30):
                 if lib.bitlinear_last_status() != 0:
                     raise RuntimeError(f"bitlinear_int8xint2 rejected N={N} K={K}")
 
-        run = GraphRun(launch)
+        kernel_name = []
+
+        def launch_and_name(sp):
+            launch(sp)
+            kernel_name[:] = [lib.bitlinear_last_kernel().decode()]
+
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+        def launch_probe(sp):  # the same bytes, requested and dropped
+            for i in range(nl):
+                arr = (ctypes.c_void_p * 1)(w.data_ptr() + (i % copies) * nbytes)
+                if lib.bitlinear_probe_weight_stream(arr, 1, N, K, _p(sink), sp) != 0:
+                    raise RuntimeError(f"bitlinear_probe_weight_stream rejected N={N} K={K}")
+
+        run = GraphRun(launch_and_name)
         run.replay(3)
         best = min(run.timed(5)[1] / 5 for _ in range(3)) * 1e3 / nl  # us per launch
+        del run
+        run = GraphRun(launch_probe)
+        run.replay(3)
+        floor = min(run.timed(5)[1] / 5 for _ in range(3)) * 1e3 / nl
         out[f"{N}x{K}"] = {
             "us_per_launch": round(best, 2),
             "weight_GBps": round(nbytes / best / 1e3, 1),
             "frac_of_hbm_peak": round(nbytes / best / 1e3 / HBM_PEAK_GBPS, 4),
             "weight_bytes": nbytes,
+            "kernel": kernel_name[0],
+            "load_only_us_per_launch": round(floor, 2),
+            "load_only_frac_of_hbm_peak": round(nbytes / floor / 1e3 / HBM_PEAK_GBPS, 4),
+            "frac_of_load_only": round(floor / best, 4),
         }
         del run, w
         torch.cuda.empty_cache()
     return {"large_shapes_product_only": out}
+
+
+def latency_floor(lib, shapes, layers, dev, n_timed=20):
+    """What a dependent launch costs on this machine before any BitLinear
+    arithmetic, measured in the same run and the same way as the headline (a HIP
+    graph of 120 launches on one stream, replayed; HIP events on that stream;
+    the weights of 30 layers, so nothing is cache-hot): a kernel with an empty
+    body (one wave, and with the product's grid), and a kernel that only
+    requests one call's packed weights and drops them (per 2B shape)."""
+    import torch
+
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    n_layers = len(layers)
+
+    def timed_us(fn, launches):
+        g = GraphRun(fn)
+        g.replay(3)
+        us = min(g.timed(n_timed)[1] / n_timed for _ in range(3)) * 1e3 / launches
+        del g
+        return us
+
+    def empty(blocks, threads):
+        def fn(sp):
+            for _ in range(4 * n_layers):
+                assert lib.bitlinear_probe_empty(blocks, threads, sp) == 0
+        return fn
+
+    out = {
+        "how": "HIP graph of 120 dependent launches on one stream (as the headline), HIP events, min of 3 x %d replays" % n_timed,
+        "empty_kernel_us": {"1x64": round(timed_us(empty(1, 64), 4 * n_layers), 3)},
+        "load_only_us": {},
+        "hbm_time_at_peak_us": {},
+    }
+    for sh in shapes:
+        out["empty_kernel_us"][f"{sh.N // 16}x512 ({sh.name} grid)"] = round(timed_us(empty(sh.N // 16, 512), 4 * n_layers), 3)
+    tot_floor = 0.0
+    for i, sh in enumerate(shapes):
+        def fn(sp, i=i, sh=sh):
+            for rep in range(4):
+                for row in layers:
+                    arr = (ctypes.c_void_p * 1)(row[i].data_ptr())
+                    assert lib.bitlinear_probe_weight_stream(arr, 1, sh.N, sh.K, _p(sink), sp) == 0
+        us = timed_us(fn, 4 * n_layers)
+        tot_floor += us
+        out["load_only_us"][sh.name] = round(us, 3)
+        out["hbm_time_at_peak_us"][sh.name] = round(sh.weight_bytes / HBM_PEAK_GBPS / 1e3, 3)
+    step_bytes = sum(sh.weight_bytes for sh in shapes) * n_layers
+    out["load_only_us"]["mean_of_the_four"] = round(tot_floor / len(shapes), 3)
+    out["load_only_chain_GBps"] = round(step_bytes / (tot_floor * n_layers) / 1e3, 1)
+    out["load_only_chain_frac_of_hbm_peak"] = round(step_bytes / (tot_floor * n_layers) / 1e3 / HBM_PEAK_GBPS, 4)
+    out["note"] = (
+        "load_only = bitlinear_probe_weight_stream: the streaming kernel's grid, 16-byte loads and software pipeline with "
+        "the activation operand, the decode, the MFMAs and the output removed; the chain figure is what 120 such launches "
+        "per step would stream: the ceiling of any per-call kernel in a dependent chain on this machine"
+    )
+    return {"latency_floor": out}
+
+
+def grouped_launches(lib, shapes, layers, scales, dev, M=1):
+    """bitlinear_int8xint2_grouped: the 30 layers' products of one 2B shape in ONE
+    launch (independent problems: their own int8 rows, scales and outputs), and
+    the same bytes through the load-only probe.  What the kernels stream when
+    the cost of starting a kernel is paid once per 49-265 MB instead of once per
+    1.6-8.8 MB."""
+    import torch
+
+    from bitnet_amd import _lib
+
+    out = {}
+    L = len(layers)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    for i, sh in enumerate(shapes):
+        a = torch.randint(-127, 128, (L, M, sh.K), dtype=torch.int8, device=dev)
+        s = torch.full((L, M), 3.0, dtype=torch.bfloat16, device=dev)
+        o = torch.empty(L, M, sh.N, dtype=torch.bfloat16, device=dev)
+        nbytes = sh.weight_bytes * L
+        # enough further sets of 30 weights (random bytes: timing only) that a replay streams at least 600 MB
+        # of distinct weights: nothing is left in the 256 MB last-level cache when a set comes round again
+        sets = max(1, -(-(600 << 20) // nbytes))
+        extra = torch.randint(0, 255, (sets - 1, L, sh.weight_bytes), dtype=torch.uint8, device=dev) if sets > 1 else None
+
+        def wptr(k, l):
+            return layers[l][i].data_ptr() if k == 0 else extra[k - 1, l].data_ptr()
+
+        arrs, ptrs = [], []
+        for k in range(sets):
+            arr = (_lib.Problem * L)()
+            pp = (ctypes.c_void_p * L)()
+            for l in range(L):
+                arr[l] = _lib.Problem(a[l].data_ptr(), wptr(k, l), o[l].data_ptr(), s[l].data_ptr(), scales[i].data_ptr(),
+                                      M, sh.N, sh.K)
+                pp[l] = wptr(k, l)
+            arrs.append(arr)
+            ptrs.append(pp)
+        name = []
+
+        def fn(sp):
+            for arr in arrs:
+                st = lib.bitlinear_int8xint2_grouped(arr, L, sp)
+                assert st == 0, lib.bitlinear_status_string(st)
+            name[:] = [lib.bitlinear_last_kernel().decode()]
+
+        def probe(sp):
+            for pp in ptrs:
+                assert lib.bitlinear_probe_weight_stream(pp, L, sh.N, sh.K, _p(sink), sp) == 0
+
+        res = []
+        for f in (fn, probe):
+            g = GraphRun(f)
+            g.replay(3)
+            res.append(min(g.timed(10)[1] / 10 for _ in range(3)) * 1e3 / sets)
+            del g
+        out[sh.name] = {
+            "problems_per_launch": L,
+            "bytes_per_launch": nbytes,
+            "us_per_launch": round(res[0], 2),
+            "weight_GBps": round(nbytes / res[0] / 1e3, 1),
+            "frac_of_hbm_peak": round(nbytes / res[0] / 1e3 / HBM_PEAK_GBPS, 4),
+            "kernel": name[0],
+            "load_only_us_per_launch": round(res[1], 2),
+            "load_only_frac_of_hbm_peak": round(nbytes / res[1] / 1e3 / HBM_PEAK_GBPS, 4),
+            "launches_per_replay": sets,
+        }
+        del extra
+        torch.cuda.empty_cache()
+    return {f"grouped_launch_M{M}": out}
 
 
 def end_to_end_decode(batches=(1, 8), prompt_len=512, gen_len=128):
@@ -571,7 +719,10 @@ def main():
             "launch latency overlapped, not a decode step; wall clock",
         },
     }
+    result.update(latency_floor(lib, shapes, layers, dev))
     if not args.no_sweeps:
+        result.update(grouped_launches(lib, shapes, layers, scales, dev, 1))
+        result.update(grouped_launches(lib, shapes, layers, scales, dev, 4))
         result.update(batched_and_prefill(lib, shapes, layers, scales, dev))
         result.update(large_shapes(lib, dev))
     if not args.no_e2e:

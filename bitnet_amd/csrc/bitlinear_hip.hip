@@ -1499,6 +1499,151 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// BitLinearKernel.forward for one to four tokens with waves that prepare their own operands
+// ---------------------------------------------------------------------------
+// Same decomposition as bitlinear_fused_kernel (a workgroup owns RB 16-row blocks, S waves split K
+// for each, one packed word per lane and k-step is the MFMA's row operand) but no wave waits for
+// another before its products are done: every wave takes the row maximum of the activation rows
+// itself (the whole rows, a few KB that every wave of the machine reads from cache: redundant work,
+// but no workgroup-wide reduction, no LDS atomics and no barrier in front of the products),
+// quantizes only the slice of k that its own k-steps multiply, and hands it to itself through a
+// private LDS region.  The +2 of the stored codes is removed per wave with the sum of its own slice.
+// One barrier, behind the products: the waves' partial tiles are added by the threads that finish
+// the outputs.  A wave's instruction stream is what a call of this size costs, and this one is
+// about half as long as the shared-prologue kernel's.
+constexpr int kSoloMaxTokens = 4;
+constexpr int kSoloMaxUPW = 8;  // at most 8 k-steps (512 k = 64 vectors of 8 values) per wave: one slice vector per lane
+
+template <int UPW, int VROW, int MT>
+__global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
+    // parameter order: what stands between the kernel's entry and its first loads comes first
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, uint16_t* __restrict__ out,
+    const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
+    int32_t* __restrict__ acc_out) {
+    __shared__ __attribute__((aligned(16))) int8_t lds_q[kMaxWaves][MT][kSoloMaxUPW * 64];  // a wave's quantized slice per token
+    __shared__ __attribute__((aligned(16))) int red[kMaxWaves][256];                        // a wave's partial 16 x 16 tile
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rbl = (wave >= S ? 1 : 0) + (wave >= 2 * S ? 1 : 0) + (wave >= 3 * S ? 1 : 0);  // wave / S, RB <= 4
+    const int ks = wave - rbl * S;
+    const int rb = blockIdx.x * RB + rbl;
+    const bool rows_ok = rb < (N >> 4);
+    const int g = lane >> 4;
+    const int p = lane & 15;
+
+    // requests, all at once: the slice's vectors (needed last, but they are part of the rows and
+    // return with them), the whole rows for the maximum, then the weight words
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00020000);
+    const int slice_k0 = ks * (UPW * 64);
+    const bool slice_lane = lane < UPW * 8 && slice_k0 + lane * 8 < K;
+    uint4 sv[MT];
+    uint4 rv[MT][VROW];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row_off = (m < M ? m : M - 1) * K * 2;
+        // a lane without a slice vector, or a vector past the end of the row, asks past the end of the buffer: zeros, no access
+        sv[m] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                              x_rsrc, slice_lane ? row_off + (slice_k0 + lane * 8) * 2 : 0x7ffffff0, 0, 0));
+#pragma unroll
+        for (int v = 0; v < VROW; ++v) {
+            const int k = (lane + v * 64) * 8;
+            rv[m][v] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, k < K ? row_off + k * 2 : 0x7ffffff0, 0, 0));
+        }
+    }
+    const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((const char*)wq + (size_t)(rows_ok ? rb : 0) * K * 4), 0, rows_ok ? K * 4 : 0, 0x00020000);
+    const int w_voff = lane_word * 4 + ks * (UPW * 256);
+    uint32_t w[UPW];
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) w[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + j * 256, 0, 2 /* nt */);
+    // epilogue operand, raw bits: the weight scale of the workgroup's first row (a workgroup that
+    // straddles a slot boundary fetches per row in the epilogue)
+    const int n_first = blockIdx.x * RB * 16;
+    const int n_last = (n_first + RB * 16 - 1) < N ? (n_first + RB * 16 - 1) : N - 1;
+    const int slot_first = scale_slot_uniform(smap, n_first), slot_last = scale_slot_uniform(smap, n_last);
+    const uint16_t wsb_first = ws[slot_first];
+
+    // row maxima -> scales; this wave's slice -> int8 in its LDS region, with the slice's sum
+    float sf[MT];
+    int qsum2[MT];  // twice the sum of the slice's int8 values
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        uint32_t am = 0;
+#pragma unroll
+        for (int v = 0; v < VROW; ++v) am = absmax_bits8(rv[m][v], am);
+        am = wave_max_u32(am);
+        sf[m] = quant_scale<0>(am);
+        const uint2 qv = quant_vec8<0>(sv[m], sf[m]);  // zeros for a lane without a slice vector
+        if (lane < UPW * 8) *(uint2*)(&lds_q[wave][m][lane * 8]) = qv;
+        const int ones = 0x01010101;
+        const int part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, 0, false), false);
+        qsum2[m] = 2 * wave_sum_i32(part);
+        if (blockIdx.x == 0 && rbl == 0 && m < M) {
+            if (q_out && slice_lane) *(uint2*)(q_out + (size_t)m * K + slice_k0 + lane * 8) = qv;
+            if (s_out && ks == 0 && lane == 0) s_out[m] = f32_to_bf16_rne(sf[m]);
+        }
+    }
+    // the same wave wrote and reads: LDS operations of a wave complete in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // products: B operand = 16 int8 of token p for the 16 k of chunk g (columns of tokens >= M repeat the last token and are never read)
+    const int8_t* brow = &lds_q[wave][p < MT ? (p < M ? p : M - 1) : 0][g * 16];
+    v4i b[UPW];
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) b[j] = *(const v4i*)(brow + j * 64);
+    v4i acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) {
+        const uint32_t wj = w[j];  // zero past the end of K
+        v4i e;
+        e.x = (int)(wj & 0x03030303u);
+        e.y = (int)((wj >> 2) & 0x03030303u);
+        e.z = (int)((wj >> 4) & 0x03030303u);
+        e.w = (int)((wj >> 6) & 0x03030303u);
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(e, b[j], acc, 0, 0, 0);
+    }
+    // lane holds token p, rows 4 g + i in register i; the +2 of the codes goes with the slice's sum
+    int q2 = qsum2[0];
+#pragma unroll
+    for (int m = 1; m < MT; ++m) q2 = p == m ? qsum2[m] : q2;
+    {
+        int* dst = &red[wave][lane];
+        dst[0] = acc.x - q2;
+        dst[64] = acc.y - q2;
+        dst[128] = acc.z - q2;
+        dst[192] = acc.w - q2;
+    }
+    lds_barrier();
+
+    // every thread finishes the output slots t = tid, tid + nthreads, ... of the workgroup: [row block][reg][lane]
+    const int nthreads = 64 * RB * S;
+#pragma unroll
+    for (int r = 0; r < kFusedMaxRB; ++r) {
+        const int t = tid + r * nthreads;
+        if (t >= RB * 256) break;
+        const int l = t & 63;
+        const int m = l & 15;
+        const int tb = t >> 8;  // row block of the slot
+        const int n = (blockIdx.x * RB + tb) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
+        if (m < M && n < N) {
+            int sum = 0;
+            for (int k = 0; k < S; ++k) sum += red[tb * S + k][t & 255];
+            if (acc_out) acc_out[(size_t)m * N + n] = sum;  // uniform: parity tests only
+            float sv_ = sf[0];
+#pragma unroll
+            for (int mm = 1; mm < MT; ++mm) sv_ = m == mm ? sf[mm] : sv_;
+            uint16_t wsb = wsb_first;
+            if (slot_first != slot_last) wsb = ws[scale_slot(smap, n)];  // uniform branch, rare
+            if (out) out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sv_ * bf16_to_f32(wsb));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 thread_local int g_status = BITLINEAR_OK;
@@ -1521,6 +1666,9 @@ struct Tuning {
     int stream = 0;        // product through the streaming kernel: 0 = built-in choice, 1 = whenever it applies, 2 = never
     int stream_depth = 0;  // its ring depth (0 = built-in choice)
     int stream_waves = 0;  // its waves per CU (0 = built-in choice)
+    int solo = 0;          // forward through the kernel whose waves prepare their own operands: 0 = built-in choice, 1..4 = always,
+                           // with that many row blocks per workgroup, 5 = never
+    int solo_s = 0, solo_upw = 0;  // its waves per row block and k-steps per wave when forced
 };
 std::mutex g_tuning_mutex;
 Tuning g_tuning_shared;
@@ -1690,6 +1838,14 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
         if (pl.upw == 0) pl.upw = 8;  // several rounds per wave: short rounds measured best (K = 27648: 9.3 us with 8, 10.7 with 16)
         pl.s = (units + pl.upw - 1) / pl.upw;
         if (pl.s > max_s) pl.s = max_s;
+        // three to six tokens through the plain quantizer: more waves than the k-steps need, because the
+        // quantizer's work grows with the tokens and is shared by the workgroup's threads (measured at
+        // K = 2560: 4 tokens 4.72 -> 4.15 us with 12 waves, 6 tokens 5.38 -> 5.06 with 16)
+        if (pro == 0 && M >= 3 && units <= 64 && pl.rb == 1) {
+            pl.s = M <= 4 ? 12 : 16;
+            pl.upw = 4;
+            while (pl.upw * pl.s < units) pl.upw = pl.upw == 4 ? 5 : (pl.upw == 5 ? 8 : (pl.upw == 8 ? 10 : 16));
+        }
     }
     const int nvec = M * (K / (pro == 3 ? 16 : 8));
     int need = (nvec + 64 * pl.rb * pl.s - 1) / (64 * pl.rb * pl.s);
@@ -1777,6 +1933,93 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 #undef BITLINEAR_LAUNCH_UV
 #undef BITLINEAR_LAUNCH_UVP
 #undef BITLINEAR_LAUNCH_UVPR
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+// Launch shape of bitlinear_solo_kernel: every wave multiplies exactly UPW (<= 8) k-steps, so S * UPW
+// must cover K / 64; instances exist for one token (rows up to 8192 values), two (up to 4096) and
+// three or four (up to 2560).
+struct SoloPlan {
+    int rb, s, upw, vrow, mt;
+    bool ok;
+};
+
+// Where the library takes it by itself.  Measured per call (HIP graph of dependent launches, distinct
+// weights), one token: 3840 x 2560 3.38 -> 3.16 us, 2560 x 2560 3.32 -> 3.11, 13824 x 2560 5.06 -> 4.80;
+// 2560 x 6912 4.57 -> 5.25 (14 row vectors per lane for the maximum: the redundant part outgrows what the
+// barriers cost); two tokens 3.85 -> 4.01 / 3.75 -> 3.70 / 5.14 -> 6.11, four tokens 4.15 -> 5.18.
+bool solo_wanted(int M, int N, int K) {
+    (void)N;
+    return M == 1 && K <= 4096;
+}
+
+SoloPlan plan_solo(int M, int N, int K) {
+    SoloPlan pl = {1, 8, 5, 5, 1, false};
+    if (M < 1 || M > kSoloMaxTokens) return pl;
+    if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31 || (long long)M * K * 2 >= 0x7ffffff0ll) return pl;
+    const int units = K / 64;
+    const int need_v = (K + 511) / 512;
+    pl.mt = M == 1 ? 1 : (M == 2 ? 2 : 4);
+    const int vmax = pl.mt == 1 ? 16 : (pl.mt == 2 ? 8 : 5);
+    if (need_v > vmax) return pl;
+    pl.vrow = need_v <= 5 ? 5 : (need_v <= 8 ? 8 : (need_v <= 14 ? 14 : 16));
+    if (t_tune.solo >= 1 && t_tune.solo <= 4) {
+        pl.rb = t_tune.solo;
+        pl.s = t_tune.solo_s;
+        pl.upw = t_tune.solo_upw;
+    } else {
+        // one row block per workgroup; with few row blocks (about one workgroup per CU) short waves of five
+        // k-steps, with many the fewest waves per row block (13824 x 2560: 4.80 us with 5 waves of 8 k-steps,
+        // 5.28 with 8 of 5)
+        const int blocks16 = N / 16;
+        pl.rb = 1;
+        const int order_few[4] = {5, 7, 8, 4}, order_many[4] = {8, 7, 5, 4};
+        const int* order = blocks16 >= 432 ? order_many : order_few;
+        pl.upw = 0;
+        for (int i = 0; i < 4; ++i)
+            if ((units + order[i] - 1) / order[i] <= (blocks16 >= 432 ? kMaxWaves : 10)) {
+                pl.upw = order[i];
+                break;
+            }
+        if (pl.upw == 0) pl.upw = 8;
+        pl.s = (units + pl.upw - 1) / pl.upw;
+    }
+    pl.ok = pl.rb >= 1 && pl.rb <= kFusedMaxRB && pl.s >= 1 && pl.rb * pl.s <= kMaxWaves && pl.s * pl.upw >= units &&
+            (pl.upw == 4 || pl.upw == 5 || pl.upw == 7 || pl.upw == 8);
+    return pl;
+}
+
+int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* ws,
+                const ScaleMap& smap, int8_t* q_out, uint16_t* s_out, int M, int N, int K, const SoloPlan& pl,
+                hipStream_t stream) {
+    const int blocks16 = N / 16;
+    const dim3 grid((blocks16 + pl.rb - 1) / pl.rb, 1, 1);
+    const dim3 block(64 * pl.rb * pl.s, 1, 1);
+    const uint32_t* wq = (const uint32_t*)packed;
+    g_last_kernel = "bitlinear_solo_kernel";
+#define BITLINEAR_LAUNCH_SOLO(U, V, T)                                                                               \
+    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, out, ws, smap, \
+                       q_out, s_out, acc_out)
+#define BITLINEAR_LAUNCH_SOLO_U(U)                                  \
+    if (pl.mt == 1) {                                               \
+        if (pl.vrow == 5) BITLINEAR_LAUNCH_SOLO(U, 5, 1);           \
+        else if (pl.vrow == 8) BITLINEAR_LAUNCH_SOLO(U, 8, 1);      \
+        else if (pl.vrow == 14) BITLINEAR_LAUNCH_SOLO(U, 14, 1);    \
+        else BITLINEAR_LAUNCH_SOLO(U, 16, 1);                       \
+    } else if (pl.mt == 2) {                                        \
+        if (pl.vrow == 5) BITLINEAR_LAUNCH_SOLO(U, 5, 2);           \
+        else BITLINEAR_LAUNCH_SOLO(U, 8, 2);                        \
+    } else {                                                        \
+        BITLINEAR_LAUNCH_SOLO(U, 5, 4);                             \
+    }
+    switch (pl.upw) {
+        case 4: BITLINEAR_LAUNCH_SOLO_U(4); break;
+        case 5: BITLINEAR_LAUNCH_SOLO_U(5); break;
+        case 7: BITLINEAR_LAUNCH_SOLO_U(7); break;
+        default: BITLINEAR_LAUNCH_SOLO_U(8); break;
+    }
+#undef BITLINEAR_LAUNCH_SOLO_U
+#undef BITLINEAR_LAUNCH_SOLO
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
@@ -2065,7 +2308,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = 0;
+        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -2079,6 +2322,18 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         g.stream = a;
         g.stream_depth = b;
         g.stream_waves = c;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 8) {
+        if (a == 0 || a == 5) {
+            g.solo = a;
+            return set_status(BITLINEAR_OK);
+        }
+        const bool upw_ok = c == 4 || c == 5 || c == 7 || c == 8;
+        if (a < 1 || a > kFusedMaxRB || b < 1 || a * b > kMaxWaves || !upw_ok) return set_status(BITLINEAR_ERR_ARG);
+        g.solo = a;
+        g.solo_s = b;
+        g.solo_upw = c;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 1) {
@@ -2237,6 +2492,12 @@ static int forward_impl(const uint16_t* x, const int8_t* packed, uint16_t* outpu
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
     if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)q_ws)) & 15u) return set_status(BITLINEAR_ERR_ARG);
     const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    // up to four tokens: the kernel whose waves quantize their own slices
+    if (mode == 0 && t_tune.path == 0 && t_tune.solo != 5 && M <= kSoloMaxTokens) {
+        const SoloPlan sp = plan_solo(M, N, K);
+        if (sp.ok && (t_tune.solo >= 1 || solo_wanted(M, N, K)))
+            return set_status(launch_solo(x, packed, output0, acc_out, ws, sm, q_ws, s_ws, M, N, K, sp, (hipStream_t)stream));
+    }
     const FusedPlan pl = plan_fused(M, N, K);
     // one kernel while the activation block is small enough for every workgroup to quantize it
     // again (or when the caller gave no workspaces for the two-kernel path)
