@@ -1514,7 +1514,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
 constexpr int kSoloMaxTokens = 4;
 constexpr int kSoloMaxUPW = 8;  // at most 8 k-steps (512 k = 64 vectors of 8 values) per wave: one slice vector per lane
 
-template <int UPW, int VROW, int MT>
+// COOP: the row maximum is taken over the workgroup's slices and exchanged through LDS (one barrier more,
+// no redundant reads of the rows): for rows too long for every wave to scan them
+template <int UPW, int VROW, int MT, bool COOP>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     // parameter order: what stands between the kernel's entry and its first loads comes first
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, uint16_t* __restrict__ out,
@@ -1522,6 +1524,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     int32_t* __restrict__ acc_out) {
     __shared__ __attribute__((aligned(16))) int8_t lds_q[kMaxWaves][MT][kSoloMaxUPW * 64];  // a wave's quantized slice per token
     __shared__ __attribute__((aligned(16))) int red[kMaxWaves][256];                        // a wave's partial 16 x 16 tile
+    __shared__ uint32_t wmax[kMaxWaves][MT];                                                // COOP: a wave's slice maximum per token
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1545,10 +1548,12 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
         // a lane without a slice vector, or a vector past the end of the row, asks past the end of the buffer: zeros, no access
         sv[m] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
                                               x_rsrc, slice_lane ? row_off + (slice_k0 + lane * 8) * 2 : 0x7ffffff0, 0, 0));
+        if (!COOP) {
 #pragma unroll
-        for (int v = 0; v < VROW; ++v) {
-            const int k = (lane + v * 64) * 8;
-            rv[m][v] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, k < K ? row_off + k * 2 : 0x7ffffff0, 0, 0));
+            for (int v = 0; v < VROW; ++v) {
+                const int k = (lane + v * 64) * 8;
+                rv[m][v] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, k < K ? row_off + k * 2 : 0x7ffffff0, 0, 0));
+            }
         }
     }
     const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
@@ -1568,12 +1573,25 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     // row maxima -> scales; this wave's slice -> int8 in its LDS region, with the slice's sum
     float sf[MT];
     int qsum2[MT];  // twice the sum of the slice's int8 values
+    if (COOP) {
+        // the S waves of a row block cover all of K between them: their slice maxima make the row maximum
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const uint32_t am = wave_max_u32(absmax_bits8(sv[m], 0u));
+            if (lane == 0) wmax[wave][m] = am;
+        }
+        lds_barrier();
+    }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         uint32_t am = 0;
+        if (COOP) {
+            for (int k = 0; k < S; ++k) am = max(am, wmax[rbl * S + k][m]);
+        } else {
 #pragma unroll
-        for (int v = 0; v < VROW; ++v) am = absmax_bits8(rv[m][v], am);
-        am = wave_max_u32(am);
+            for (int v = 0; v < VROW; ++v) am = absmax_bits8(rv[m][v], am);
+            am = wave_max_u32(am);
+        }
         sf[m] = quant_scale<0>(am);
         const uint2 qv = quant_vec8<0>(sv[m], sf[m]);  // zeros for a lane without a slice vector
         if (lane < UPW * 8) *(uint2*)(&lds_q[wave][m][lane * 8]) = qv;
@@ -1669,6 +1687,7 @@ struct Tuning {
     int solo = 0;          // forward through the kernel whose waves prepare their own operands: 0 = built-in choice, 1..4 = always,
                            // with that many row blocks per workgroup, 5 = never
     int solo_s = 0, solo_upw = 0;  // its waves per row block and k-steps per wave when forced
+    int solo_coop = 0;             // row maximum: 0 = built-in choice, 1 = exchanged between the waves, 2 = every wave scans the rows
 };
 std::mutex g_tuning_mutex;
 Tuning g_tuning_shared;
@@ -1941,28 +1960,34 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 // three or four (up to 2560).
 struct SoloPlan {
     int rb, s, upw, vrow, mt;
+    bool coop;
     bool ok;
 };
 
 // Where the library takes it by itself.  Measured per call (HIP graph of dependent launches, distinct
-// weights), one token: 3840 x 2560 3.38 -> 3.16 us, 2560 x 2560 3.32 -> 3.11, 13824 x 2560 5.06 -> 4.80;
-// 2560 x 6912 4.57 -> 5.25 (14 row vectors per lane for the maximum: the redundant part outgrows what the
-// barriers cost); two tokens 3.85 -> 4.01 / 3.75 -> 3.70 / 5.14 -> 6.11, four tokens 4.15 -> 5.18.
+// weights; shared-prologue kernel -> this one): one token 3840 x 2560 3.40 -> 3.18 us, 2560 x 2560
+// 3.33 -> 3.13, 13824 x 2560 5.03 -> 4.81, 2560 x 6912 4.56 -> 4.31 (row maximum exchanged between the
+// waves; 5.24 with every wave scanning the 13.8 KB row); two tokens 3.86 -> 3.69 / 3.75 -> 3.62 / 5.14 -> 6.07
+// (not taken) / 5.61 -> 5.21; four tokens 4.16 -> 4.59 (not taken) and 6.81 -> 6.61 at K = 6912.
 bool solo_wanted(int M, int N, int K) {
-    (void)N;
-    return M == 1 && K <= 4096;
+    if (M == 1) return K <= 8192;
+    if (K > 4096) return true;  // long rows, two to four tokens
+    return M == 2 && (N / 16) < 432;
 }
 
 SoloPlan plan_solo(int M, int N, int K) {
-    SoloPlan pl = {1, 8, 5, 5, 1, false};
+    SoloPlan pl = {1, 8, 5, 5, 1, false, false};
     if (M < 1 || M > kSoloMaxTokens) return pl;
     if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31 || (long long)M * K * 2 >= 0x7ffffff0ll) return pl;
     const int units = K / 64;
     const int need_v = (K + 511) / 512;
     pl.mt = M == 1 ? 1 : (M == 2 ? 2 : 4);
     const int vmax = pl.mt == 1 ? 16 : (pl.mt == 2 ? 8 : 5);
-    if (need_v > vmax) return pl;
-    pl.vrow = need_v <= 5 ? 5 : (need_v <= 8 ? 8 : (need_v <= 14 ? 14 : 16));
+    // every wave scans the whole rows while they are short and there is one token; otherwise the
+    // row maximum is exchanged between the waves of the workgroup
+    pl.coop = t_tune.solo_coop == 1 || (t_tune.solo_coop == 0 && (need_v > 8 || M > 1));
+    if (need_v > vmax) pl.coop = true;
+    pl.vrow = pl.coop ? 1 : (need_v <= 5 ? 5 : (need_v <= 8 ? 8 : (need_v <= 14 ? 14 : 16)));
     if (t_tune.solo >= 1 && t_tune.solo <= 4) {
         pl.rb = t_tune.solo;
         pl.s = t_tune.solo_s;
@@ -1977,7 +2002,7 @@ SoloPlan plan_solo(int M, int N, int K) {
         const int* order = blocks16 >= 432 ? order_many : order_few;
         pl.upw = 0;
         for (int i = 0; i < 4; ++i)
-            if ((units + order[i] - 1) / order[i] <= (blocks16 >= 432 ? kMaxWaves : 10)) {
+            if ((units + order[i] - 1) / order[i] <= ((blocks16 >= 432 || units > 64) ? kMaxWaves : 10)) {
                 pl.upw = order[i];
                 break;
             }
@@ -1997,20 +2022,24 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
     g_last_kernel = "bitlinear_solo_kernel";
-#define BITLINEAR_LAUNCH_SOLO(U, V, T)                                                                               \
-    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, out, ws, smap, \
-                       q_out, s_out, acc_out)
-#define BITLINEAR_LAUNCH_SOLO_U(U)                                  \
-    if (pl.mt == 1) {                                               \
-        if (pl.vrow == 5) BITLINEAR_LAUNCH_SOLO(U, 5, 1);           \
-        else if (pl.vrow == 8) BITLINEAR_LAUNCH_SOLO(U, 8, 1);      \
-        else if (pl.vrow == 14) BITLINEAR_LAUNCH_SOLO(U, 14, 1);    \
-        else BITLINEAR_LAUNCH_SOLO(U, 16, 1);                       \
-    } else if (pl.mt == 2) {                                        \
-        if (pl.vrow == 5) BITLINEAR_LAUNCH_SOLO(U, 5, 2);           \
-        else BITLINEAR_LAUNCH_SOLO(U, 8, 2);                        \
-    } else {                                                        \
-        BITLINEAR_LAUNCH_SOLO(U, 5, 4);                             \
+#define BITLINEAR_LAUNCH_SOLO(U, V, T, C)                                                                            \
+    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, out, ws, \
+                       smap, q_out, s_out, acc_out)
+#define BITLINEAR_LAUNCH_SOLO_U(U)                                      \
+    if (pl.coop) {                                                      \
+        if (pl.mt == 1) BITLINEAR_LAUNCH_SOLO(U, 1, 1, true);           \
+        else if (pl.mt == 2) BITLINEAR_LAUNCH_SOLO(U, 1, 2, true);      \
+        else BITLINEAR_LAUNCH_SOLO(U, 1, 4, true);                      \
+    } else if (pl.mt == 1) {                                            \
+        if (pl.vrow == 5) BITLINEAR_LAUNCH_SOLO(U, 5, 1, false);        \
+        else if (pl.vrow == 8) BITLINEAR_LAUNCH_SOLO(U, 8, 1, false);   \
+        else if (pl.vrow == 14) BITLINEAR_LAUNCH_SOLO(U, 14, 1, false); \
+        else BITLINEAR_LAUNCH_SOLO(U, 16, 1, false);                    \
+    } else if (pl.mt == 2) {                                            \
+        if (pl.vrow == 5) BITLINEAR_LAUNCH_SOLO(U, 5, 2, false);        \
+        else BITLINEAR_LAUNCH_SOLO(U, 8, 2, false);                     \
+    } else {                                                            \
+        BITLINEAR_LAUNCH_SOLO(U, 5, 4, false);                          \
     }
     switch (pl.upw) {
         case 4: BITLINEAR_LAUNCH_SOLO_U(4); break;
@@ -2308,7 +2337,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = 0;
+        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -2322,6 +2351,11 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         g.stream = a;
         g.stream_depth = b;
         g.stream_waves = c;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 9) {
+        if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
+        g.solo_coop = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 8) {

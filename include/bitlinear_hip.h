@@ -139,9 +139,9 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s,
 /*
  * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer (mode
  * as above), product and epilogue.  While the activation block is small
- * (M * K <= 16384 elements) this is ONE kernel: every workgroup (for one token
- * and K <= 4096 every wave) quantizes x itself, keeps the int8 rows in LDS and
- * never reads s from memory.  Larger
+ * (M * K <= 16384 elements) this is ONE kernel: every workgroup (or every wave
+ * its own slice of k) quantizes x itself, keeps the int8 rows in LDS and never
+ * reads s from memory.  Larger
  * blocks run the quantizer once, in a kernel of its own, and then the product
  * kernel (M <= 16: int8 rows staged in LDS per workgroup; M > 16: MFMA GEMM).
  *   q_ws (int8 [M, K], 16-byte aligned) and s_ws (bf16 [M]) receive the
@@ -243,11 +243,16 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *   kernel 8: bitlinear_forward_bf16 (mode 0, M <= 4) through the kernel whose
  *             waves take the row maximum and quantize their own slice of k
  *             themselves (no workgroup-wide step in front of the products):
- *             a = 0 built-in choice (one token, K <= 4096), a = 1..4 always, with a
+ *             a = 0 built-in choice (one token; two to four where measured faster), a = 1..4 always, with a
  *             16-row blocks per workgroup, b waves per row block and c (4, 5, 7 or
  *             8) k-steps per wave (a * b <= 16; b * c * 64 must cover K, else the
  *             built-in kernel runs), a = 5 never.  Applies with kernel 0 only;
  *             kernel 0 resets it.
+ *   kernel 9: how that kernel takes the row maximum: a = 0 built-in choice, 1 =
+ *             slice maxima exchanged between the waves of a workgroup (one
+ *             barrier), 2 = every wave scans the whole rows (no barrier; one
+ *             token up to K = 8192, two up to 4096, more up to 2560).
+ *             Kernel 0 resets it.
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 
