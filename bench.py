@@ -15,7 +15,7 @@ Inputs are resident in HBM before timing starts.
 
 Prints ONE JSON line.  `value` is packed-weight bytes (K*N/4 per product) per
 second over the whole step.  `roofline` is for the kernel those launches run
-(bitlinear_fused_kernel): the same timed region, measured with HIP events on
+(bitlinear_solo_kernel): the same timed region, measured with HIP events on
 the stream the graph is replayed on, divided by the 120 launches of a step.
 `cpu_baseline` is the C restatement of the reference's CPU I2_S kernel timed
 on this host on a bounded sample of the same workload.
@@ -593,7 +593,20 @@ def main():
         torch.cuda.synchronize()
         launch_path(None)
         torch.cuda.synchronize()
-        print(json.dumps({"pmc_probe": "3 copies of 268435456 B (read 256 MiB + write 256 MiB each), then the 120 launches of one step"}))
+        # and one grouped launch per 2B shape (the 30 layers' products of that shape in one launch of the streaming kernel)
+        from bitnet_amd import _lib as _l
+
+        L = len(layers)
+        for i, sh in enumerate(shapes):
+            o = torch.empty(L, M, sh.N, dtype=torch.bfloat16, device=dev)
+            arr = (_l.Problem * L)()
+            for l in range(L):
+                arr[l] = _l.Problem(q_buf[i].data_ptr(), layers[l][i].data_ptr(), o[l].data_ptr(), s_buf[i].data_ptr(),
+                                    scales[i].data_ptr(), M, sh.N, sh.K)
+            assert lib.bitlinear_int8xint2_grouped(arr, L, None) == 0
+            torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": "3 copies of 268435456 B (read 256 MiB + write 256 MiB each), then the 120 launches of one "
+                          "step, then one grouped launch per 2B shape (30 problems each)"}))
         return
 
     step_bytes = sum(sh.weight_bytes for sh in shapes) * len(layers)
@@ -662,13 +675,17 @@ def main():
     _, q_ms = quant.timed(args.steps)
     quant_us = q_ms * 1e3 / (args.steps * n_gemv)
 
-    traffic = None
-    # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs, kept with their commands in profiles/
-    tpath = os.path.join(ROOT, "profiles", "bitlinear_fused_m1_bitnet2b_hbm_traffic.txt")
+    traffic, traffic_source = None, None
+    # HBM bytes per launch are NOT measured in this run (counters need the profiler): the figure is the one the
+    # FETCH_SIZE / WRITE_SIZE counter runs gave for the same 120 launches, kept with its commands, date and commit
+    # in profiles/; this run only repeats it
+    tpath = os.path.join(ROOT, "profiles", "bitlinear_forward_m1_bitnet2b_hbm_traffic.txt")
     if M == 1 and os.path.exists(tpath):
         for line in open(tpath):
             if line.startswith("traffic_bytes_per_launch:"):
                 traffic = int(float(line.split(":", 1)[1]))
+            if line.startswith("measured:"):
+                traffic_source = "profiles/bitlinear_forward_m1_bitnet2b_hbm_traffic.txt (rocprofv3 --pmc, " + line.split(":", 1)[1].strip() + "); not re-measured in this run"
 
     result = {
         "metric": METRIC,
@@ -703,8 +720,9 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "kernel": "bitlinear_fused_kernel (quantizer + int8 x int2 product + epilogue), mean over the 120 "
-            "launches of a step, HIP events on the replay stream over the timed region",
+            "traffic_source": traffic_source,
+            "kernel": "bitlinear_solo_kernel (BitLinearKernel.forward in one kernel: quantizer + int8 x int2 product + "
+            "epilogue), mean over the 120 launches of a step, HIP events on the replay stream over the timed region",
             "bytes_per_launch": step_bytes // n_gemv,
             "us_per_launch": round(fused_us, 3),
         },
