@@ -32,6 +32,9 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.POINTER(_c_int), _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
     "bitlinear_quant_absmax": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
+    "bitlinear_quant_absmax_rowsum": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
+    "bitlinear_repacked_size": (ctypes.c_size_t, [_c_int, _c_int]),
+    "bitlinear_repack": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]),
     "bitlinear_forward_bf16": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],

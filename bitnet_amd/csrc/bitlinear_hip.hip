@@ -1014,8 +1014,10 @@ __device__ __forceinline__ float quant_scale(uint32_t amax_bits) {
 template <int MODE>
 __global__ __launch_bounds__(kQuantMaxThreads) void quant_absmax_kernel(const uint16_t* __restrict__ x,
                                                                      int8_t* __restrict__ q,
-                                                                     uint16_t* __restrict__ s, int K) {
+                                                                     uint16_t* __restrict__ s, int K,
+                                                                     int32_t* __restrict__ rowsum) {
     __shared__ uint32_t wmax[kQuantMaxThreads / 64];
+    __shared__ int wsum[kQuantMaxThreads / 64];
     const int nthreads = blockDim.x;  // 256, or up to 1024 for long rows so that a row still fits the registers
     const int row = blockIdx.x;
     const int tid = threadIdx.x;
@@ -1048,13 +1050,32 @@ __global__ __launch_bounds__(kQuantMaxThreads) void quant_absmax_kernel(const ui
     const float s32 = quant_scale<MODE>(am);
     if (tid == 0) s[row] = f32_to_bf16_rne(s32);
 
+    int part = 0;  // sum of this thread's int8 values (only kept when the caller asks for the row sums)
+    const int ones = 0x01010101;
 #pragma unroll
     for (int r = 0; r < kQuantRegVecs; ++r) {
         const int idx = tid + r * nthreads;
-        if (idx < nvec) qr[idx] = quant_vec8<MODE>(v[r], s32);
+        if (idx < nvec) {
+            const uint2 qv = quant_vec8<MODE>(v[r], s32);
+            qr[idx] = qv;
+            part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, part, false), false);
+        }
     }
-    for (int idx = tid + kQuantRegVecs * nthreads; idx < nvec; idx += nthreads)
-        qr[idx] = quant_vec8<MODE>(xr[idx], s32);
+    for (int idx = tid + kQuantRegVecs * nthreads; idx < nvec; idx += nthreads) {
+        const uint2 qv = quant_vec8<MODE>(xr[idx], s32);
+        qr[idx] = qv;
+        part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, part, false), false);
+    }
+    if (rowsum) {  // uniform
+        const int ws_ = wave_sum_i32(part);
+        if ((tid & 63) == 0) wsum[tid >> 6] = ws_;
+        __syncthreads();
+        if (tid == 0) {
+            int tot = 0;
+            for (int i = 0; i < (nthreads >> 6); ++i) tot += wsum[i];
+            rowsum[row] = tot;
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1519,8 +1540,10 @@ constexpr int kSoloMaxUPW = 8;  // at most 8 k-steps (512 k = 64 vectors of 8 va
 template <int UPW, int VROW, int MT, bool COOP>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     // parameter order: what stands between the kernel's entry and its first loads comes first
-    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, uint16_t* __restrict__ out,
-    const uint16_t* __restrict__ ws, ScaleMap smap, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
+    // (the weight scales' slots are runs of slot_rows output rows each, the reference's rule n / (N / ws_num):
+    // one integer among the leading arguments instead of a table behind them)
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, int slot_rows,
+    const uint16_t* __restrict__ ws, uint16_t* __restrict__ out, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
     int32_t* __restrict__ acc_out) {
     __shared__ __attribute__((aligned(16))) int8_t lds_q[kMaxWaves][MT][kSoloMaxUPW * 64];  // a wave's quantized slice per token
     __shared__ __attribute__((aligned(16))) int red[kMaxWaves][256];                        // a wave's partial 16 x 16 tile
@@ -1564,11 +1587,18 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
 #pragma unroll
     for (int j = 0; j < UPW; ++j) w[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + j * 256, 0, 2 /* nt */);
     // epilogue operand, raw bits: the weight scale of the workgroup's first row (a workgroup that
-    // straddles a slot boundary fetches per row in the epilogue)
+    // straddles a slot boundary fetches per row in the epilogue); the slot by a few scalar
+    // comparisons (at most six slots), so that this request leaves with the others
     const int n_first = blockIdx.x * RB * 16;
     const int n_last = (n_first + RB * 16 - 1) < N ? (n_first + RB * 16 - 1) : N - 1;
-    const int slot_first = scale_slot_uniform(smap, n_first), slot_last = scale_slot_uniform(smap, n_last);
+    int slot_first = 0, slot_last = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSeg; ++j) {
+        slot_first += n_first >= j * slot_rows ? 1 : 0;
+        slot_last += n_last >= j * slot_rows ? 1 : 0;
+    }
     const uint16_t wsb_first = ws[slot_first];
+    __builtin_amdgcn_sched_barrier(0);  // every request above is on its way before anything below is looked at
 
     // row maxima -> scales; this wave's slice -> int8 in its LDS region, with the slice's sum
     float sf[MT];
@@ -1655,7 +1685,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
 #pragma unroll
             for (int mm = 1; mm < MT; ++mm) sv_ = m == mm ? sf[mm] : sv_;
             uint16_t wsb = wsb_first;
-            if (slot_first != slot_last) wsb = ws[scale_slot(smap, n)];  // uniform branch, rare
+            if (slot_first != slot_last) wsb = ws[n / slot_rows];  // uniform branch, rare
             if (out) out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sv_ * bf16_to_f32(wsb));
         }
     }
@@ -2021,10 +2051,14 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
     const dim3 grid((blocks16 + pl.rb - 1) / pl.rb, 1, 1);
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
+    // equal slots only (what the forward entry points use): rows per slot
+    const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
+    for (int j = 0; j + 1 < smap.nseg; ++j)
+        if (smap.ends[j] != (j + 1) * slot_rows) return BITLINEAR_ERR_ARG;
     g_last_kernel = "bitlinear_solo_kernel";
 #define BITLINEAR_LAUNCH_SOLO(U, V, T, C)                                                                            \
-    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, out, ws, \
-                       smap, q_out, s_out, acc_out)
+    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, slot_rows, \
+                       ws, out, q_out, s_out, acc_out)
 #define BITLINEAR_LAUNCH_SOLO_U(U)                                      \
     if (pl.coop) {                                                      \
         if (pl.mt == 1) BITLINEAR_LAUNCH_SOLO(U, 1, 1, true);           \
@@ -2502,7 +2536,35 @@ int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1, uint16_t
     return set_status(launch_gemv(input0, input1, output0, nullptr, s, ws, sm, M, N, K, (hipStream_t)stream));
 }
 
+static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t* rowsum, int M, int K, int mode, void* stream);
+
 int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s, int M, int K, int mode, void* stream) {
+    return quant_absmax_impl(x, q, s, nullptr, M, K, mode, stream);
+}
+
+int bitlinear_quant_absmax_rowsum(const uint16_t* x, int8_t* q, uint16_t* s, int32_t* rowsum, int M, int K, int mode,
+                                  void* stream) {
+    if (!rowsum) return set_status(BITLINEAR_ERR_NULL);
+    return quant_absmax_impl(x, q, s, rowsum, M, K, mode, stream);
+}
+
+size_t bitlinear_repacked_size(int N, int K) {
+    if (N < 16 || K < 64 || (N % 16) != 0 || (K % 64) != 0) return 0;
+    return (size_t)N * (size_t)K / 4;
+}
+
+int bitlinear_repack(const int8_t* packed_ref, void* packed_out, int N, int K, void* stream) {
+    const size_t bytes = bitlinear_repacked_size(N, K);
+    if (bytes == 0) return set_status(BITLINEAR_ERR_SHAPE);
+    if (!packed_ref || !packed_out) return set_status(BITLINEAR_ERR_NULL);
+    if (packed_ref == packed_out) return set_status(BITLINEAR_OK);  // in place: nothing to do
+    // the kernels consume the reference's layout as it is: the converter is a copy
+    return set_status(hipMemcpyAsync(packed_out, packed_ref, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream) == hipSuccess
+                          ? BITLINEAR_OK
+                          : BITLINEAR_ERR_LAUNCH);
+}
+
+static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t* rowsum, int M, int K, int mode, void* stream) {
     if (M < 1 || K < 8 || (K % 8) != 0) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !q || !s) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
@@ -2512,9 +2574,9 @@ int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s, int M, int
     while (threads < kQuantMaxThreads && K > threads * kQuantRegVecs * 8) threads *= 2;
     const dim3 grid(M, 1, 1), block(threads, 1, 1);
     if (mode == 0)
-        hipLaunchKernelGGL(quant_absmax_kernel<0>, grid, block, 0, (hipStream_t)stream, x, q, s, K);
+        hipLaunchKernelGGL(quant_absmax_kernel<0>, grid, block, 0, (hipStream_t)stream, x, q, s, K, rowsum);
     else
-        hipLaunchKernelGGL(quant_absmax_kernel<1>, grid, block, 0, (hipStream_t)stream, x, q, s, K);
+        hipLaunchKernelGGL(quant_absmax_kernel<1>, grid, block, 0, (hipStream_t)stream, x, q, s, K, rowsum);
     return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
 }
 

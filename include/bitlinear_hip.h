@@ -17,6 +17,7 @@
 #ifndef BITLINEAR_HIP_H
 #define BITLINEAR_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -135,6 +136,31 @@ int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1,
  */
 int bitlinear_quant_absmax(const uint16_t* x, int8_t* q, uint16_t* s,
                            int M, int K, int mode, void* stream);
+
+/*
+ * The same quantizer, also storing rowsum[m] = sum_k q[m, k] (int32 [M]).  The
+ * stored weight codes are w + 2 (gpu/pack_weight.py:80), so a product over the
+ * codes is sum(w * q) + 2 * rowsum: a caller that multiplies codes itself needs
+ * this sum; the library's own product kernels take it on the way.
+ */
+int bitlinear_quant_absmax_rowsum(const uint16_t* x, int8_t* q, uint16_t* s,
+                                  int32_t* rowsum, int M, int K, int mode,
+                                  void* stream);
+
+/*
+ * The load-time weight converter.  The kernels consume the layout the
+ * reference packer writes (gpu/pack_weight.py:76-98) in place -- one packed
+ * word is already the MFMA row operand of 16 consecutive k of one row -- so
+ * the converted form IS the reference form: bitlinear_repacked_size returns
+ * N * K / 4 bytes (0 for a shape the library does not take) and
+ * bitlinear_repack copies (device to device, on the stream; a no-op when
+ * source and destination are the same buffer).  They exist so that a loader
+ * written against "convert at load time" keeps working if a later version of
+ * the library prefers another layout.
+ */
+size_t bitlinear_repacked_size(int N, int K);
+int bitlinear_repack(const int8_t* packed_ref, void* packed_out, int N, int K,
+                     void* stream);
 
 /*
  * BitLinearKernel.forward (gpu/model.py:73-75) in one call: quantizer (mode

@@ -51,6 +51,11 @@ def test_host_only_entry_points():
     for (n, k), v in table.items():
         assert lib.bitlinear_ws_num(n, k) == v
     assert lib.bitlinear_ws_num(1024, 4096) == 1
+    # the load-time converter is the identity: the converted weight has the reference's size
+    assert lib.bitlinear_repacked_size(2560, 6912) == 2560 * 6912 // 4
+    assert lib.bitlinear_repacked_size(100, 2560) == 0 and lib.bitlinear_repacked_size(2560, 100) == 0
+    assert lib.bitlinear_repack(None, None, 100, 2560, None) == 1 and lib.bitlinear_repack(None, None, 2560, 2560, None) == 2
+    assert lib.bitlinear_quant_absmax_rowsum(None, None, None, None, 1, 2560, 0, None) == 2
     assert lib.bitlinear_status_string(0) == b"ok"
     assert b"shape" in lib.bitlinear_status_string(1)
     assert lib.bitlinear_set_tuning(2, 8, 4, 0) == 0

@@ -980,6 +980,39 @@ def test_forward_kernel_whose_waves_quantize_their_own_slices(n, k, m, shape, co
     _assert_bits_equal(host_bits(out4), want1, "mode 1")
 
 
+def test_quantizer_row_sums_and_the_identity_repack():
+    """bitlinear_quant_absmax_rowsum: q and s as the plain quantizer, rowsum[m] =
+    sum_k q[m, k]; bitlinear_repack: the converted weight is byte-identical to
+    what the reference packer wrote, and the product on it equals the product on
+    the original."""
+    import ctypes
+
+    lib = _lib.load_library()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    for m, k, mode in ((1, 2560, 0), (5, 6912, 0), (3, 27648, 1), (16, 64, 0), (2, 8, 1)):
+        rng = np.random.default_rng(m * 7 + k)
+        xb = o.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32) * 3.0)
+        x = dev_bf16(xb)
+        q = torch.empty(m, k, dtype=torch.int8, device="cuda")
+        s = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+        rs = torch.full((m,), 12345, dtype=torch.int32, device="cuda")
+        assert lib.bitlinear_quant_absmax_rowsum(P(x), P(q), P(s), P(rs), m, k, mode, None) == 0
+        torch.cuda.synchronize()
+        wq, wsb = o.quant_input(xb, mode)
+        assert np.array_equal(q.cpu().numpy(), wq) and np.array_equal(host_bits(s), wsb)
+        assert np.array_equal(rs.cpu().numpy(), wq.astype(np.int64).sum(axis=1).astype(np.int32))
+    n, k = 3840, 2560
+    w, a = _rand_case(n, k, 2, seed=4)
+    pk = _packed_dev(w)
+    assert lib.bitlinear_repacked_size(n, k) == pk.numel()
+    conv = torch.zeros_like(pk)
+    assert lib.bitlinear_repack(P(pk), P(conv), n, k, None) == 0
+    assert lib.bitlinear_repack(P(pk), P(pk), n, k, None) == 0  # in place
+    torch.cuda.synchronize()
+    assert torch.equal(conv, pk)
+    assert torch.equal(bitlinear.bitnet_int8xint2_acc(dev_i8(a), conv), bitlinear.bitnet_int8xint2_acc(dev_i8(a), pk))
+
+
 def test_3d_input_and_out_argument():
     n, k = 2560, 2560
     w, a = _rand_case(n, k, 6, seed=3)
