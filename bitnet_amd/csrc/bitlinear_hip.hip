@@ -1533,44 +1533,63 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_fused_kernel(
 // the outputs.  A wave's instruction stream is what a call of this size costs, and this one is
 // about half as long as the shared-prologue kernel's.
 constexpr int kSoloMaxTokens = 4;
+constexpr int kSoloRedSlots = 32;  // partial tiles a workgroup keeps (one token; 16 with more): row blocks x waves per row block
 constexpr int kSoloMaxUPW = 8;  // at most 8 k-steps (512 k = 64 vectors of 8 values) per wave: one slice vector per lane
 
 // COOP: the row maximum is taken over the workgroup's slices and exchanged through LDS (one barrier more,
 // no redundant reads of the rows): for rows too long for every wave to scan them
-template <int UPW, int VROW, int MT, bool COOP>
+// PRO 1: RMSNorm in front of the quantizer (aux = its weights), 2: squared-ReLU gate, then the RMSNorm (x holds
+// [M, 2K] = (x1 | x3)); both with the sums of squares exchanged like the maxima (COOP only, one more barrier).
+// RES: out = bf16(residual + bf16(result)).  The arithmetic is that of bitlinear_fused_kernel's prologues.
+// RPW: 16-row blocks per wave.  A wave multiplies its slice with the words of RPW consecutive row blocks: the
+// slice is prepared once for all of them (with many row blocks the preparation, repeated in every wave of the
+// machine, is what the vector units spend their time on).
+template <int UPW, int VROW, int MT, bool COOP, int PRO, bool RES, int RPW>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     // parameter order: what stands between the kernel's entry and its first loads comes first
     // (the weight scales' slots are runs of slot_rows output rows each, the reference's rule n / (N / ws_num):
     // one integer among the leading arguments instead of a table behind them)
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, int slot_rows,
-    const uint16_t* __restrict__ ws, uint16_t* __restrict__ out, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
+    const uint16_t* __restrict__ aux, const uint16_t* __restrict__ ws, uint16_t* __restrict__ out,
+    const uint16_t* __restrict__ residual, float eps, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
     int32_t* __restrict__ acc_out) {
+    static_assert(PRO == 0 || COOP, "the norm prologues exchange their partial sums between the waves");
     __shared__ __attribute__((aligned(16))) int8_t lds_q[kMaxWaves][MT][kSoloMaxUPW * 64];  // a wave's quantized slice per token
-    __shared__ __attribute__((aligned(16))) int red[kMaxWaves][256];                        // a wave's partial 16 x 16 tile
+    __shared__ __attribute__((aligned(16))) int red[MT == 1 ? kSoloRedSlots : kMaxWaves][256];                    // a wave's partial 16 x 16 tiles, [row block * S + k slice]
     __shared__ uint32_t wmax[kMaxWaves][MT];                                                // COOP: a wave's slice maximum per token
+    __shared__ double wsq[PRO ? kMaxWaves : 1][MT];                                         // PRO 1, 2: a wave's slice sum of squares per token
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int rbl = (wave >= S ? 1 : 0) + (wave >= 2 * S ? 1 : 0) + (wave >= 3 * S ? 1 : 0);  // wave / S, RB <= 4
     const int ks = wave - rbl * S;
-    const int rb = blockIdx.x * RB + rbl;
-    const bool rows_ok = rb < (N >> 4);
+    const int rb = (blockIdx.x * RB + rbl) * RPW;  // the wave's first row block
     const int g = lane >> 4;
     const int p = lane & 15;
 
     // requests, all at once: the slice's vectors (needed last, but they are part of the rows and
     // return with them), the whole rows for the maximum, then the weight words
-    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00020000);
+    const int xstride = PRO == 2 ? 2 * K : K;  // elements between token rows of x
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * xstride * 2, 0x00020000);
     const int slice_k0 = ks * (UPW * 64);
     const bool slice_lane = lane < UPW * 8 && slice_k0 + lane * 8 < K;
     uint4 sv[MT];
+    uint4 s3[PRO == 2 ? MT : 1];
     uint4 rv[MT][VROW];
+    uint4 gvec = make_uint4(0u, 0u, 0u, 0u);
+    if (PRO != 0) {
+        const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)aux, 0, K * 2, 0x00020000);
+        gvec = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, slice_lane ? (slice_k0 + lane * 8) * 2 : 0x7ffffff0, 0, 0));
+    }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        const int row_off = (m < M ? m : M - 1) * K * 2;
+        const int row_off = (m < M ? m : M - 1) * xstride * 2;
         // a lane without a slice vector, or a vector past the end of the row, asks past the end of the buffer: zeros, no access
         sv[m] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
                                               x_rsrc, slice_lane ? row_off + (slice_k0 + lane * 8) * 2 : 0x7ffffff0, 0, 0));
+        if (PRO == 2)
+            s3[m] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  x_rsrc, slice_lane ? row_off + (K + slice_k0 + lane * 8) * 2 : 0x7ffffff0, 0, 0));
         if (!COOP) {
 #pragma unroll
             for (int v = 0; v < VROW; ++v) {
@@ -1580,17 +1599,22 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
         }
     }
     const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
-    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)((const char*)wq + (size_t)(rows_ok ? rb : 0) * K * 4), 0, rows_ok ? K * 4 : 0, 0x00020000);
+    // one descriptor per row block, spanning exactly its K * 4 bytes: a k-step past the end of K reads as zero
     const int w_voff = lane_word * 4 + ks * (UPW * 256);
-    uint32_t w[UPW];
+    uint32_t w[RPW][UPW];
 #pragma unroll
-    for (int j = 0; j < UPW; ++j) w[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + j * 256, 0, 2 /* nt */);
+    for (int i = 0; i < RPW; ++i) {
+        const bool rows_ok = rb + i < (N >> 4);
+        const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)((const char*)wq + (size_t)(rows_ok ? rb + i : 0) * K * 4), 0, rows_ok ? K * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) w[i][j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + j * 256, 0, 2 /* nt */);
+    }
     // epilogue operand, raw bits: the weight scale of the workgroup's first row (a workgroup that
     // straddles a slot boundary fetches per row in the epilogue); the slot by a few scalar
     // comparisons (at most six slots), so that this request leaves with the others
-    const int n_first = blockIdx.x * RB * 16;
-    const int n_last = (n_first + RB * 16 - 1) < N ? (n_first + RB * 16 - 1) : N - 1;
+    const int n_first = blockIdx.x * RB * RPW * 16;
+    const int n_last = (n_first + RB * RPW * 16 - 1) < N ? (n_first + RB * RPW * 16 - 1) : N - 1;
     int slot_first = 0, slot_last = 0;
 #pragma unroll
     for (int j = 1; j < kMaxSeg; ++j) {
@@ -1598,7 +1622,42 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
         slot_last += n_last >= j * slot_rows ? 1 : 0;
     }
     const uint16_t wsb_first = ws[slot_first];
+    const int nthreads = 64 * RB * S;
+    uint16_t e_res[kFusedMaxRB];
+    if (RES) {
+        // the residual values of the output slots this thread will finish; slots it does not own get an
+        // offset past the end of the descriptor, which costs no memory access
+        const __amdgpu_buffer_rsrc_t r_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)residual, 0, M * N * 2, 0x00020000);
+#pragma unroll
+        for (int r = 0; r < kFusedMaxRB; ++r) {
+            const int t = tid + r * nthreads;
+            const int n = (blockIdx.x * RB * RPW + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
+            const int m = t & 15;
+            const bool live = t < RB * RPW * 256 && m < M && n < N;
+            e_res[r] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r_rsrc, live ? (m * N + n) * 2 : 0x7fff0000, 0, 0);
+        }
+    }
     __builtin_amdgcn_sched_barrier(0);  // every request above is on its way before anything below is looked at
+
+    if (PRO != 0) {
+        // gate (PRO 2), the slices' sums of squares exchanged (fp64: exact, so the order of the additions does
+        // not matter), then y = bf16(h * rstd * g) on the wave's own slice
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (PRO == 2) sv[m] = glu8(sv[m], s3[m]);
+            const double wsum = wave_sum_f64(sumsq8(sv[m]));  // lanes without a slice vector hold zeros
+            if (lane == 0) wsq[wave][m] = wsum;
+        }
+        lds_barrier();
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            double total = 0.0;
+            for (int k = 0; k < S; ++k) total += wsq[rbl * S + k][m];
+            const float mean = (float)total / (float)K;
+            const float rstd = 1.0f / __builtin_sqrtf(mean + eps);
+            sv[m] = norm8(sv[m], gvec, rstd);
+        }
+    }
 
     // row maxima -> scales; this wave's slice -> int8 in its LDS region, with the slice's sum
     float sf[MT];
@@ -1643,23 +1702,24 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     v4i b[UPW];
 #pragma unroll
     for (int j = 0; j < UPW; ++j) b[j] = *(const v4i*)(brow + j * 64);
-    v4i acc = {0, 0, 0, 0};
-#pragma unroll
-    for (int j = 0; j < UPW; ++j) {
-        const uint32_t wj = w[j];  // zero past the end of K
-        v4i e;
-        e.x = (int)(wj & 0x03030303u);
-        e.y = (int)((wj >> 2) & 0x03030303u);
-        e.z = (int)((wj >> 4) & 0x03030303u);
-        e.w = (int)((wj >> 6) & 0x03030303u);
-        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(e, b[j], acc, 0, 0, 0);
-    }
     // lane holds token p, rows 4 g + i in register i; the +2 of the codes goes with the slice's sum
     int q2 = qsum2[0];
 #pragma unroll
     for (int m = 1; m < MT; ++m) q2 = p == m ? qsum2[m] : q2;
-    {
-        int* dst = &red[wave][lane];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            const uint32_t wj = w[i][j];  // zero past the end of K
+            v4i e;
+            e.x = (int)(wj & 0x03030303u);
+            e.y = (int)((wj >> 2) & 0x03030303u);
+            e.z = (int)((wj >> 4) & 0x03030303u);
+            e.w = (int)((wj >> 6) & 0x03030303u);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(e, b[j], acc, 0, 0, 0);
+        }
+        int* dst = &red[(rbl * RPW + i) * S + ks][lane];
         dst[0] = acc.x - q2;
         dst[64] = acc.y - q2;
         dst[128] = acc.z - q2;
@@ -1668,15 +1728,14 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     lds_barrier();
 
     // every thread finishes the output slots t = tid, tid + nthreads, ... of the workgroup: [row block][reg][lane]
-    const int nthreads = 64 * RB * S;
 #pragma unroll
     for (int r = 0; r < kFusedMaxRB; ++r) {
         const int t = tid + r * nthreads;
-        if (t >= RB * 256) break;
+        if (t >= RB * RPW * 256) break;
         const int l = t & 63;
         const int m = l & 15;
         const int tb = t >> 8;  // row block of the slot
-        const int n = (blockIdx.x * RB + tb) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
+        const int n = (blockIdx.x * RB * RPW + tb) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
         if (m < M && n < N) {
             int sum = 0;
             for (int k = 0; k < S; ++k) sum += red[tb * S + k][t & 255];
@@ -1686,7 +1745,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
             for (int mm = 1; mm < MT; ++mm) sv_ = m == mm ? sf[mm] : sv_;
             uint16_t wsb = wsb_first;
             if (slot_first != slot_last) wsb = ws[n / slot_rows];  // uniform branch, rare
-            if (out) out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sv_ * bf16_to_f32(wsb));
+            uint16_t o = f32_to_bf16_rne((float)sum / sv_ * bf16_to_f32(wsb));
+            if (RES) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
+            if (out) out[(size_t)m * N + n] = o;
         }
     }
 }
@@ -1718,6 +1779,7 @@ struct Tuning {
                            // with that many row blocks per workgroup, 5 = never
     int solo_s = 0, solo_upw = 0;  // its waves per row block and k-steps per wave when forced
     int solo_coop = 0;             // row maximum: 0 = built-in choice, 1 = exchanged between the waves, 2 = every wave scans the rows
+    int solo_rpw = 0;              // row blocks per wave: 0 = built-in choice, 1, 2, 4
 };
 std::mutex g_tuning_mutex;
 Tuning g_tuning_shared;
@@ -1989,7 +2051,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 // must cover K / 64; instances exist for one token (rows up to 8192 values), two (up to 4096) and
 // three or four (up to 2560).
 struct SoloPlan {
-    int rb, s, upw, vrow, mt;
+    int rb, s, upw, vrow, mt, rpw;
     bool coop;
     bool ok;
 };
@@ -2005,10 +2067,20 @@ bool solo_wanted(int M, int N, int K) {
     return M == 2 && (N / 16) < 432;
 }
 
-SoloPlan plan_solo(int M, int N, int K) {
-    SoloPlan pl = {1, 8, 5, 5, 1, false, false};
+// The same with an RMSNorm (pro 1) or gate + RMSNorm (pro 2) in front: measured against the shared-prologue kernel
+// at one token, see bitlinear_norm_forward_bf16.
+bool solo_norm_wanted(int M, int N, int K, int pro) {
+    (void)N;
+    // measured at one token (shared-prologue kernel -> this one): 3840 x 2560 3.95 -> 3.80 us, 2560 x 2560 with
+    // the residual 3.91 -> 3.80, 13824 x 2560 5.44 -> 5.16; 2560 x 6912 with the gate and the residual 5.87 -> 6.12
+    // (not taken); two to four tokens 4.7 -> 4.9 and worse (not taken)
+    return M == 1 && pro == 1 && K <= 4096;
+}
+
+SoloPlan plan_solo(int M, int N, int K, int pro = 0, bool has_res = false) {
+    SoloPlan pl = {1, 8, 5, 5, 1, 1, false, false};
     if (M < 1 || M > kSoloMaxTokens) return pl;
-    if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31 || (long long)M * K * 2 >= 0x7ffffff0ll) return pl;
+    if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31 || (long long)M * K * 4 >= 0x7ffffff0ll) return pl;
     const int units = K / 64;
     const int need_v = (K + 511) / 512;
     pl.mt = M == 1 ? 1 : (M == 2 ? 2 : 4);
@@ -2016,7 +2088,7 @@ SoloPlan plan_solo(int M, int N, int K) {
     // every wave scans the whole rows while they are short and there is one token; otherwise the
     // row maximum is exchanged between the waves of the workgroup
     pl.coop = t_tune.solo_coop == 1 || (t_tune.solo_coop == 0 && (need_v > 8 || M > 1));
-    if (need_v > vmax) pl.coop = true;
+    if (need_v > vmax || pro != 0) pl.coop = true;
     pl.vrow = pl.coop ? 1 : (need_v <= 5 ? 5 : (need_v <= 8 ? 8 : (need_v <= 14 ? 14 : 16)));
     if (t_tune.solo >= 1 && t_tune.solo <= 4) {
         pl.rb = t_tune.solo;
@@ -2038,7 +2110,26 @@ SoloPlan plan_solo(int M, int N, int K) {
             }
         if (pl.upw == 0) pl.upw = 8;
         pl.s = (units + pl.upw - 1) / pl.upw;
+        // one token and many row blocks: waves of five k-steps that take two or four row blocks each, so that a
+        // slice is prepared once for all of them (13824 x 2560: 4.80 -> 4.46 us; with the RMSNorm in front 5.44,
+        // the shared-prologue kernel's time, -> 5.16)
+        if (M == 1 && pro <= 1 && !has_res && blocks16 >= 432 && (units + 4) / 5 <= 16 && (pl.coop || pl.vrow == 5)) {
+            const int s5 = (units + 4) / 5;
+            int rpw = blocks16 >= 864 ? 4 : 2;
+            while (rpw > 1 && (rpw * s5 > kSoloRedSlots || rpw > s5)) --rpw;
+            if (rpw > 1) {
+                pl.upw = 5;
+                pl.s = s5;
+                pl.rpw = rpw;
+            }
+        }
     }
+    // several row blocks per wave: instances exist for one token, 5 or 8 k-steps per wave, and the plain or
+    // norm prologue without residual
+    if (t_tune.solo_rpw >= 1) pl.rpw = t_tune.solo_rpw;
+    if (pl.rpw > 1 && !(M == 1 && (pl.upw == 5 || pl.upw == 8) && pro <= 1 && !has_res && (pl.coop || pl.vrow == 5) && pl.s >= pl.rpw &&
+                        pl.rb * pl.rpw * pl.s <= kSoloRedSlots && pl.rpw >= 2 && pl.rpw <= 4))
+        pl.rpw = 1;
     pl.ok = pl.rb >= 1 && pl.rb <= kFusedMaxRB && pl.s >= 1 && pl.rb * pl.s <= kMaxWaves && pl.s * pl.upw >= units &&
             (pl.upw == 4 || pl.upw == 5 || pl.upw == 7 || pl.upw == 8);
     return pl;
@@ -2046,19 +2137,60 @@ SoloPlan plan_solo(int M, int N, int K) {
 
 int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* ws,
                 const ScaleMap& smap, int8_t* q_out, uint16_t* s_out, int M, int N, int K, const SoloPlan& pl,
-                hipStream_t stream) {
+                hipStream_t stream, int pro = 0, const uint16_t* norm_weight = nullptr, float eps = 0.0f,
+                const uint16_t* residual = nullptr) {
     const int blocks16 = N / 16;
-    const dim3 grid((blocks16 + pl.rb - 1) / pl.rb, 1, 1);
+    const dim3 grid((blocks16 + pl.rb * pl.rpw - 1) / (pl.rb * pl.rpw), 1, 1);
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
     // equal slots only (what the forward entry points use): rows per slot
     const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
     for (int j = 0; j + 1 < smap.nseg; ++j)
         if (smap.ends[j] != (j + 1) * slot_rows) return BITLINEAR_ERR_ARG;
-    g_last_kernel = "bitlinear_solo_kernel";
-#define BITLINEAR_LAUNCH_SOLO(U, V, T, C)                                                                            \
-    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, slot_rows, \
-                       ws, out, q_out, s_out, acc_out)
+    if (pro != 0 && (!pl.coop || !norm_weight)) return BITLINEAR_ERR_ARG;
+    g_last_kernel = pro == 0 ? "bitlinear_solo_kernel" : (pro == 1 ? "bitlinear_solo_kernel<norm>" : "bitlinear_solo_kernel<gate+norm>");
+#define BITLINEAR_LAUNCH_SOLO_W(U, V, T, C, P, R, W)                                                                      \
+    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C, P, R, W>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, \
+                       slot_rows, norm_weight, ws, out, residual, eps, q_out, s_out, acc_out)
+#define BITLINEAR_LAUNCH_SOLO_P(U, V, T, C, P, R) BITLINEAR_LAUNCH_SOLO_W(U, V, T, C, P, R, 1)
+#define BITLINEAR_LAUNCH_SOLO(U, V, T, C) BITLINEAR_LAUNCH_SOLO_P(U, V, T, C, 0, false)
+    if (pl.rpw > 1) {
+        // one token, several row blocks per wave (plan_solo admits only what is instantiated here)
+        if (residual || pro > 1 || pl.mt != 1) return BITLINEAR_ERR_ARG;
+#define BITLINEAR_LAUNCH_SOLO_RW(U, W)                                        \
+    if (pro == 1) BITLINEAR_LAUNCH_SOLO_W(U, 1, 1, true, 1, false, W);        \
+    else if (pl.coop) BITLINEAR_LAUNCH_SOLO_W(U, 1, 1, true, 0, false, W);    \
+    else BITLINEAR_LAUNCH_SOLO_W(U, 5, 1, false, 0, false, W)
+        if (pl.upw == 8) {
+            if (pl.rpw == 2) { BITLINEAR_LAUNCH_SOLO_RW(8, 2); } else if (pl.rpw == 3) { BITLINEAR_LAUNCH_SOLO_RW(8, 3); } else { BITLINEAR_LAUNCH_SOLO_RW(8, 4); }
+        } else {
+            if (pl.rpw == 2) { BITLINEAR_LAUNCH_SOLO_RW(5, 2); } else if (pl.rpw == 3) { BITLINEAR_LAUNCH_SOLO_RW(5, 3); } else { BITLINEAR_LAUNCH_SOLO_RW(5, 4); }
+        }
+#undef BITLINEAR_LAUNCH_SOLO_RW
+        return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    }
+    // norm / gate prologues: the exchanging variant only, with or without the residual epilogue
+#define BITLINEAR_LAUNCH_SOLO_N(U, T)                                        \
+    if (pro == 1) {                                                          \
+        if (residual) BITLINEAR_LAUNCH_SOLO_P(U, 1, T, true, 1, true);       \
+        else BITLINEAR_LAUNCH_SOLO_P(U, 1, T, true, 1, false);               \
+    } else {                                                                 \
+        if (residual) BITLINEAR_LAUNCH_SOLO_P(U, 1, T, true, 2, true);       \
+        else BITLINEAR_LAUNCH_SOLO_P(U, 1, T, true, 2, false);               \
+    }
+#define BITLINEAR_LAUNCH_SOLO_NU(U)                          \
+    if (pl.mt == 1) { BITLINEAR_LAUNCH_SOLO_N(U, 1) }        \
+    else if (pl.mt == 2) { BITLINEAR_LAUNCH_SOLO_N(U, 2) }   \
+    else { BITLINEAR_LAUNCH_SOLO_N(U, 4) }
+    if (pro != 0) {
+        switch (pl.upw) {
+            case 4: BITLINEAR_LAUNCH_SOLO_NU(4); break;
+            case 5: BITLINEAR_LAUNCH_SOLO_NU(5); break;
+            case 7: BITLINEAR_LAUNCH_SOLO_NU(7); break;
+            default: BITLINEAR_LAUNCH_SOLO_NU(8); break;
+        }
+        return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    }
 #define BITLINEAR_LAUNCH_SOLO_U(U)                                      \
     if (pl.coop) {                                                      \
         if (pl.mt == 1) BITLINEAR_LAUNCH_SOLO(U, 1, 1, true);           \
@@ -2082,7 +2214,11 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
         default: BITLINEAR_LAUNCH_SOLO_U(8); break;
     }
 #undef BITLINEAR_LAUNCH_SOLO_U
+#undef BITLINEAR_LAUNCH_SOLO_NU
+#undef BITLINEAR_LAUNCH_SOLO_N
 #undef BITLINEAR_LAUNCH_SOLO
+#undef BITLINEAR_LAUNCH_SOLO_P
+#undef BITLINEAR_LAUNCH_SOLO_W
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
@@ -2371,7 +2507,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = 0;
+        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -2388,8 +2524,9 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 9) {
-        if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 0 || a > 2 || b < 0 || b > 4) return set_status(BITLINEAR_ERR_ARG);
         g.solo_coop = a;
+        g.solo_rpw = b;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 8) {
@@ -2665,6 +2802,13 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, 
     if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)norm_weight) | ((uintptr_t)q_ws)) & 15u)
         return set_status(BITLINEAR_ERR_ARG);
     const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    // up to four tokens: the kernel whose waves prepare their own slices
+    if (mode == 0 && t_tune.path == 0 && t_tune.solo != 5 && M <= kSoloMaxTokens) {
+        const SoloPlan sp = plan_solo(M, N, K, glu ? 2 : 1, residual != nullptr);
+        if (sp.ok && (t_tune.solo >= 1 || solo_norm_wanted(M, N, K, glu ? 2 : 1)))
+            return set_status(launch_solo(x, packed, output0, nullptr, ws, sm, nullptr, nullptr, M, N, K, sp,
+                                          (hipStream_t)stream, glu ? 2 : 1, norm_weight, eps, residual));
+    }
     const FusedPlan pl = plan_fused(M, N, K, glu ? 2 : 1);
     const bool small = (long long)M * K <= kFuseMaxElemsNorm || t_tune.path == 3 || !q_ws || !s_ws;
     if (pl.ok && small && t_tune.path != 4) {

@@ -277,8 +277,12 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *   kernel 9: how that kernel takes the row maximum: a = 0 built-in choice, 1 =
  *             slice maxima exchanged between the waves of a workgroup (one
  *             barrier), 2 = every wave scans the whole rows (no barrier; one
- *             token up to K = 8192, two up to 4096, more up to 2560).
- *             Kernel 0 resets it.
+ *             token up to K = 8192, two up to 4096, more up to 2560);
+ *             b = 16-row blocks a wave multiplies its slice with: 0 built-in
+ *             choice, 1..4 (more than one: one token, 5 or 8 k-steps per wave,
+ *             at most as many as waves per row block; otherwise one).
+ *             bitlinear_norm_forward_bf16 takes the same kernel (always
+ *             exchanging) under the kernel 8 settings.  Kernel 0 resets it.
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 

@@ -685,6 +685,43 @@ def test_fused_norm_gate_residual_forward(n, k, m, path, glu, res):
     _assert_bits_equal(host_bits(out), want, f"norm forward glu={glu} res={res}")
 
 
+@pytest.mark.parametrize("glu,res", [(0, 0), (0, 1), (1, 1), (1, 0)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("n,k,s_,upw", [(2560, 2560, 8, 5), (13824, 2560, 5, 8), (2560, 6912, 16, 7), (48, 192, 1, 4),
+                                        (1040, 3200, 10, 5), (1040, 3200, 8, 7), (64, 8192, 16, 8)])
+def test_solo_norm_gate_residual_forward(n, k, s_, upw, m, glu, res):
+    """The kernel whose waves prepare their own slices, with the RMSNorm / gate
+    prologues and the residual epilogue, forced for one to four tokens (the
+    library takes it by itself at one token): bit for bit against the oracle
+    chain, and the kernel that ran is the one meant."""
+    import ctypes
+
+    lib = _lib.load_library()
+    rng = np.random.default_rng(3 * n + k + m + 7 * glu + res)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    xin = rng.standard_normal((m, 2 * k if glu else k)).astype(np.float32) * 2.3
+    xin[0, 5] = -41.0  # the row maximum sits in one wave's slice
+    xb = o.f32_to_bf16_bits(xin)
+    gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+    rb = o.f32_to_bf16_bits(rng.standard_normal((m, n)).astype(np.float32)) if res else None
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=bool(glu), residual_bits=rb)
+    x, g, pk, wsd = dev_bf16(xb), dev_bf16(gb), _packed_dev(w), dev_bf16(ws_bits)
+    r = dev_bf16(rb) if res else None
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    assert lib.bitlinear_set_tuning(8, 1, s_, upw) == 0
+    try:
+        st = lib.bitlinear_norm_forward_bf16(P(x), P(g), 1e-5, glu, P(pk), P(wsd), P(r), P(out), None, None, m, n, k, 0, None)
+        name = bitlinear.last_kernel()
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert st == 0
+    assert name == ("bitlinear_solo_kernel<gate+norm>" if glu else "bitlinear_solo_kernel<norm>")
+    _assert_bits_equal(host_bits(out), want, f"solo norm forward glu={glu} res={res}")
+
+
 def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
     import ctypes
 
@@ -700,7 +737,8 @@ def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
     xb = o.f32_to_bf16_bits(rng.standard_normal((8, k)).astype(np.float32))
     want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=None)
     out = torch.full((8, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-    st = lib.bitlinear_norm_forward_bf16(P(dev_bf16(xb)), P(g), 1e-5, 0, P(pk), P(wsd), None, P(out), None, None, 8, n, k, 0, None)
+    xd8 = dev_bf16(xb)
+    st = lib.bitlinear_norm_forward_bf16(P(xd8), P(g), 1e-5, 0, P(pk), P(wsd), None, P(out), None, None, 8, n, k, 0, None)
     torch.cuda.synchronize()
     assert st == 0
     _assert_bits_equal(host_bits(out), want, "norm forward, no workspaces")
@@ -978,6 +1016,51 @@ def test_forward_kernel_whose_waves_quantize_their_own_slices(n, k, m, shape, co
     q1, s1 = o.quant_input(xb, 1)
     _, want1 = o.bitlinear_int8xint2(q1, w, s1, ws_bits)
     _assert_bits_equal(host_bits(out4), want1, "mode 1")
+
+
+@pytest.mark.parametrize("norm", [0, 1])
+@pytest.mark.parametrize("coop", [1, 2])
+@pytest.mark.parametrize("rpw", [0, 2, 3, 4])
+@pytest.mark.parametrize("n,k,s_,upw", [(13824, 2560, 8, 5), (13824, 2560, 5, 8), (7008, 2560, 8, 5), (80, 320, 1, 5),
+                                        (1040, 3200, 10, 5), (20480, 3200, 10, 5), (176, 2048, 4, 8)])
+def test_solo_kernel_with_several_row_blocks_per_wave(n, k, s_, upw, rpw, coop, norm):
+    """One token, waves that multiply their slice with two to four consecutive row
+    blocks (rpw = 0: the library's own plan, which takes them for many row blocks):
+    row-block counts that the group does not divide, three scale slots, a group
+    larger than the waves per row block (falls back to one); accumulators and
+    outputs bit for bit against the oracle chain, plain and behind the RMSNorm."""
+    import ctypes
+
+    lib = _lib.load_library()
+    if norm and coop == 2:
+        pytest.skip("the norm prologue always exchanges")
+    rng = np.random.default_rng(n + 3 * k + rpw)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    xb = o.f32_to_bf16_bits(rng.standard_normal((1, k)).astype(np.float32) * 3.0)
+    gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    pk, wsd = _packed_dev(w), dev_bf16(ws_bits)
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    try:
+        if rpw:
+            assert lib.bitlinear_set_tuning(8, 1, s_, upw) == 0
+            assert lib.bitlinear_set_tuning(9, coop, rpw, 0) == 0
+        if norm:
+            want = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=None)
+            out = torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            xd, gd = dev_bf16(xb), dev_bf16(gb)  # named: the device buffers must outlive the call
+            st = lib.bitlinear_norm_forward_bf16(P(xd), P(gd), 1e-5, 0, P(pk), P(wsd), None, P(out), None, None, 1, n, k, 0, None)
+            assert st == 0 and bitlinear.last_kernel() == "bitlinear_solo_kernel<norm>"
+        else:
+            q, s_bits = o.quant_input(xb, 0)
+            acc_want, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+            out, acc = bitlinear.bitlinear_forward_acc(dev_bf16(xb), pk, wsd)
+            assert bitlinear.last_kernel() == "bitlinear_solo_kernel"
+            assert np.array_equal(acc.cpu().numpy(), acc_want)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    _assert_bits_equal(host_bits(out), want, f"rpw={rpw}")
 
 
 def test_quantizer_row_sums_and_the_identity_repack():
