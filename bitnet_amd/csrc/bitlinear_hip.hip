@@ -612,7 +612,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 template <int MT, int NT, int KS>
 __global__ __launch_bounds__(kPfWaves * 64 * KS)
-__attribute__((amdgpu_waves_per_eu(MT == 2 && NT == 2 && KS == 1 ? 3 : 1)))
+__attribute__((amdgpu_waves_per_eu(MT == 2 && NT == 2 && KS == 1 ? 3 : (MT * NT == 8 && KS == 1 ? 2 : 1))))
 void gemm_i2_prefill_kernel(
     // parameter order: what the first loads need comes first (kernel-argument preload)
     // (band and seg_cols repeat gridDim.x / 8 and gridDim.y: the grid's own size is not among the preloaded dwords)
@@ -675,17 +675,14 @@ void gemm_i2_prefill_kernel(
     const __amdgpu_buffer_rsrc_t a_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(act + (size_t)m0 * K), 0, rows_here * K, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (N >> 2) * K, 0x00020000);
-    int a_off[PPT];
-    int a_dst[PPT];
-    int a_koff[PPT];
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-        const int pce = tid + i * NTHR;
-        const int row = pce / kPfPieces;
-        a_koff[i] = (pce % kPfPieces) * 16;
-        a_off[i] = row * K + a_koff[i];
-        a_dst[i] = row * kPfRowBytes + a_koff[i];
-    }
+    // (NTHR / kPfPieces = 16 rows per round i: piece i of a thread is its piece 0 moved down 16 * i rows, so one
+    // offset per thread and constants / scalar multiples of K do for all of them)
+    static_assert(NTHR % kPfPieces == 0, "a thread's pieces share their k offset");
+    constexpr int kRowsPerRound = NTHR / kPfPieces;
+    const int a_koff = (tid % kPfPieces) * 16;
+    const int a_off0 = (tid / kPfPieces) * K + a_koff;
+    const int a_dst0 = (tid / kPfPieces) * kPfRowBytes + a_koff;
+    const int a_round = kRowsPerRound * K;  // bytes between a thread's consecutive pieces in global memory
     // packed word of (column n, 32-k step, k-half kc), as a byte offset; columns past N re-read column N-1
     int w_off[NT];
 #pragma unroll
@@ -727,17 +724,22 @@ void gemm_i2_prefill_kernel(
     const int ones = 0x01010101;
     const int last_step_off = (ksteps - 1) * 128;  // byte offset of the last 32-k step inside a row block
     auto load_piece = [&](int c, int i) -> v4i {
-        // a chunk past the end re-reads chunk 0; it is never staged into a buffer that is multiplied
+        // a chunk past the end re-reads chunk 0; it is never staged into a buffer that is multiplied.
+        // The whole offset is the vector offset, the one the descriptor's range check sees: a piece past the end
+        // of K in the workgroup's last row, or in a row past M, lies beyond the descriptor and is not fetched
+        // (the scalar offset is outside that check).
         const int k0 = (c * KS + grp) * kPfChunk < K ? (c * KS + grp) * kPfChunk : 0;
-        return __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], k0, 0);
+        int base = a_off0 + k0;
+        asm volatile("" : "+v"(base));  // one add per piece here instead of PPT offsets kept in registers
+        return __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, base + i * a_round, 0, 0);
     };
     auto load_word = [&](int c, int ks, int nt) -> uint32_t {
         const int so = ((c * KS + grp) * kPfSteps + ks) * 128;
         return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_off[nt], so < last_step_off ? so : last_step_off, 0);
     };
     auto stage_piece = [&](int c, int i, const v4i& piece, int8_t* buf) {
-        const v4i v = ((c * KS + grp) * kPfChunk + a_koff[i]) >= K ? zero4 : piece;  // ragged last chunk, or a chunk past the end
-        *(v4i*)(buf + a_dst[i]) = v;
+        const v4i v = ((c * KS + grp) * kPfChunk + a_koff) >= K ? zero4 : piece;  // ragged last chunk, or a chunk past the end
+        *(v4i*)(buf + a_dst0 + i * (kRowsPerRound * kPfRowBytes)) = v;
         rs[i] = __builtin_amdgcn_sdot4(v.x, ones, rs[i], false);
         rs[i] = __builtin_amdgcn_sdot4(v.y, ones, rs[i], false);
         rs[i] = __builtin_amdgcn_sdot4(v.z, ones, rs[i], false);
@@ -1798,7 +1800,7 @@ constexpr int kStreamMinBlocks = 2048;
 constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
 constexpr int kPrefillFewTiles = 330;   // up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles
 constexpr int kPrefillSplit2Tiles = 320;  // up to this many 32 x 128 tiles two groups of waves split a tile's K,
-constexpr int kPrefillSplit4Tiles = 160;  // up to this many, and a long K, four
+constexpr int kPrefillSplit4Tiles = 200;  // up to this many, and a long K, four
 constexpr int kPrefillSplit4MinK = 5120;
 
 int set_status(int st) {
@@ -2251,6 +2253,13 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // us at 3840 x 2560, 21.5 -> 16.4 at 2560 x 6912).
     const long long narrow_tiles = (long long)((N + 127) / 128) * ((M + 63) / 64);
     int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : (narrow_tiles <= kPrefillFewTiles ? 4 : 0);
+    // 64 x 256 tiles run three workgroups per CU (768 at a time), 128 x 256 tiles two (512): with a little more than
+    // one full round of the former, one round of the latter finishes earlier (13824 x 2560 at M = 1024: 864 tiles,
+    // 46.5 -> 42.3 us; 3840 x 2560 at M = 4096: 960 tiles, 45.1 -> 44.1)
+    if (tile == 2) {
+        const long long wide_tiles = (long long)((N + 255) / 256) * ((M + 63) / 64);
+        if (wide_tiles > 768 && wide_tiles <= 1024) tile = 1;
+    }
     if (t_tune.path == 5) tile = t_tune.prefill_big;
     // groups of waves that split a tile's K between them (small tiles only): while the small tiles
     // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
@@ -2262,6 +2271,13 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // 11.6 -> 13.6 us)
     if (tile == 4 && small_tiles <= kPrefillSplit2Tiles)
         ks = (small_tiles <= kPrefillSplit4Tiles && K >= kPrefillSplit4MinK) ? 4 : 2;
+    // between half a tile and about one tile of 64 x 128 per CU: those tiles, with two groups of waves each
+    // (2560 x 6912: M = 512 19.1 -> 17.3 us, M = 640 20.5 -> 17.7, M = 768 22.1 -> 20.0; 2560 x 2560: M = 640
+    // 10.2 -> 9.5; 3840 x 2560: M = 384 10.0 -> 9.5; with 240 tiles and K = 2560 10.7 -> 12.1..12.7, not taken)
+    if (t_tune.path != 5 && tile == 4 && narrow_tiles > 128 && narrow_tiles <= (K >= kPrefillSplit4MinK ? 256 : 216)) {
+        tile = 0;
+        ks = 2;
+    }
     if (t_tune.path == 5 && t_tune.prefill_ks > 0) ks = (tile == 4 || (tile == 0 && t_tune.prefill_ks == 2)) ? t_tune.prefill_ks : 1;
     if (K <= kPfChunk * (ks - 1)) ks = 1;  // fewer chunks than groups
     const dim3 block(kPfWaves * 64 * ks, 1, 1);
