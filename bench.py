@@ -263,6 +263,36 @@ def batched_and_prefill(lib, shapes, layers, scales, dev, decode_ms=(2, 4, 8, 16
     return out
 
 
+def mfma_ceiling(lib, dev, iters=20000):
+    """What v_mfma_i32_32x32x32_i8 sustains on this machine in a register-only
+    loop (bitlinear_probe_mfma_i8: three waves per SIMD, no memory traffic), for
+    all-zero operands and for the operand values of this workload (random int8
+    activations x random ternary codes, changing with every MFMA): the rate
+    depends on the values, because switching activity decides the power the
+    pipe draws and the clock it gets.  HIP events, best of 3 launches of about
+    20 to 30 ms each."""
+    import ctypes
+
+    import torch
+
+    out = {"how": "register-only loop of v_mfma_i32_32x32x32_i8, 3 waves per SIMD on every CU, HIP events, best of 3"}
+    for mode, name in ((0, "zero_operands_TOPS"), (1, "random_int8_x_ternary_codes_TOPS")):
+        ops = ctypes.c_longlong(0)
+        best = None
+        for _ in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            st = lib.bitlinear_probe_mfma_i8(mode, iters, None, ctypes.byref(ops), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            e1.record()
+            torch.cuda.synchronize()
+            assert st == 0
+            ms = e0.elapsed_time(e1)
+            best = ms if best is None else min(best, ms)
+        out[name] = round(ops.value / (best * 1e-3) / 1e12, 1)
+    out["nominal_peak_TOPS"] = INT8_MFMA_PEAK_TOPS
+    return out
+
+
 def large_shapes(lib, dev, budget_bytes=1 << 30):
     """The other (N, K) of the reference's dispatch table (bitnet_kernels.cu:4-33:
     the 3B-class and the largest shapes) at M = 1 through the drop-in entry
@@ -741,7 +771,12 @@ def main():
     if not args.no_sweeps:
         result.update(grouped_launches(lib, shapes, layers, scales, dev, 1))
         result.update(grouped_launches(lib, shapes, layers, scales, dev, 4))
-        result.update(batched_and_prefill(lib, shapes, layers, scales, dev))
+        bp = batched_and_prefill(lib, shapes, layers, scales, dev)
+        ceil = mfma_ceiling(lib, dev)
+        for leg in bp["prefill"].values():  # the nominal peak prices the roofline; the measured ceiling stands beside it
+            leg["roofline"]["frac_of_measured_ceiling"] = round(leg["layer_gemm_TOPS"] / ceil["random_int8_x_ternary_codes_TOPS"], 4)
+        bp["prefill"]["mfma_ceiling"] = ceil
+        result.update(bp)
         result.update(large_shapes(lib, dev))
     if not args.no_e2e:
         del path, gemv, quant, layers

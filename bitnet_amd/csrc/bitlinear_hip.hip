@@ -903,6 +903,76 @@ void gemm_i2_prefill_kernel(
                 }
         }
     }
+    if (out && !acc_out) {
+        // bf16 output through LDS: a lane holds one token and four consecutive columns per register quad, so
+        // storing from the accumulator layout writes 8-byte pieces of 32 different rows per instruction (a row's
+        // 128 bytes arrive as 16 separate partial writes).  Each wave instead parks the 32 rows of one row tile
+        // in a region of its own (the staging buffers are free: every wave is past the last chunk's barrier,
+        // and group 0 past the reduction), padded so that neither the 8-byte writes nor the 16-byte reads
+        // pile up on a bank, and stores them as 16-byte pieces, a row's bytes side by side: 4 * NT store
+        // instructions per wave and row tile, every one of them whole 64-byte runs.
+        constexpr int kRowB = NT * 64 + 16;                       // bytes per parked row
+        // (with several k-groups, behind the accumulators the other groups left: another wave of this group may still be adding its share)
+        constexpr int kRedBytes = (KS - 1) * kPfWaves * MT * NT * 16 * 64 * 4;
+        int8_t* park = lds_all + kRedBytes + wave * (32 * kRowB);
+        static_assert(kRedBytes + kPfWaves * 32 * kRowB <= KS * 2 * MT * 32 * kPfRowBytes, "parked rows must fit the staging buffers");
+        constexpr int kPiecesPerRow = NT * 4;                     // 16-byte pieces
+        constexpr int kRowsPerStore = 64 / kPiecesPerRow;
+        const int pr = lane / kPiecesPerRow, pc = lane % kPiecesPerRow;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int ml = mt * 32 + nl;
+            int rs2 = 0;
+#pragma unroll
+            for (int g = 0; g < KS; ++g) rs2 += 2 * rowsum[g][ml];
+            const float sv = sval[ml], ri = rinv[ml];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    float h[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float a = (float)(acc[mt][nt][g4 * 4 + j] - rs2);
+                        const float q0 = a * ri;
+                        const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
+                        h[j] = q * wsf[nt][g4 * 4 + j];
+                    }
+                    *(uint2*)(park + nl * kRowB + (nt * 32 + g4 * 8 + kc * 4) * 2) =
+                        make_uint2(f32x2_to_bf16x2(h[0], h[1]), f32x2_to_bf16x2(h[2], h[3]));
+                }
+            // the same wave wrote and reads: LDS operations of a wave complete in order
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int r0 = 0; r0 < 32; r0 += kRowsPerStore) {
+                const int row = r0 + pr;
+                const int m = m0 + mt * 32 + row;
+                const int n = n0 + pc * 8;  // N % 16 == 0 and n0 % 32 == 0: the eight columns are in or out together
+                uint4 v = *(const uint4*)(park + row * kRowB + pc * 16);
+                if (m < M && n < N) {
+                    const size_t o = (size_t)m * N + n;
+                    if (residual) {  // out = bf16(residual + bf16(result))
+                        const uint4 rv = *(const uint4*)(residual + o);
+                        const uint32_t a4[4] = {v.x, v.y, v.z, v.w}, r4[4] = {rv.x, rv.y, rv.z, rv.w};
+                        uint32_t o4[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            o4[j] = f32x2_to_bf16x2(__uint_as_float(r4[j] << 16) + __uint_as_float(a4[j] << 16),
+                                                    __uint_as_float(r4[j] & 0xffff0000u) + __uint_as_float(a4[j] & 0xffff0000u));
+                        v = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+                    }
+                    *(uint4*)(out + o) = v;
+                }
+            }
+            // the next row tile's writes must not overtake these reads
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int ml = mt * 32 + nl;
@@ -2463,6 +2533,60 @@ ScaleMap equal_slots(int N, int ws_num) {
     return sm;
 }
 
+// What the matrix pipe sustains on this machine for given operand VALUES: a register-only loop of
+// v_mfma_i32_32x32x32_i8 (three waves per SIMD on every CU, four accumulators per wave, no memory traffic).
+// mode 0: all operands zero; 1: random int8 activations x random codes 1..3 (the products this library
+// computes), eight operand pairs in rotation so that the inputs change with every MFMA.  The rate depends on
+// the values: switching activity decides the power the pipe draws and with it the clock it is given.
+__device__ __forceinline__ unsigned probe_hash32(unsigned x) {
+    x ^= x >> 16;
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void probe_mfma_i8_kernel(int iters, uint32_t* sink) {
+    v16i acc[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][r] = 0;
+    v4i act[8], code[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const unsigned seed = (threadIdx.x * 8 + i) * 4 + blockIdx.x * 977;
+        act[i] = v4i{0, 0, 0, 0};
+        code[i] = v4i{0, 0, 0, 0};
+        if (MODE == 1) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                act[i][j] = (int)probe_hash32(seed + j);
+                const unsigned h = probe_hash32(seed + 50 + j);
+                unsigned c = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) c |= (1u + ((h >> (8 * b)) & 0xffu) % 3u) << (8 * b);
+                code[i][j] = (int)c;
+            }
+        }
+    }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                acc[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(code[(u * 3 + a) & 7], act[(u + 2 * a) & 7], acc[a], 0, 0, 0);
+    }
+    int x = 0;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x ^= acc[a][r];
+    if (sink && x == 0x12345678) sink[0] = (uint32_t)x;  // keeps the loop alive; practically never true
+}
+
 }  // namespace
 
 extern "C" {
@@ -2474,6 +2598,20 @@ __global__ void probe_empty_kernel() {}
 int bitlinear_probe_empty(int blocks, int threads, void* stream) {
     if (blocks < 1 || threads < 1 || threads > 1024) return BITLINEAR_ERR_ARG;
     hipLaunchKernelGGL(probe_empty_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream);
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+int bitlinear_probe_mfma_i8(int mode, int iters, uint32_t* sink, long long* ops, void* stream) {
+    if ((mode != 0 && mode != 1) || iters < 1 || iters > (1 << 20)) return BITLINEAR_ERR_ARG;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        return BITLINEAR_ERR_LAUNCH;
+    const int blocks = 3 * cus;  // one wave per SIMD and workgroup, three workgroups per CU
+    if (mode == 0)
+        hipLaunchKernelGGL(probe_mfma_i8_kernel<0>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, iters, sink);
+    else
+        hipLaunchKernelGGL(probe_mfma_i8_kernel<1>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, iters, sink);
+    if (ops) *ops = 2ll * 32 * 32 * 32 * 32 * (long long)iters * 4 * blocks;  // 32 MFMAs per iteration and wave
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 

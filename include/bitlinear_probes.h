@@ -2,8 +2,8 @@
  * Measurement probes of libbitlinear_hip.so.  Not part of the drop-in interface
  * (the reference has no counterpart): bench.py uses them to measure, in the same
  * run and launch style as its headline, what a kernel launch costs on this
- * machine when the kernel does nothing and when it only requests a matrix's
- * bytes.  Same conventions as include/bitlinear_hip.h: device pointers owned by
+ * machine when the kernel does nothing, when it only requests a matrix's bytes,
+ * and what the matrix pipe sustains on the operand values of this workload.  Same conventions as include/bitlinear_hip.h: device pointers owned by
  * the caller, no allocation, no synchronisation, launches on the given stream.
  */
 #ifndef BITLINEAR_PROBES_H
@@ -29,6 +29,20 @@ int bitlinear_probe_empty(int blocks, int threads, void* stream);
  */
 int bitlinear_probe_weight_stream(const int8_t* const* packed, int count, int N, int K,
                                   uint32_t* sink, void* stream);
+
+/*
+ * One launch of a register-only loop of v_mfma_i32_32x32x32_i8 that fills every
+ * SIMD of the device with three waves (four accumulators per wave, 32 MFMAs
+ * per iteration, no memory traffic): what the matrix pipe sustains for given
+ * operand values.  mode 0: all operands zero; mode 1: random int8 activations
+ * x random codes 1..3 (the products this library computes), the operands
+ * changing with every MFMA.  The two differ, because switching activity
+ * decides the power the pipe draws and the clock it is given.  iters:
+ * 1..2^20.  *ops (host, may be NULL) receives the integer operations of the
+ * launch (2 per multiply-add).  sink: one device word that is practically
+ * never written (may be NULL).  Returns 0, 3 or 4 as above.
+ */
+int bitlinear_probe_mfma_i8(int mode, int iters, uint32_t* sink, long long* ops, void* stream);
 
 #ifdef __cplusplus
 }
