@@ -1063,6 +1063,23 @@ def test_solo_kernel_with_several_row_blocks_per_wave(n, k, s_, upw, rpw, coop, 
     _assert_bits_equal(host_bits(out), want, f"rpw={rpw}")
 
 
+def test_matrix_pipe_probe_runs_and_reports_its_operations():
+    """bitlinear_probe_mfma_i8 (the bench's ceiling leg): both operand modes
+    launch, report 32 MFMAs of 32 x 32 x 32 per iteration for three waves on
+    every SIMD, and refuse bad arguments."""
+    import ctypes
+
+    lib = _lib.load_library()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for mode in (0, 1):
+        ops = ctypes.c_longlong(0)
+        assert lib.bitlinear_probe_mfma_i8(mode, 10, None, ctypes.byref(ops), None) == 0
+        torch.cuda.synchronize()
+        assert ops.value == 2 * 32 ** 3 * 32 * 10 * 4 * 3 * cus
+    assert lib.bitlinear_probe_mfma_i8(2, 10, None, None, None) == 4
+    assert lib.bitlinear_probe_mfma_i8(0, 0, None, None, None) == 4
+
+
 def test_quantizer_row_sums_and_the_identity_repack():
     """bitlinear_quant_absmax_rowsum: q and s as the plain quantizer, rowsum[m] =
     sum_k q[m, k]; bitlinear_repack: the converted weight is byte-identical to
