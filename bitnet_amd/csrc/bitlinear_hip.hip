@@ -1825,6 +1825,129 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// The drop-in product (int8 rows in, up to 16 tokens) in the same decomposition: no staging at all
+// ---------------------------------------------------------------------------
+// A workgroup owns RB x RPW 16-row blocks, S waves split K, every wave multiplies exactly UPW k-steps
+// (bitlinear_solo_kernel's launch shapes).  The activation operand of a k-step -- 16 int8 of token p
+// for the 16 k of chunk g, p = lane % 16, g = lane / 16 -- is one 16-byte load per lane straight from
+// the caller's rows, requested together with the weight words: nothing passes through LDS before the
+// products and no wave waits for another.  The +2 of the stored codes leaves with a second product
+// per k-step whose row operand is all ones (sum_k a[p, k] in every row of the tile), shared by the
+// wave's row blocks.  One barrier, behind the products, as in bitlinear_solo_kernel.
+template <int UPW, int RPW, bool RES>
+__global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_solo_kernel(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, int slot_rows,
+    const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws, uint16_t* __restrict__ out,
+    const uint16_t* __restrict__ residual, int32_t* __restrict__ acc_out) {
+    __shared__ __attribute__((aligned(16))) int red[kSoloRedSlots][256];  // partial 16 x 16 tiles, [row block * S + k slice]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rbl = (wave >= S ? 1 : 0) + (wave >= 2 * S ? 1 : 0) + (wave >= 3 * S ? 1 : 0);  // wave / S, RB <= 4
+    const int ks = wave - rbl * S;
+    const int rb = (blockIdx.x * RB + rbl) * RPW;  // the wave's first row block
+    const int g = lane >> 4;
+    const int p = lane & 15;
+
+    // requests: the slice's activation operands (a token past M, or a k-step past the end of K, asks past
+    // the end of the descriptor: zeros, no access), then the weight words, then what the epilogue needs
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)act, 0, M * K, 0x00020000);
+    const int slice_k0 = ks * (UPW * 64);
+    v4i b[UPW];
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) {
+        const bool live = p < M && slice_k0 + j * 64 < K;  // K % 64 == 0: a k-step is inside K or outside
+        b[j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, live ? p * K + slice_k0 + j * 64 + g * 16 : 0x7ffffff0, 0, 0);
+    }
+    const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
+    const int w_voff = lane_word * 4 + ks * (UPW * 256);
+    uint32_t w[RPW][UPW];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+        // one descriptor per row block, spanning exactly its K * 4 bytes: a k-step past the end of K reads as zero
+        const bool rows_ok = rb + i < (N >> 4);
+        const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)((const char*)wq + (size_t)(rows_ok ? rb + i : 0) * K * 4), 0, rows_ok ? K * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) w[i][j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + j * 256, 0, 2 /* nt */);
+    }
+    const int n_first = blockIdx.x * RB * RPW * 16;
+    const int n_last = (n_first + RB * RPW * 16 - 1) < N ? (n_first + RB * RPW * 16 - 1) : N - 1;
+    int slot_first = 0, slot_last = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSeg; ++j) {
+        slot_first += n_first >= j * slot_rows ? 1 : 0;
+        slot_last += n_last >= j * slot_rows ? 1 : 0;
+    }
+    const uint16_t wsb_first = ws[slot_first];
+    const uint16_t e_sb = s[(tid & 15) < M ? (tid & 15) : M - 1];  // every output slot of a thread belongs to token tid % 16
+    const int nthreads = 64 * RB * S;
+    uint16_t e_res[kFusedMaxRB];
+    if (RES) {
+        const __amdgpu_buffer_rsrc_t r_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)residual, 0, M * N * 2, 0x00020000);
+#pragma unroll
+        for (int r = 0; r < kFusedMaxRB; ++r) {
+            const int t = tid + r * nthreads;
+            const int n = (blockIdx.x * RB * RPW + (t >> 8)) * 16 + 4 * ((t & 63) >> 4) + ((t >> 6) & 3);
+            const int m = t & 15;
+            const bool live = t < RB * RPW * 256 && m < M && n < N;
+            e_res[r] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r_rsrc, live ? (m * N + n) * 2 : 0x7fff0000, 0, 0);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // every request above is on its way before anything below is looked at
+
+    // sum_k a[p, k] over the slice, in the accumulator layout (every row of the tile holds it)
+    const int ones_w = 0x01010101;
+    const v4i ones = {ones_w, ones_w, ones_w, ones_w};
+    v4i asum = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, b[j], asum, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            const uint32_t wj = w[i][j];  // zero past the end of K
+            v4i e;
+            e.x = (int)(wj & 0x03030303u);
+            e.y = (int)((wj >> 2) & 0x03030303u);
+            e.z = (int)((wj >> 4) & 0x03030303u);
+            e.w = (int)((wj >> 6) & 0x03030303u);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(e, b[j], acc, 0, 0, 0);
+        }
+        // lane holds token p, rows 4 g + i in register i
+        int* dst = &red[(rbl * RPW + i) * S + ks][lane];
+        dst[0] = acc.x - 2 * asum.x;
+        dst[64] = acc.y - 2 * asum.y;
+        dst[128] = acc.z - 2 * asum.z;
+        dst[192] = acc.w - 2 * asum.w;
+    }
+    lds_barrier();
+
+    // every thread finishes the output slots t = tid, tid + nthreads, ... of the workgroup: [row block][reg][lane]
+    const float sf = bf16_to_f32(e_sb);
+#pragma unroll
+    for (int r = 0; r < kFusedMaxRB; ++r) {
+        const int t = tid + r * nthreads;
+        if (t >= RB * RPW * 256) break;
+        const int l = t & 63;
+        const int m = l & 15;
+        const int tb = t >> 8;  // row block of the slot
+        const int n = (blockIdx.x * RB * RPW + tb) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
+        if (m < M && n < N) {
+            int sum = 0;
+            for (int k = 0; k < S; ++k) sum += red[tb * S + k][t & 255];
+            if (acc_out) acc_out[(size_t)m * N + n] = sum;  // uniform: parity tests only
+            uint16_t wsb = wsb_first;
+            if (slot_first != slot_last) wsb = ws[n / slot_rows];  // uniform branch, rare
+            uint16_t o = f32_to_bf16_rne((float)sum / sf * bf16_to_f32(wsb));
+            if (RES) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
+            if (out) out[(size_t)m * N + n] = o;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 thread_local int g_status = BITLINEAR_OK;
@@ -1852,6 +1975,8 @@ struct Tuning {
     int solo_s = 0, solo_upw = 0;  // its waves per row block and k-steps per wave when forced
     int solo_coop = 0;             // row maximum: 0 = built-in choice, 1 = exchanged between the waves, 2 = every wave scans the rows
     int solo_rpw = 0;              // row blocks per wave: 0 = built-in choice, 1, 2, 4
+    int prod_solo = 0;             // the drop-in product through gemv_i2_solo_kernel: 0 = built-in choice, 1 = always (prod_s waves of prod_upw k-steps), 2 = never
+    int prod_s = 0, prod_upw = 0;
 };
 std::mutex g_tuning_mutex;
 Tuning g_tuning_shared;
@@ -2294,6 +2419,76 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 
+// Launch shape of gemv_i2_solo_kernel (up to 16 tokens): one row block per group of S waves, UPW k-steps per wave
+// as in plan_solo; with many row blocks a wave takes two or four of them.
+struct ProdPlan {
+    int s, upw, rpw;
+    bool ok;
+};
+
+ProdPlan plan_prod_solo(int M, int N, int K) {
+    ProdPlan pl = {8, 5, 1, false};
+    if (M < 1 || M > 16) return pl;
+    if ((size_t)N * (size_t)K / 4 >= (size_t)1 << 31) return pl;
+    const int units = K / 64;
+    const int blocks16 = N / 16;
+    if (t_tune.prod_solo == 1) {
+        pl.s = t_tune.prod_s;
+        pl.upw = t_tune.prod_upw;
+    } else {
+        const int order[4] = {5, 7, 8, 4};
+        pl.upw = 0;
+        for (int i = 0; i < 4; ++i)
+            if ((units + order[i] - 1) / order[i] <= (units > 64 ? kMaxWaves : 10)) {
+                pl.upw = order[i];
+                break;
+            }
+        if (pl.upw == 0) pl.upw = 8;
+        pl.s = (units + pl.upw - 1) / pl.upw;
+        // measured at 13824 x 2560: up to four tokens two row blocks per wave (4.19 / 4.22 / 4.33 us at one / two /
+        // four tokens, 4.39 / 4.41 / 4.49 with four), from eight tokens on four (4.62 against 4.67; 5.15 against 5.78 at 16)
+        if (blocks16 >= 432) pl.rpw = (blocks16 >= 864 && M > 4) ? 4 : 2;
+    }
+    if (t_tune.solo_rpw >= 1) pl.rpw = t_tune.solo_rpw;
+    if (pl.rpw == 3) pl.rpw = 2;
+    while (pl.rpw > 1 && (pl.rpw * pl.s > kSoloRedSlots || pl.rpw > pl.s)) pl.rpw >>= 1;
+    pl.ok = pl.s >= 1 && pl.s <= kMaxWaves && pl.s * pl.upw >= units && (pl.upw == 4 || pl.upw == 5 || pl.upw == 7 || pl.upw == 8);
+    return pl;
+}
+
+int launch_prod_solo(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
+                     const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, const ProdPlan& pl, hipStream_t stream,
+                     const uint16_t* residual) {
+    const int blocks16 = N / 16;
+    const dim3 grid((blocks16 + pl.rpw - 1) / pl.rpw, 1, 1);
+    const dim3 block(64 * pl.s, 1, 1);
+    const uint32_t* wq = (const uint32_t*)packed;
+    const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
+    for (int j = 0; j + 1 < smap.nseg; ++j)
+        if (smap.ends[j] != (j + 1) * slot_rows) return BITLINEAR_ERR_ARG;  // equal slots only
+    g_last_kernel = "gemv_i2_solo_kernel";
+#define BITLINEAR_LAUNCH_PS(U, W, R)                                                                               \
+    hipLaunchKernelGGL((gemv_i2_solo_kernel<U, W, R>), grid, block, 0, stream, act, wq, M, N, K, 1, pl.s, slot_rows, \
+                       s, ws, out, residual, acc_out)
+#define BITLINEAR_LAUNCH_PS_W(U, W)         \
+    if (residual) BITLINEAR_LAUNCH_PS(U, W, true); \
+    else BITLINEAR_LAUNCH_PS(U, W, false)
+#define BITLINEAR_LAUNCH_PS_U(U)                       \
+    if (pl.rpw == 1) { BITLINEAR_LAUNCH_PS_W(U, 1); }  \
+    else if (pl.rpw == 2) { BITLINEAR_LAUNCH_PS_W(U, 2); } \
+    else { BITLINEAR_LAUNCH_PS_W(U, 4); }
+    switch (pl.upw) {
+        case 4: BITLINEAR_LAUNCH_PS_U(4); break;
+        case 5: BITLINEAR_LAUNCH_PS_U(5); break;
+        case 7: BITLINEAR_LAUNCH_PS_U(7); break;
+        default: BITLINEAR_LAUNCH_PS_U(8); break;
+    }
+#undef BITLINEAR_LAUNCH_PS_U
+#undef BITLINEAR_LAUNCH_PS_W
+#undef BITLINEAR_LAUNCH_PS
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
 int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                    const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream,
                    const uint16_t* residual = nullptr) {
@@ -2503,6 +2698,22 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
             return launch_stream(&one, 1, M, N, K, smap, acc_out, stream);
         }
     }
+    // Up to 16 tokens through the kernel without staging, where it measured faster than the kernels below (LDS-staged
+    // up to four tokens, split-K beyond): many row blocks (13824 x 2560: 4.46 -> 4.19 us at one token, 4.88 -> 4.62
+    // at eight, 6.00 -> 5.15 at sixteen) and more than four tokens (3840 x 2560: 3.40 -> 3.34 at eight, 3.83 -> 3.72
+    // at sixteen; 2560 x 6912: 4.90 -> 4.71 and 6.11 -> 5.89); elsewhere the staged kernel stays (2.89 against 2.95
+    // at 3840 x 2560 and 3.65 against 4.06 at 2560 x 6912, one token)
+    const bool prod_solo_wanted = t_tune.prod_solo == 1 || (t_tune.prod_solo == 0 && t_tune.staged == 0 && ((N / 16) >= 432 || M > kDecodeMaxTokens) &&
+                                                            (N / 16) < kStreamMinBlocks);
+    if (prod_solo_wanted && t_tune.path != 1 && t_tune.path != 2 && M <= 16) {
+        const ProdPlan pp = plan_prod_solo(M, N, K);
+        bool equal = true;
+        const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
+        for (int j = 0; j + 1 < smap.nseg; ++j) equal = equal && smap.ends[j] == (j + 1) * slot_rows;
+        if (pp.ok && equal)
+            return launch_prod_solo(act, packed, out, acc_out, out ? s : (const uint16_t*)packed, out ? ws : (const uint16_t*)packed,
+                                    smap, M, N, K, pp, stream, residual);
+    }
     // (The accumulator export takes the same kernel choice as the drop-in call, so what the parity
     // tests read is what the drop-in entry computes.  Without an output there are no scales: the
     // kernel's unconditional scale requests then go to an address that exists.)
@@ -2661,7 +2872,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = 0;
+        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = g.prod_solo = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -2681,6 +2892,18 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         if (a < 0 || a > 2 || b < 0 || b > 4) return set_status(BITLINEAR_ERR_ARG);
         g.solo_coop = a;
         g.solo_rpw = b;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 10) {
+        if (a == 0 || a == 2) {
+            g.prod_solo = a;
+            return set_status(BITLINEAR_OK);
+        }
+        const bool upw_ok = c == 4 || c == 5 || c == 7 || c == 8;
+        if (a != 1 || b < 1 || b > kMaxWaves || !upw_ok) return set_status(BITLINEAR_ERR_ARG);
+        g.prod_solo = 1;
+        g.prod_s = b;
+        g.prod_upw = c;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 8) {

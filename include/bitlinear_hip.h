@@ -283,6 +283,13 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
  *             at most as many as waves per row block; otherwise one).
  *             bitlinear_norm_forward_bf16 takes the same kernel (always
  *             exchanging) under the kernel 8 settings.  Kernel 0 resets it.
+ *   kernel 10: the product of int8 rows (M <= 16) through the kernel that reads
+ *             its activation operands straight from the caller's rows (no
+ *             staging, one barrier): a = 0 built-in choice (many row blocks, or
+ *             more than four tokens), a = 1 always, with b waves per row block
+ *             and c (4, 5, 7 or 8) k-steps per wave (b * c * 64 must cover K,
+ *             else the built-in kernels run; row blocks per wave from kernel 9's
+ *             b), a = 2 never.  Applies with kernel 0 only; kernel 0 resets it.
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 

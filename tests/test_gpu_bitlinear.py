@@ -137,8 +137,9 @@ def test_default_path_accumulators_bit_exact_at_2b_shapes(shape_id, m):
     acc = bitlinear.bitnet_int8xint2_acc(qd, pk)
     k_acc = bitlinear.last_kernel()
     assert k_acc == k_dropin, (k_acc, k_dropin)
-    if m <= 4:
-        assert k_dropin == "bitlinear_fused_kernel<staged int8>"  # what bench.py's product-only figure times
+    # what bench.py's product-only figures time: the LDS-staged kernel up to four tokens, the kernel
+    # without staging beyond and on the shape with many row blocks
+    assert k_dropin == ("bitlinear_fused_kernel<staged int8>" if (m <= 4 and sh.N // 16 < 432) else "gemv_i2_solo_kernel")
     assert np.array_equal(acc.cpu().numpy(), acc_want), k_acc
     _assert_bits_equal(host_bits(out), want, f"{sh.name} M={m} ({k_dropin})")
     # accumulators and output in ONE call of the export (s and ws given)
@@ -1061,6 +1062,68 @@ def test_solo_kernel_with_several_row_blocks_per_wave(n, k, s_, upw, rpw, coop, 
     finally:
         lib.bitlinear_set_tuning(0, 0, 0, 0)
     _assert_bits_equal(host_bits(out), want, f"rpw={rpw}")
+
+
+@pytest.mark.parametrize("res", [0, 1])
+@pytest.mark.parametrize("m", [1, 3, 4, 8, 13, 16])
+@pytest.mark.parametrize("n,k,s_,upw,rpw", [(2560, 2560, 8, 5, 1), (3840, 2560, 5, 8, 1), (13824, 2560, 8, 5, 2),
+                                            (13824, 2560, 8, 5, 4), (13824, 2560, 0, 0, 0), (2560, 6912, 16, 7, 1),
+                                            (2560, 6912, 0, 0, 0), (7008, 2560, 10, 4, 4), (48, 192, 1, 4, 1),
+                                            (1040, 3200, 10, 5, 2), (80, 8192, 16, 8, 1)])
+def test_product_kernel_without_staging(n, k, s_, upw, rpw, m, res):
+    """gemv_i2_solo_kernel (int8 rows in, activation operands straight from the
+    caller's rows, the code offset removed with a product against ones): forced
+    launch shapes and the library's own choice ((0, 0, 0): many row blocks, or
+    more than four tokens), one to four row blocks per wave with counts the group
+    does not divide, three scale slots, every token count up to 16, with and
+    without the residual epilogue (the two-kernel path of the norm-fused call);
+    int32 accumulators and bf16 outputs bit for bit against the oracle."""
+    import ctypes
+
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=n + k + 7 * m)
+    rng = np.random.default_rng(m + n)
+    s_bits = o.f32_to_bf16_bits((0.5 + 30 * rng.random(m)).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    acc_want, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    pk, ad, sd, wsd = _packed_dev(w), dev_i8(a), dev_bf16(s_bits), dev_bf16(ws_bits)
+    try:
+        if s_:
+            assert lib.bitlinear_set_tuning(10, 1, s_, upw) == 0
+            assert lib.bitlinear_set_tuning(9, 0, rpw, 0) == 0
+        out = bitlinear.bitnet_int8xint2_linear(ad, pk, sd, wsd)
+        name = bitlinear.last_kernel()
+        acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
+        assert bitlinear.last_kernel() == name
+        if res:
+            # the residual epilogue: RMSNorm + quantizer kernel, then this product (path 4 = never one kernel)
+            assert lib.bitlinear_set_tuning(4, 0, 0, 0) == 0
+            if s_:
+                assert lib.bitlinear_set_tuning(10, 1, s_, upw) == 0
+            xin = rng.standard_normal((m, k)).astype(np.float32) * 1.3
+            xb = o.f32_to_bf16_bits(xin)
+            gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+            rb_ = o.f32_to_bf16_bits(rng.standard_normal((m, n)).astype(np.float32))
+            want_n = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, glu=False, residual_bits=rb_)
+            xd, gd, rd = dev_bf16(xb), dev_bf16(gb), dev_bf16(rb_)
+            out_n = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            q_ws = torch.empty(m, k, dtype=torch.int8, device="cuda")
+            s_ws = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+            P = lambda t: ctypes.c_void_p(t.data_ptr())
+            st = lib.bitlinear_norm_forward_bf16(P(xd), P(gd), 1e-5, 0, P(pk), P(wsd), P(rd), P(out_n), P(q_ws), P(s_ws), m, n, k, 0, None)
+            name_n = bitlinear.last_kernel()
+            assert st == 0
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    if s_ or n // 16 >= 432 or m > 4:
+        assert name == "gemv_i2_solo_kernel"
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    _assert_bits_equal(host_bits(out), want, f"product {name}")
+    if res:
+        if s_:
+            assert name_n == "gemv_i2_solo_kernel"
+        _assert_bits_equal(host_bits(out_n), want_n, f"norm + product with residual {name_n}")
 
 
 def test_matrix_pipe_probe_runs_and_reports_its_operations():
