@@ -2703,8 +2703,9 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // at eight, 6.00 -> 5.15 at sixteen) and more than four tokens (3840 x 2560: 3.40 -> 3.34 at eight, 3.83 -> 3.72
     // at sixteen; 2560 x 6912: 4.90 -> 4.71 and 6.11 -> 5.89); elsewhere the staged kernel stays (2.89 against 2.95
     // at 3840 x 2560 and 3.65 against 4.06 at 2560 x 6912, one token)
+    // (from 1024 row blocks on the staged kernel's many small workgroups stay: 20480 x 3200 5.0 us against 5.9)
     const bool prod_solo_wanted = t_tune.prod_solo == 1 || (t_tune.prod_solo == 0 && t_tune.staged == 0 && ((N / 16) >= 432 || M > kDecodeMaxTokens) &&
-                                                            (N / 16) < kStreamMinBlocks);
+                                                            (N / 16) < 1024);
     if (prod_solo_wanted && t_tune.path != 1 && t_tune.path != 2 && M <= 16) {
         const ProdPlan pp = plan_prod_solo(M, N, K);
         bool equal = true;
