@@ -913,9 +913,13 @@ void gemm_i2_prefill_kernel(
         // instructions per wave and row tile, every one of them whole 64-byte runs.
         constexpr int kRowB = NT * 64 + 16;                       // bytes per parked row
         // (with several k-groups, behind the accumulators the other groups left: another wave of this group may still be adding its share)
+        // (where both do not fit, the group's waves meet once more before they park over them: the other groups'
+        // waves have ended by then, and a barrier waits for the surviving waves only)
         constexpr int kRedBytes = (KS - 1) * kPfWaves * MT * NT * 16 * 64 * 4;
-        int8_t* park = lds_all + kRedBytes + wave * (32 * kRowB);
-        static_assert(kRedBytes + kPfWaves * 32 * kRowB <= KS * 2 * MT * 32 * kPfRowBytes, "parked rows must fit the staging buffers");
+        constexpr bool kParkOverRed = kRedBytes + kPfWaves * 32 * kRowB > KS * 2 * MT * 32 * kPfRowBytes;
+        if (kParkOverRed) lds_barrier();
+        int8_t* park = lds_all + (kParkOverRed ? 0 : kRedBytes) + wave * (32 * kRowB);
+        static_assert(kPfWaves * 32 * kRowB <= KS * 2 * MT * 32 * kPfRowBytes, "parked rows must fit the staging buffers");
         constexpr int kPiecesPerRow = NT * 4;                     // 16-byte pieces
         constexpr int kRowsPerStore = 64 / kPiecesPerRow;
         const int pr = lane / kPiecesPerRow, pc = lane % kPiecesPerRow;
@@ -2508,6 +2512,9 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
         if (e == hipSuccess)
             e = hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<2, 1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     2 * 2 * 64 * kPfRowBytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<2, 2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    2 * 2 * 64 * kPfRowBytes);
         return e;
     });
     if (lds_err != hipSuccess) return BITLINEAR_ERR_LAUNCH;
@@ -2517,14 +2524,14 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // many workgroups on the machine and finish a tile's chain of k-chunks earlier (M = 128: 11.4 -> 9.0
     // us at 3840 x 2560, 21.5 -> 16.4 at 2560 x 6912).
     const long long narrow_tiles = (long long)((N + 127) / 128) * ((M + 63) / 64);
-    int tile = ((N >= 8192 && M >= 512) || narrow_tiles >= 900) ? 2 : (narrow_tiles <= kPrefillFewTiles ? 4 : 0);
+    // (beyond the few-tile range the wide tile: against 64 x 128 it measured level or ahead from 330 tiles on --
+    // 2560 x 6912 at M = 1536 31.7 -> 29.2 us, 2560 x 2560 there 14.3 -> 13.6, elsewhere within 2 %)
+    const long long wide_tiles = (long long)((N + 255) / 256) * ((M + 63) / 64);
+    int tile = ((N >= 8192 && M >= 512) || narrow_tiles > kPrefillFewTiles) ? 2 : 4;
     // 64 x 256 tiles run three workgroups per CU (768 at a time), 128 x 256 tiles two (512): with a little more than
     // one full round of the former, one round of the latter finishes earlier (13824 x 2560 at M = 1024: 864 tiles,
     // 46.5 -> 42.3 us; 3840 x 2560 at M = 4096: 960 tiles, 45.1 -> 44.1)
-    if (tile == 2) {
-        const long long wide_tiles = (long long)((N + 255) / 256) * ((M + 63) / 64);
-        if (wide_tiles > 768 && wide_tiles <= 1024) tile = 1;
-    }
+    if (tile == 2 && wide_tiles > 768 && wide_tiles <= 1024) tile = 1;
     if (t_tune.path == 5) tile = t_tune.prefill_big;
     // groups of waves that split a tile's K between them (small tiles only): while the small tiles
     // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
@@ -2538,12 +2545,20 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
         ks = (small_tiles <= kPrefillSplit4Tiles && K >= kPrefillSplit4MinK) ? 4 : 2;
     // between half a tile and about one tile of 64 x 128 per CU: those tiles, with two groups of waves each
     // (2560 x 6912: M = 512 19.1 -> 17.3 us, M = 640 20.5 -> 17.7, M = 768 22.1 -> 20.0; 2560 x 2560: M = 640
-    // 10.2 -> 9.5; 3840 x 2560: M = 384 10.0 -> 9.5; with 240 tiles and K = 2560 10.7 -> 12.1..12.7, not taken)
-    if (t_tune.path != 5 && tile == 4 && narrow_tiles > 128 && narrow_tiles <= (K >= kPrefillSplit4MinK ? 256 : 216)) {
+    // 10.2 -> 9.5; 3840 x 2560: M = 384 10.0 -> 9.5, M = 512 9.7 -> 9.3)
+    if (t_tune.path != 5 && tile == 4 && narrow_tiles > 128 && narrow_tiles <= 256) {
         tile = 0;
         ks = 2;
     }
-    if (t_tune.path == 5 && t_tune.prefill_ks > 0) ks = (tile == 4 || (tile == 0 && t_tune.prefill_ks == 2)) ? t_tune.prefill_ks : 1;
+    // about one 64 x 256 tile per CU: those tiles, two groups of waves each (2560 x 6912: M = 1024 25.9 -> 23.4 us,
+    // M = 1536 29.2 -> 27.9; 13824 x 2560 at M = 256 15.8 -> 14.3; 2560 x 2560 at M = 1280 13.6 -> 13.1; with 320
+    // tiles 42.6 -> 49.4: not taken; at K = 2560 the 32 x 128 tiles stay ahead up to 330 of the 64 x 128 kind)
+    if (t_tune.path != 5 && (tile == 2 || (tile == 4 && K >= kPrefillSplit4MinK)) && wide_tiles > 128 && wide_tiles <= 256 &&
+        narrow_tiles > 256) {
+        tile = 2;
+        ks = 2;
+    }
+    if (t_tune.path == 5 && t_tune.prefill_ks > 0) ks = (tile == 4 || ((tile == 0 || tile == 2) && t_tune.prefill_ks == 2)) ? t_tune.prefill_ks : 1;
     if (K <= kPfChunk * (ks - 1)) ks = 1;  // fewer chunks than groups
     const dim3 block(kPfWaves * 64 * ks, 1, 1);
     // grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
@@ -2586,7 +2601,11 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     } else if (tile == 3) {
         BITLINEAR_LAUNCH_PF(2, 4, 1);
     } else if (tile == 2) {
-        BITLINEAR_LAUNCH_PF(2, 2, 1);
+        if (ks == 2) {
+            BITLINEAR_LAUNCH_PF(2, 2, 2);
+        } else {
+            BITLINEAR_LAUNCH_PF(2, 2, 1);
+        }
     } else if (ks == 2) {
         BITLINEAR_LAUNCH_PF(2, 1, 2);
     } else {

@@ -489,7 +489,7 @@ def test_prefill_gemm_acc_bit_exact(m, n, k, tile):
     assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
 
 
-@pytest.mark.parametrize("tile,ks", [(4, 2), (4, 4), (0, 2)])
+@pytest.mark.parametrize("tile,ks", [(4, 2), (4, 4), (0, 2), (2, 2)])
 @pytest.mark.parametrize("m,n,k", [(17, 48, 192), (64, 128, 64), (100, 272, 320), (128, 2560, 2560), (33, 3840, 2560),
                                    (300, 1040, 3200), (512, 2560, 6912), (70, 256, 768), (40, 512, 1024)])
 def test_prefill_gemm_with_k_split_between_wave_groups(m, n, k, tile, ks):
