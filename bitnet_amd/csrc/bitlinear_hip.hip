@@ -1027,6 +1027,7 @@ void gemm_i2_prefill_kernel(
 constexpr int kQuantThreads = 256;
 constexpr int kQuantMaxThreads = 1024;
 constexpr int kQuantRegVecs = 4;  // 16-byte vectors (8 bf16) kept in registers per thread
+constexpr int kQuantRowsMin = 64;  // from this many rows on the quantizer runs a wave per row
 
 // max |x| over 8 packed bf16 as a bit pattern (|x| as bf16 bits orders like the values): one
 // and + one packed 16-bit max per pair
@@ -1151,6 +1152,47 @@ __global__ __launch_bounds__(kQuantMaxThreads) void quant_absmax_kernel(const ui
             for (int i = 0; i < (nthreads >> 6); ++i) tot += wsum[i];
             rowsum[row] = tot;
         }
+    }
+}
+
+// The same quantizer for many rows (a prompt): one WAVE per row, four rows per workgroup.  The row stays in the
+// wave's registers (V vectors of 8 values per lane), the maximum and the row sum are wave reductions: no LDS, no
+// barrier, all of a row's loads in flight at once, and enough independent rows per CU to keep the memory busy
+// (one workgroup per row leaves a 5 KB row to a chain of load -> reduce -> barrier -> quantize -> store).
+template <int MODE, int V>
+__global__ __launch_bounds__(256) void quant_absmax_rows_kernel(const uint16_t* __restrict__ x, int8_t* __restrict__ q,
+                                                                uint16_t* __restrict__ s, int M, int K,
+                                                                int32_t* __restrict__ rowsum) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;  // uniform per wave; nothing below synchronises across waves
+    const int nvec = K >> 3;
+    const uint4* xr = (const uint4*)(x + (size_t)row * K);
+    uint2* qr = (uint2*)(q + (size_t)row * K);
+    uint4 v[V];
+    uint32_t am = 0;
+#pragma unroll
+    for (int r = 0; r < V; ++r) {
+        const int idx = lane + r * 64;
+        v[r] = idx < nvec ? xr[idx] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < V; ++r) am = absmax_bits8(v[r], am);
+    am = wave_max_u32(am);
+    const float s32 = quant_scale<MODE>(am);
+    if (lane == 0) s[row] = f32_to_bf16_rne(s32);
+    int part = 0;
+    const int ones = 0x01010101;
+#pragma unroll
+    for (int r = 0; r < V; ++r) {
+        const int idx = lane + r * 64;
+        const uint2 qv = quant_vec8<MODE>(v[r], s32);
+        if (idx < nvec) qr[idx] = qv;
+        part = __builtin_amdgcn_sdot4((int)qv.x, ones, __builtin_amdgcn_sdot4((int)qv.y, ones, part, false), false);  // zeros past the row
+    }
+    if (rowsum) {  // uniform
+        const int tot = wave_sum_i32(part);
+        if (lane == 0) rowsum[row] = tot;
     }
 }
 
@@ -1318,6 +1360,54 @@ __global__ __launch_bounds__(kPreThreads) void norm_quant_kernel(const uint16_t*
 #pragma unroll
     for (int r = 0; r < VQ; ++r) {
         const int idx = tid + r * kPreThreads;
+        if (idx < nvec) qr[idx] = mode == 0 ? quant_vec8<0>(xv[r], s32) : quant_vec8<1>(xv[r], s32);
+    }
+}
+
+// The same for many rows (a prompt): one wave per row, four rows per workgroup, the row in the wave's registers,
+// every reduction a wave reduction (no LDS, no barrier).  Same arithmetic, in the same order, as norm_quant_kernel:
+// the fp64 sum of squares is exact, so the order of its additions does not matter.
+template <int PRO, int V>  // V: vectors of 8 values per lane, V * 64 * 8 >= K
+__global__ __launch_bounds__(256) void norm_quant_rows_kernel(const uint16_t* __restrict__ x,
+                                                              const uint16_t* __restrict__ norm_weight, float eps,
+                                                              int8_t* __restrict__ q, uint16_t* __restrict__ s, int M,
+                                                              int K, int mode) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;  // uniform per wave; nothing below synchronises across waves
+    const int nvec = K >> 3;
+    const int xstride = PRO == 2 ? 2 * K : K;
+    const uint16_t* xr = x + (size_t)row * xstride;
+    uint4 xv[V], gv[V], x3v[PRO == 2 ? V : 1];
+#pragma unroll
+    for (int r = 0; r < V; ++r) {
+        const int idx = (lane + r * 64) < nvec ? (lane + r * 64) : (nvec - 1);
+        xv[r] = *(const uint4*)(xr + idx * 8);
+        if (PRO == 2) x3v[r] = *(const uint4*)(xr + K + idx * 8);
+        gv[r] = *(const uint4*)(norm_weight + idx * 8);
+    }
+    double sq = 0.0;
+#pragma unroll
+    for (int r = 0; r < V; ++r) {
+        if (PRO == 2) xv[r] = glu8(xv[r], x3v[r]);
+        if (lane + r * 64 < nvec) sq += sumsq8(xv[r]);
+    }
+    const double total = wave_sum_f64(sq);
+    const float mean = (float)total / (float)K;
+    const float rstd = 1.0f / __builtin_sqrtf(mean + eps);
+    uint32_t am = 0;
+#pragma unroll
+    for (int r = 0; r < V; ++r) {
+        xv[r] = norm8(xv[r], gv[r], rstd);
+        if (lane + r * 64 < nvec) am = absmax_bits8(xv[r], am);
+    }
+    am = wave_max_u32(am);
+    const float s32 = mode == 0 ? quant_scale<0>(am) : quant_scale<1>(am);
+    if (lane == 0) s[row] = f32_to_bf16_rne(s32);
+    uint2* qr = (uint2*)(q + (size_t)row * K);
+#pragma unroll
+    for (int r = 0; r < V; ++r) {
+        const int idx = lane + r * 64;
         if (idx < nvec) qr[idx] = mode == 0 ? quant_vec8<0>(xv[r], s32) : quant_vec8<1>(xv[r], s32);
     }
 }
@@ -3104,6 +3194,23 @@ static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t*
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
     // 256 threads keep rows of up to 8192 elements in registers between the two passes; longer rows
     // get more threads (a second pass that re-reads the row costs a chain of dependent loads)
+    // many rows: a wave per row while a lane holds at most 8 vectors of the row (measured at K = 2560: 4.49 -> 3.66 us
+    // at 64 rows, 5.79 -> 5.39 at 2048, 14.7 -> 12.4 at 8192; at K = 6912 level with the kernel below, which stays)
+    if (M >= kQuantRowsMin && K <= 8 * 64 * 8) {
+        const int per_lane = (K / 8 + 63) / 64;
+        const dim3 grid((M + 3) / 4, 1, 1), block(256, 1, 1);
+#define BITLINEAR_LAUNCH_QR(MODE_, V_) \
+    hipLaunchKernelGGL((quant_absmax_rows_kernel<MODE_, V_>), grid, block, 0, (hipStream_t)stream, x, q, s, M, K, rowsum)
+#define BITLINEAR_LAUNCH_QR_V(V_)          \
+    if (mode == 0) BITLINEAR_LAUNCH_QR(0, V_); \
+    else BITLINEAR_LAUNCH_QR(1, V_)
+        if (per_lane <= 2) { BITLINEAR_LAUNCH_QR_V(2); }
+        else if (per_lane <= 5) { BITLINEAR_LAUNCH_QR_V(5); }
+        else { BITLINEAR_LAUNCH_QR_V(8); }
+#undef BITLINEAR_LAUNCH_QR_V
+#undef BITLINEAR_LAUNCH_QR
+        return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
+    }
     int threads = kQuantThreads;
     while (threads < kQuantMaxThreads && K > threads * kQuantRegVecs * 8) threads *= 2;
     const dim3 grid(M, 1, 1), block(threads, 1, 1);
@@ -3216,6 +3323,22 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, 
     // larger blocks: gate / norm / quantizer once per token row, then the product with the residual epilogue
     if (!q_ws || !s_ws) return set_status(pl.ok ? BITLINEAR_ERR_NULL : BITLINEAR_ERR_SHAPE);
     if (K > kPreThreads * kPreVecs * 8) return set_status(BITLINEAR_ERR_SHAPE);
+    // very many rows, no gate, short rows: a wave per row (norm + product at K = 2560: 32.2 -> 30.1 us at 2048 rows,
+    // 53.6 -> 48.7 at 4096; below 1024 rows 0.2-0.9 us behind, with the gate at K = 6912 4-7 us behind: not taken)
+    if (M >= 1024 && !glu && K <= 8 * 64 * 8) {
+        const int per_lane = (K / 8 + 63) / 64;
+        const dim3 rgrid((M + 3) / 4, 1, 1), rblock(256, 1, 1);
+#define BITLINEAR_LAUNCH_NR(P, V) \
+    hipLaunchKernelGGL((norm_quant_rows_kernel<P, V>), rgrid, rblock, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, M, K, mode)
+#define BITLINEAR_LAUNCH_NR_V(V) BITLINEAR_LAUNCH_NR(1, V)
+        if (per_lane <= 2) { BITLINEAR_LAUNCH_NR_V(2); }
+        else if (per_lane <= 5) { BITLINEAR_LAUNCH_NR_V(5); }
+        else { BITLINEAR_LAUNCH_NR_V(8); }
+#undef BITLINEAR_LAUNCH_NR_V
+#undef BITLINEAR_LAUNCH_NR
+        if (hipGetLastError() != hipSuccess) return set_status(BITLINEAR_ERR_LAUNCH);
+        return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream, residual));
+    }
     const dim3 grid(M, 1, 1), block(kPreThreads, 1, 1);
     const int per_thread = (K / 8 + kPreThreads - 1) / kPreThreads;
 #define BITLINEAR_LAUNCH_PRE(P, V) \

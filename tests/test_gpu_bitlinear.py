@@ -761,7 +761,8 @@ def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
 
 @pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
 @pytest.mark.parametrize("m,n,k,glu", [(40, 2560, 2560, 0), (130, 3840, 2560, 0), (300, 2560, 6912, 1), (77, 48, 192, 1),
-                                       (513, 1040, 640, 0)])
+                                       (513, 1040, 640, 0), (1030, 64, 2560, 0), (1025, 272, 640, 0), (1024, 48, 4096, 0),
+                                       (1026, 32, 6912, 1)])  # from 1024 rows on without the gate: a wave per row
 def test_norm_forward_with_residual_beyond_decode_sizes(m, n, k, glu, tile):
     """Prompt-sized blocks: gate / norm / quantizer kernel, then the product with
     the residual added in its epilogue -- through the library's own choice of
