@@ -371,6 +371,12 @@ def _random_shape_cases(count=36, seed=20240611):
         if n * k > 9_000_000:
             continue
         cases.append((n, k, m))
+    # the row-block counts at which the library changes kernels or launch shapes (432, 864, 1024, 2048 and
+    # their neighbours), at token counts on both sides of its limits, short and decode-sized rows
+    for blocks in (431, 432, 433, 863, 864, 865, 1023, 1024, 2047, 2048):
+        for k, m in ((192, 1), (320, 5), (2560, 1), (2560, 4), (2560, 16)):
+            if blocks * 16 * k <= 45_000_000 and (k < 2560 or blocks in (432, 865, 1023, 2048)):
+                cases.append((blocks * 16, k, m))
     return cases
 
 
