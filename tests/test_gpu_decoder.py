@@ -699,3 +699,36 @@ def test_full_size_decode_step_substeps_against_the_torch_glue(model_2b, B):
     top2 = torch.topk(logits_f, 2, dim=-1).values
     clear = (top2[:, 0] - top2[:, 1]) > 2e-2  # rows whose best logit is not a near tie
     assert torch.equal(tok_lib[clear], torch.argmax(logits_f, dim=-1)[clear])
+
+
+def test_decoder_loaded_from_a_gguf_file_gives_the_same_logits(tmp_path):
+    """A decoder written out as a GGUF file with I2_S projections (the CPU stack's format) and read back
+    through the transcoder computes, prompt and decode step, what the original computes: the packed bytes,
+    the scale slots and the norms survive the trip bit for bit, so the logits are equal."""
+    from bitnet_amd import gguf
+
+    model = _build(SMALL, seed=4)
+    state = {k: v.detach().cpu() for k, v in model.state_dict().items()}
+    path = str(tmp_path / "small.gguf")
+    gguf.int2_state_to_gguf(state, SMALL, path, embed_dtype=torch.bfloat16)
+    with gguf.GGUFReader(path) as r:
+        args = gguf.model_args_from_gguf(r)
+        back = gguf.gguf_to_int2_state(r)
+    assert args == SMALL
+    for k, v in state.items():
+        assert torch.equal(back[k], v), k
+    clone = _build(args, seed=9)  # other weights, then overwritten by the file's
+    clone.load_state_dict(back, strict=True)
+    B, P, S = 2, 20, 32
+    dev = torch.device("cuda")
+    cos, sin = decoder.rope_tables(SMALL.dim // SMALL.n_heads, S, SMALL.rope_theta, dev)
+    g = torch.Generator(device="cuda").manual_seed(8)
+    prompt = torch.randint(0, SMALL.vocab_size, (B, P), generator=g, device=dev)
+    pos = torch.arange(P, device=dev)[None].expand(B, P).contiguous()
+    c1, c2 = model.make_cache(B, S, dev), clone.make_cache(B, S, dev)
+    l1 = model.forward_tokens(prompt, pos, c1, cos, sin)
+    l2 = clone.forward_tokens(prompt, pos, c2, cos, sin)
+    assert torch.equal(l1, l2) and bool(torch.isfinite(l1).all())
+    tok = torch.argmax(l1[:, -1], dim=-1).view(B, 1)
+    p1 = torch.full((B, 1), P, device=dev)
+    assert torch.equal(model.forward_tokens(tok, p1, c1, cos, sin), clone.forward_tokens(tok, p1, c2, cos, sin))
