@@ -444,6 +444,19 @@ def random_init_(model: Transformer, seed: int = 0) -> Transformer:
     return model
 
 
+def top_p_sample(probs: torch.Tensor, p: float, generator: Optional[torch.Generator] = None) -> torch.Tensor:
+    """Nucleus sampling, one draw per row of probs [B, V] -> int64 [B, 1]: a token
+    stays in the draw while the probability mass of the tokens more likely than
+    it is at most p (so the most likely token always stays, and the kept set is
+    the shortest prefix of the sorted distribution whose mass exceeds p); the
+    kept probabilities are renormalised by the draw itself (gpu/sample_utils.py:9-33)."""
+    ranked, order = torch.sort(probs, dim=-1, descending=True)
+    mass_before = torch.cumsum(ranked, dim=-1) - ranked
+    kept = torch.where(mass_before > p, torch.zeros_like(ranked), ranked)
+    pick = torch.multinomial(kept, num_samples=1, generator=generator)
+    return torch.gather(order, -1, pick)
+
+
 class Generator:
     """Greedy generation: prefill of the whole prompt in one call, then one
     graph replay per generated token (gpu/generate.py:216-288)."""
@@ -521,18 +534,30 @@ class Generator:
         logits = self.model.forward_tokens(prompt, pos, self.cache, self.cos, self.sin)
         return torch.argmax(logits[:, -1, :], dim=-1)
 
+    def _set_positions(self, start_pos) -> None:
+        if isinstance(start_pos, torch.Tensor):
+            self.pos.copy_(start_pos.to(self.pos.device, torch.int64).view(-1, 1))
+        else:
+            self.pos.fill_(start_pos)
+
     @torch.no_grad()
-    def decode(self, first: torch.Tensor, start_pos: int, steps: int) -> torch.Tensor:
-        """Feeds `first` at position start_pos and generates `steps` further
-        tokens greedily.  Returns [steps, B]."""
+    def decode(self, first: torch.Tensor, start_pos, steps: int, eos_id: Optional[int] = None) -> torch.Tensor:
+        """Feeds `first` at position start_pos (an int, or one position per
+        sequence: int64 [B], ragged prompts) and generates up to `steps` further
+        tokens greedily.  With eos_id the loop ends after the first step in which
+        any sequence produced that token, as the reference's loop does
+        (gpu/generate.py:283-284; one device-to-host copy per step).  Returns
+        [steps taken, B]."""
         if steps > self.history.shape[0]:
             raise ValueError("more steps than the generator was sized for")
-        if start_pos < 0 or start_pos + steps > self.max_seq:
-            raise ValueError(
-                f"decode: positions {start_pos}..{start_pos + steps - 1} do not fit a cache of {self.max_seq} rows"
-            )
+        lo = int(start_pos.min()) if isinstance(start_pos, torch.Tensor) else start_pos
+        hi = int(start_pos.max()) if isinstance(start_pos, torch.Tensor) else start_pos
+        if isinstance(start_pos, torch.Tensor) and start_pos.numel() != self.batch:
+            raise ValueError(f"decode: {start_pos.numel()} start positions for a batch of {self.batch}")
+        if lo < 0 or hi + steps > self.max_seq:
+            raise ValueError(f"decode: positions {lo}..{hi + steps - 1} do not fit a cache of {self.max_seq} rows")
         self.tok.copy_(first.view(-1, 1))
-        self.pos.fill_(start_pos)
+        self._set_positions(start_pos)
         if self.use_graph and self.graph is None:
             # capture with the real inputs in place; the captured step is re-run below
             saved_k = [ck.clone() for ck, _ in self.cache]
@@ -542,14 +567,109 @@ class Generator:
                 ck.copy_(sk)
                 cv.copy_(sv)
             self.tok.copy_(first.view(-1, 1))
-            self.pos.fill_(start_pos)
+            self._set_positions(start_pos)
         self.step_idx.zero_()
+        taken = 0
         for i in range(steps):
             if self.use_graph:
                 self.graph.replay()
             else:
                 self._step()
-        out = self.history[:steps].clone()
+            taken = i + 1
+            if eos_id is not None and bool((self.next_tok == eos_id).any()):
+                break
+        out = self.history[:taken].clone()
         if self.fused:
             self.attn_ws.check()  # one small copy to the host per decode() call
         return out
+
+    @torch.no_grad()
+    def _prefill_ragged(self, prompts, pad_id: int, want_logits: bool):
+        """Prompts of different lengths, padded on the right to the longest (attention is causal: a pad never
+        reaches a real token, and the cache rows the pads leave behind are overwritten before a decode step
+        reads them).  Returns (first greedy token [B], logits fp32 [B, V] or None, lengths int64 [B])."""
+        dev = self.tok.device
+        lens = torch.tensor([len(q) for q in prompts], dtype=torch.int64, device=dev)
+        P = int(lens.max())
+        prompt = torch.full((self.batch, P), pad_id, dtype=torch.int64, device=dev)
+        for b, q in enumerate(prompts):
+            prompt[b, : len(q)] = torch.tensor(q, dtype=torch.int64, device=dev)
+        rows = torch.arange(self.batch, device=dev)
+        V = self.model.args.vocab_size
+        if self.lm_head:
+            h = self.model.prefill_hidden_fused(prompt, self.cache, self.cos, self.sin)
+            logits = torch.empty(self.batch, V, dtype=torch.float32, device=dev) if want_logits else None
+            tok = lm_head_greedy(h[rows, lens - 1].contiguous(), self.model.norm, self.model.output.weight, self.lm_ws,
+                                 logits_out=logits)
+            return tok, logits, lens
+        pos = torch.arange(P, device=dev)[None, :].expand(self.batch, P).contiguous()
+        logits = self.model.forward_tokens(prompt, pos, self.cache, self.cos, self.sin)[rows, lens - 1]
+        return torch.argmax(logits, dim=-1), logits, lens
+
+    @torch.no_grad()
+    def generate_all(self, prompts, gen_length: int, use_sampling: bool = False, temperature: float = 0.7,
+                     top_p: float = 0.95, eos_id: Optional[int] = None, pad_id: int = 1,
+                     rng: Optional[torch.Generator] = None):
+        """FastGen.generate_all of the reference (gpu/generate.py:217-304) on token
+        ids: `prompts` is one list of ids per sequence of the batch (lengths may
+        differ; padded with pad_id, the reference's 1); the whole batch is
+        prefilled in one pass, then one token per sequence and step is generated,
+        greedily or -- use_sampling -- from softmax(logits / temperature) cut to
+        the top_p nucleus (the reference's 0.7 / 0.95), until gen_length tokens
+        are out or, with eos_id, until any sequence has produced it.  Every
+        answer is cut behind its first eos_id.  Greedy steps replay the captured
+        graph of the whole step; a sampled step runs the same kernels and draws
+        with torch between them (`rng` makes the draws reproducible)."""
+        if len(prompts) != self.batch:
+            raise ValueError(f"generate_all: {len(prompts)} prompts for a generator of batch {self.batch}")
+        if any(len(q) < 1 for q in prompts):
+            raise ValueError("generate_all: empty prompt")
+        longest = max(len(q) for q in prompts)
+        if gen_length < 1 or longest + gen_length > self.max_seq or gen_length > self.history.shape[0]:
+            raise ValueError(f"generate_all: prompt of {longest} + {gen_length} tokens does not fit a cache of {self.max_seq} rows")
+        vocab = self.model.args.vocab_size
+        if any(t < 0 or t >= vocab for q in prompts for t in q):
+            raise ValueError("generate_all: token id outside the vocabulary")
+
+        def draw(logits):
+            probs = torch.softmax(logits / temperature, dim=-1)
+            return top_p_sample(probs, top_p, rng).view(-1)
+
+        first, logits, lens = self._prefill_ragged(prompts, pad_id, use_sampling)
+        if use_sampling:
+            first = draw(logits)
+        out = [first.view(1, -1)]
+        stop = eos_id is not None and bool((first == eos_id).any())
+        if gen_length > 1 and not stop:
+            if not use_sampling:
+                out.append(self.decode(first, lens, gen_length - 1, eos_id=eos_id))
+            else:
+                if logits is None or not self.lm_head:
+                    logits = torch.empty(self.batch, vocab, dtype=torch.float32, device=self.tok.device)
+                self.tok.copy_(first.view(-1, 1))
+                self._set_positions(lens)
+                for _ in range(gen_length - 1):
+                    if self.lm_head:
+                        h = self.model.decode_hidden_fused(self.tok, self.pos, self.cache, self.cos, self.sin, self.attn_ws)
+                        lm_head_greedy(h, self.model.norm, self.model.output.weight, self.lm_ws, logits_out=logits)
+                        step_logits = logits
+                    elif self.fused:
+                        step_logits = self.model.forward_decode_fused(self.tok, self.pos, self.cache, self.cos, self.sin,
+                                                                      self.attn_ws)[:, -1]
+                    else:
+                        step_logits = self.model.forward_tokens(self.tok, self.pos, self.cache, self.cos, self.sin)[:, -1]
+                    nxt = draw(step_logits)
+                    out.append(nxt.view(1, -1))
+                    self.tok.copy_(nxt.view(-1, 1))
+                    self.pos.add_(1)
+                    if eos_id is not None and bool((nxt == eos_id).any()):
+                        break
+                if self.fused:
+                    self.attn_ws.check()
+        tokens = torch.cat(out, dim=0).t().tolist()  # [B][steps]
+        answers = []
+        for ans in tokens:
+            if eos_id is not None and eos_id in ans:
+                ans = ans[: ans.index(eos_id) + 1]
+            answers.append(ans)
+        return answers

@@ -732,3 +732,62 @@ def test_decoder_loaded_from_a_gguf_file_gives_the_same_logits(tmp_path):
     tok = torch.argmax(l1[:, -1], dim=-1).view(B, 1)
     p1 = torch.full((B, 1), P, device=dev)
     assert torch.equal(model.forward_tokens(tok, p1, c1, cos, sin), clone.forward_tokens(tok, p1, c2, cos, sin))
+
+
+def test_generate_all_with_ragged_prompts_equals_one_sequence_at_a_time():
+    """FastGen.generate_all semantics (gpu/generate.py:217-304): prompts of different lengths in one batch,
+    padded on the right.  Every per-token operation is independent of the other rows and the attention of a
+    sequence only sees its own cache rows up to its own position, so each answer equals what the same prompt
+    generates alone -- on the fused path (graph replays) and on the torch-glue path."""
+    model = _build(SMALL, seed=5)
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(2, SMALL.vocab_size, (n,), generator=g).tolist() for n in (19, 7, 33)]
+    gen = 12
+    for fused in (True, False):
+        batch = decoder.Generator(model, batch=3, max_seq=64, use_graph=fused, fused=fused)
+        answers = batch.generate_all(prompts, gen)
+        assert [len(a) for a in answers] == [gen] * 3
+        for b, q in enumerate(prompts):
+            alone = decoder.Generator(model, batch=1, max_seq=64, use_graph=fused, fused=fused)
+            assert alone.generate_all([q], gen) == [answers[b]], (fused, b)
+    with pytest.raises(ValueError):
+        batch.generate_all(prompts[:2], gen)
+    with pytest.raises(ValueError):
+        batch.generate_all(prompts, 64)
+    with pytest.raises(ValueError):
+        batch.generate_all([[SMALL.vocab_size], [1], [1]], 4)
+
+
+def test_generate_all_stops_at_the_end_token_and_trims_the_answers():
+    model = _build(SMALL, seed=6)
+    g = torch.Generator().manual_seed(4)
+    prompts = [torch.randint(2, SMALL.vocab_size, (n,), generator=g).tolist() for n in (9, 14)]
+    gen = decoder.Generator(model, batch=2, max_seq=48)
+    full = gen.generate_all(prompts, 16)
+    # take a token that sequence 1 produces at step 5 as the end token
+    eos = full[1][5]
+    first_hit = min(min(a.index(eos) for a in full if eos in a), 15)
+    cut = gen.generate_all(prompts, 16, eos_id=eos)
+    for a, f in zip(cut, full):
+        want = f[: first_hit + 1]           # the loop ends after the first step in which any sequence hit it
+        if eos in want:
+            want = want[: want.index(eos) + 1]
+        assert a == want
+    assert cut[1][-1] == eos or eos in cut[0]
+
+
+def test_generate_all_sampling_is_reproducible_and_greedy_for_a_tiny_nucleus():
+    model = _build(SMALL, seed=7)
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(2, SMALL.vocab_size, (n,), generator=g).tolist() for n in (11, 6)]
+    gen = decoder.Generator(model, batch=2, max_seq=40)
+    a = gen.generate_all(prompts, 10, use_sampling=True, rng=torch.Generator(device="cuda").manual_seed(11))
+    b = gen.generate_all(prompts, 10, use_sampling=True, rng=torch.Generator(device="cuda").manual_seed(11))
+    c = gen.generate_all(prompts, 10, use_sampling=True, rng=torch.Generator(device="cuda").manual_seed(12))
+    assert a == b and all(0 <= t < SMALL.vocab_size for ans in a for t in ans)
+    assert a != c  # 20 draws at temperature 0.7 from a 512-token vocabulary
+    # a nucleus that only holds the most likely token: the greedy answer (the draw is from the bf16-rounded
+    # logits the LM head returns, the greedy token from the same values)
+    greedy = gen.generate_all(prompts, 10)
+    tiny = gen.generate_all(prompts, 10, use_sampling=True, top_p=1e-9, rng=torch.Generator(device="cuda").manual_seed(1))
+    assert tiny == greedy
