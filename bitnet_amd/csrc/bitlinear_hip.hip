@@ -1027,7 +1027,7 @@ void gemm_i2_prefill_kernel(
 constexpr int kQuantThreads = 256;
 constexpr int kQuantMaxThreads = 1024;
 constexpr int kQuantRegVecs = 4;  // 16-byte vectors (8 bf16) kept in registers per thread
-constexpr int kQuantRowsMin = 64;  // from this many rows on the quantizer runs a wave per row
+constexpr int kQuantRowsMin = 2;   // from this many rows on the quantizer runs a wave per row (rows of up to 4096 values)
 
 // max |x| over 8 packed bf16 as a bit pattern (|x| as bf16 bits orders like the values): one
 // and + one packed 16-bit max per pair
@@ -3194,8 +3194,9 @@ static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t*
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
     // 256 threads keep rows of up to 8192 elements in registers between the two passes; longer rows
     // get more threads (a second pass that re-reads the row costs a chain of dependent loads)
-    // many rows: a wave per row while a lane holds at most 8 vectors of the row (measured at K = 2560: 4.49 -> 3.66 us
-    // at 64 rows, 5.79 -> 5.39 at 2048, 14.7 -> 12.4 at 8192; at K = 6912 level with the kernel below, which stays)
+    // two rows or more: a wave per row while a lane holds at most 8 vectors of the row (measured at K = 2560: 2.41 -> 2.18 us
+    // at 8 rows, 2.45 -> 2.26 at 16, 4.49 -> 3.66 at 64, 5.79 -> 5.39 at 2048, 14.7 -> 12.4 at 8192; longer rows keep the
+    // kernel below)
     if (M >= kQuantRowsMin && K <= 8 * 64 * 8) {
         const int per_lane = (K / 8 + 63) / 64;
         const dim3 grid((M + 3) / 4, 1, 1), block(256, 1, 1);
