@@ -92,8 +92,17 @@ class GGUFReader:
         self._f = open(path, "rb")
         size = os.fstat(self._f.fileno()).st_size
         if size < 24:
+            self._f.close()
             raise GGUFError(f"{path}: {size} bytes is too short for a GGUF header")
         self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ)
+        try:
+            self._parse(size)
+        except Exception:
+            self.close()  # a refused file leaves no mapping or descriptor behind
+            raise
+
+    def _parse(self, size: int) -> None:
+        path, i2s_type = self.path, self.i2s_type
         self._pos = 0
         magic, self.version = self._unpack("<II")
         if magic != GGUF_MAGIC:
@@ -138,7 +147,10 @@ class GGUFReader:
 
     # -- parsing helpers ----------------------------------------------------
     def _unpack(self, fmt: str):
-        n = struct.calcsize(fmt)
+        try:
+            n = struct.calcsize(fmt)
+        except struct.error:  # a count field far beyond any file
+            raise GGUFError(f"{self.path}: field count at byte {self._pos} is not credible") from None
         if self._pos + n > len(self._mm):
             raise GGUFError(f"{self.path}: truncated at byte {self._pos}")
         out = struct.unpack_from(fmt, self._mm, self._pos)

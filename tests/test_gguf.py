@@ -210,3 +210,23 @@ def test_rotary_row_orders_are_inverse():
     assert torch.equal(gguf.rope_rows_interleaved_to_hf(rope_rows_hf_to_interleaved(w, 4), 4), w)
     with pytest.raises(ValueError):
         gguf.rope_rows_interleaved_to_hf(w[:10], 4)
+
+
+def test_absurd_counts_are_refused_not_allocated(tmp_path):
+    """A count field far beyond the file's size ends in GGUFError before anything is sized by it."""
+    p = str(tmp_path / "huge.gguf")
+    head = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + _s("k") + struct.pack("<IIQ", 9, 4, 2 ** 62)
+    with open(p, "wb") as f:
+        f.write(head + b"\0" * 64)
+    with pytest.raises(gguf.GGUFError):
+        gguf.GGUFReader(p)
+    head = struct.pack("<IIQQ", 0x46554747, 3, 2 ** 40, 0)
+    with open(p, "wb") as f:
+        f.write(head + b"\0" * 64)
+    with pytest.raises(gguf.GGUFError):
+        gguf.GGUFReader(p)
+    head = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + struct.pack("<Q", 2 ** 50) + b"abc"
+    with open(p, "wb") as f:
+        f.write(head + b"\0" * 64)
+    with pytest.raises(gguf.GGUFError):
+        gguf.GGUFReader(p)
