@@ -89,7 +89,8 @@ def test_writer_output_reads_back(tmp_path):
         c2, s2, n, k = r.i2s("b")
         assert torch.equal(c2, codes) and s2 == 0.5 and (n, k) == (32, 256)
     # the same bytes, parsed by hand: magic, version, counts, first key
-    raw = open(path, "rb").read()
+    with open(path, "rb") as f:
+        raw = f.read()
     assert struct.unpack_from("<IIQQ", raw) == (0x46554747, 3, 4, len(kv))
     assert raw[24 : 24 + 8 + 20] == _s("general.architecture")
 
@@ -97,7 +98,8 @@ def test_writer_output_reads_back(tmp_path):
 def test_malformed_files_are_refused(tmp_path):
     path = str(tmp_path / "bad.gguf")
     _hand_made_file(path)
-    good = open(path, "rb").read()
+    with open(path, "rb") as f:
+        good = f.read()
     cases = {"magic": b"GGUX" + good[4:], "version": good[:4] + struct.pack("<I", 1) + good[8:], "short": good[:10],
              "truncated directory": good[:120], "truncated data": good[:-40]}
     for what, data in cases.items():
