@@ -1253,3 +1253,16 @@ def test_runs_on_a_side_stream_and_in_a_graph():
         g.replay()
         torch.cuda.synchronize()
         _assert_bits_equal(host_bits(out), want, "graph replay")
+
+
+def test_kernel_test_harness_reports_the_reference_lines():
+    """bitnet_amd.kernel_test mirrors gpu/test.py:31-86: per shape a known-answer line and a timing line."""
+    from bitnet_amd import kernel_test
+
+    lines = []
+    res = kernel_test.check_and_time(shapes=kernel_test.REFERENCE_SHAPES[:2] + ((4800, 3200),), iters=5, out=lines.append)
+    assert [r["equal"] for r in res] == [True, True, True]
+    assert lines[0] == "custom == np True" and lines[1].startswith("Shape(2560, 2560), W2A8: ")
+    assert "torch BF16: " in lines[1] and len(lines) == 6
+    assert all(r["w2a8_graph_us"] > 0 and r["bf16_graph_us"] > 0 for r in res)
+    assert len(kernel_test.REFERENCE_SHAPES) == 8
