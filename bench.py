@@ -525,9 +525,43 @@ def end_to_end_decode(batches=(1, 8), prompt_len=512, gen_len=128):
             "distinct_tokens_generated": int(torch.unique(toks).numel()),
         }
         del gen
+    out["generation_latency_ms"] = generation_latency(model, dev)
     del model
     torch.cuda.empty_cache()
     return out
+
+
+def generation_latency(model, dev, inputs=(64, 256, 512), outputs=(16, 32, 64)):
+    """The reference's published end-to-end table (gpu/README.md:93-105: input length x output length,
+    one sequence): wall-clock milliseconds from the prompt's token ids to the last generated token --
+    prefill of the whole prompt, then output - 1 greedy decode steps replayed from the captured graph
+    (the first token comes out of the prefill).  Same random-init 2B decoder as above; the graph is
+    captured and every kernel has run once before anything is timed."""
+    import torch
+
+    from bitnet_amd import decoder
+
+    table = {}
+    gen = decoder.Generator(model, 1, max(inputs) + max(outputs) + 1, use_graph=True)
+    g = torch.Generator(device=dev).manual_seed(4321)
+    warm = torch.randint(0, model.args.vocab_size, (1, 8), generator=g, device=dev)
+    gen.decode(gen.prefill(warm), 8, 2)  # captures the decode graph
+    for P in inputs:
+        prompt = torch.randint(0, model.args.vocab_size, (1, P), generator=g, device=dev)
+        gen.prefill(prompt)  # first use of the prompt-size kernels at this length
+        for G in outputs:
+            best = None
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                first = gen.prefill(prompt)
+                gen.decode(first, P, G - 1)
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) * 1e3
+                best = dt if best is None else min(best, dt)
+            table[f"in{P}_out{G}"] = round(best, 3)
+    del gen
+    return {"batch": 1, "how": "prefill + (output - 1) graph-replayed greedy steps, wall clock, best of 3", **table}
 
 
 def main():
