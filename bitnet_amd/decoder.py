@@ -490,6 +490,11 @@ class Generator:
         # generated tokens of a decode() call, written from inside the step so that a graph replay is the whole step
         self.history = torch.zeros(max_seq, batch, dtype=torch.int64, device=dev)
         self.step_idx = torch.zeros(1, dtype=torch.int64, device=dev)
+        # captured prompt passes, one per (prompt length, logits wanted): a prompt is some three hundred launches,
+        # and issued one by one from Python they cost more host time than the GPU needs for a short prompt
+        # (the reference captures its prompt pass too, gpu/generate.py:102-157)
+        self._pf_graphs: dict = {}
+        self._rows = torch.arange(batch, device=dev)
 
     def _step(self):
         """One decode step including its bookkeeping: next token -> history and
@@ -522,14 +527,56 @@ class Generator:
         with torch.cuda.graph(self.graph):
             self._step()
 
+    kMaxPrefillGraphs = 12  # distinct (prompt length, logits) pairs kept captured; further ones run launch by launch
+
+    def _prefill_fused(self, prompt, lens, tok_out, logits):
+        """The prompt through the library's kernels; only each sequence's last real token goes through the LM head."""
+        h = self.model.prefill_hidden_fused(prompt, self.cache, self.cos, self.sin)
+        last = h[self._rows, lens - 1].contiguous()
+        return lm_head_greedy(last, self.model.norm, self.model.output.weight, self.lm_ws, token_out=tok_out, logits_out=logits)
+
+    def _prefill_replay(self, prompt: torch.Tensor, lens: Optional[torch.Tensor], want_logits: bool):
+        """prompt [B, P] (padded) through the captured pass for this length: (first token [B], logits or None)."""
+        B, P = prompt.shape
+        key = (P, want_logits)
+        entry = self._pf_graphs.get(key)
+        if entry is None:
+            dev = self.tok.device
+            bufs = {"prompt": torch.zeros(B, P, dtype=torch.int64, device=dev),
+                    "lens": torch.full((B,), P, dtype=torch.int64, device=dev),
+                    "tok": torch.zeros(B, dtype=torch.int64, device=dev),
+                    "logits": torch.empty(B, self.model.args.vocab_size, dtype=torch.float32, device=dev) if want_logits else None}
+            bufs["prompt"].copy_(prompt)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self._prefill_fused(bufs["prompt"], bufs["lens"], bufs["tok"], bufs["logits"])  # warm-up outside the graph
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self._prefill_fused(bufs["prompt"], bufs["lens"], bufs["tok"], bufs["logits"])
+            entry = self._pf_graphs[key] = (graph, bufs)
+        graph, bufs = entry
+        bufs["prompt"].copy_(prompt)
+        if lens is None:
+            bufs["lens"].fill_(P)
+        else:
+            bufs["lens"].copy_(lens)
+        graph.replay()
+        return bufs["tok"].clone(), (bufs["logits"] if want_logits else None)
+
     @torch.no_grad()
     def prefill(self, prompt: torch.Tensor) -> torch.Tensor:
         """prompt [B, P] int64 -> first generated token [B]."""
         B, P = prompt.shape
         if self.lm_head:
-            # the prompt through the library's kernels; only the last token's row goes through the LM head
+            if self.use_graph and B == self.batch and ((P, False) in self._pf_graphs or len(self._pf_graphs) < self.kMaxPrefillGraphs):
+                return self._prefill_replay(prompt, None, False)[0]
+            lens = torch.full((B,), P, dtype=torch.int64, device=prompt.device)
+            rows = self._rows if B == self.batch else torch.arange(B, device=prompt.device)
             h = self.model.prefill_hidden_fused(prompt, self.cache, self.cos, self.sin)
-            return lm_head_greedy(h[:, -1].contiguous(), self.model.norm, self.model.output.weight, self.lm_ws)
+            return lm_head_greedy(h[rows, lens - 1].contiguous(), self.model.norm, self.model.output.weight, self.lm_ws)
         pos = torch.arange(P, device=prompt.device)[None, :].expand(B, P).contiguous()
         logits = self.model.forward_tokens(prompt, pos, self.cache, self.cos, self.sin)
         return torch.argmax(logits[:, -1, :], dim=-1)
@@ -594,13 +641,14 @@ class Generator:
         prompt = torch.full((self.batch, P), pad_id, dtype=torch.int64, device=dev)
         for b, q in enumerate(prompts):
             prompt[b, : len(q)] = torch.tensor(q, dtype=torch.int64, device=dev)
-        rows = torch.arange(self.batch, device=dev)
+        rows = self._rows
         V = self.model.args.vocab_size
         if self.lm_head:
-            h = self.model.prefill_hidden_fused(prompt, self.cache, self.cos, self.sin)
+            if self.use_graph and ((P, want_logits) in self._pf_graphs or len(self._pf_graphs) < self.kMaxPrefillGraphs):
+                tok, logits = self._prefill_replay(prompt, lens, want_logits)
+                return tok, logits, lens
             logits = torch.empty(self.batch, V, dtype=torch.float32, device=dev) if want_logits else None
-            tok = lm_head_greedy(h[rows, lens - 1].contiguous(), self.model.norm, self.model.output.weight, self.lm_ws,
-                                 logits_out=logits)
+            tok = self._prefill_fused(prompt, lens, None, logits)
             return tok, logits, lens
         pos = torch.arange(P, device=dev)[None, :].expand(self.batch, P).contiguous()
         logits = self.model.forward_tokens(prompt, pos, self.cache, self.cos, self.sin)[rows, lens - 1]

@@ -739,9 +739,10 @@ def test_generate_all_with_ragged_prompts_equals_one_sequence_at_a_time():
     padded on the right.  Every per-token operation is independent of the other rows and the attention of a
     sequence only sees its own cache rows up to its own position, so each answer equals what the same prompt
     generates alone -- on the fused path (graph replays) and on the torch-glue path."""
-    model = _build(SMALL, seed=5)
+    model = _build(BIG_HEADS, seed=5)
+    assert decoder.Generator(model, batch=3, max_seq=64).lm_head  # head_dim 128: the folded calls and the library's LM head
     g = torch.Generator().manual_seed(3)
-    prompts = [torch.randint(2, SMALL.vocab_size, (n,), generator=g).tolist() for n in (19, 7, 33)]
+    prompts = [torch.randint(2, BIG_HEADS.vocab_size, (n,), generator=g).tolist() for n in (19, 7, 33)]
     gen = 12
     for fused in (True, False):
         batch = decoder.Generator(model, batch=3, max_seq=64, use_graph=fused, fused=fused)
@@ -755,13 +756,13 @@ def test_generate_all_with_ragged_prompts_equals_one_sequence_at_a_time():
     with pytest.raises(ValueError):
         batch.generate_all(prompts, 64)
     with pytest.raises(ValueError):
-        batch.generate_all([[SMALL.vocab_size], [1], [1]], 4)
+        batch.generate_all([[BIG_HEADS.vocab_size], [1], [1]], 4)
 
 
 def test_generate_all_stops_at_the_end_token_and_trims_the_answers():
-    model = _build(SMALL, seed=6)
+    model = _build(BIG_HEADS, seed=6)
     g = torch.Generator().manual_seed(4)
-    prompts = [torch.randint(2, SMALL.vocab_size, (n,), generator=g).tolist() for n in (9, 14)]
+    prompts = [torch.randint(2, BIG_HEADS.vocab_size, (n,), generator=g).tolist() for n in (9, 14)]
     gen = decoder.Generator(model, batch=2, max_seq=48)
     full = gen.generate_all(prompts, 16)
     # take a token that sequence 1 produces at step 5 as the end token
@@ -777,17 +778,46 @@ def test_generate_all_stops_at_the_end_token_and_trims_the_answers():
 
 
 def test_generate_all_sampling_is_reproducible_and_greedy_for_a_tiny_nucleus():
-    model = _build(SMALL, seed=7)
+    model = _build(BIG_HEADS, seed=7)
     g = torch.Generator().manual_seed(5)
-    prompts = [torch.randint(2, SMALL.vocab_size, (n,), generator=g).tolist() for n in (11, 6)]
+    prompts = [torch.randint(2, BIG_HEADS.vocab_size, (n,), generator=g).tolist() for n in (11, 6)]
     gen = decoder.Generator(model, batch=2, max_seq=40)
     a = gen.generate_all(prompts, 10, use_sampling=True, rng=torch.Generator(device="cuda").manual_seed(11))
     b = gen.generate_all(prompts, 10, use_sampling=True, rng=torch.Generator(device="cuda").manual_seed(11))
     c = gen.generate_all(prompts, 10, use_sampling=True, rng=torch.Generator(device="cuda").manual_seed(12))
-    assert a == b and all(0 <= t < SMALL.vocab_size for ans in a for t in ans)
+    assert a == b and all(0 <= t < BIG_HEADS.vocab_size for ans in a for t in ans)
     assert a != c  # 20 draws at temperature 0.7 from a 512-token vocabulary
     # a nucleus that only holds the most likely token: the greedy answer (the draw is from the bf16-rounded
     # logits the LM head returns, the greedy token from the same values)
     greedy = gen.generate_all(prompts, 10)
     tiny = gen.generate_all(prompts, 10, use_sampling=True, top_p=1e-9, rng=torch.Generator(device="cuda").manual_seed(1))
     assert tiny == greedy
+
+
+def test_captured_prompt_pass_equals_the_launch_by_launch_one():
+    """Generator.prefill replays one captured graph per prompt length; every replay, with other work of the
+    program in between (decode steps, prompts of other lengths), gives the tokens, and leaves the cache rows,
+    of the same pass issued launch by launch."""
+    model = _build(BIG_HEADS, seed=8)
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(21)
+    graphed = decoder.Generator(model, batch=2, max_seq=96, use_graph=True)
+    eager = decoder.Generator(model, batch=2, max_seq=96, use_graph=False)
+    assert graphed.lm_head and eager.lm_head
+    for rnd, P in enumerate((24, 40, 24, 24, 7, 40)):
+        prompt = torch.randint(0, BIG_HEADS.vocab_size, (2, P), generator=g, device=dev)
+        t1 = graphed.prefill(prompt)
+        t2 = eager.prefill(prompt)
+        assert torch.equal(t1, t2), (rnd, P)
+        for (k1, v1), (k2, v2) in zip(graphed.cache, eager.cache):
+            assert torch.equal(k1[:, :P], k2[:, :P]) and torch.equal(v1[:, :P], v2[:, :P])
+        # the program's own work between two replays
+        d1 = graphed.decode(t1, P, 5)
+        d2 = eager.decode(t2, P, 5)
+        assert torch.equal(d1, d2)
+    assert sorted(k[0] for k in graphed._pf_graphs) == [7, 24, 40]
+    # ragged prompts go through the same captured pass with their own lengths
+    prompts = [torch.randint(2, BIG_HEADS.vocab_size, (n,), generator=torch.Generator().manual_seed(n)).tolist() for n in (40, 13)]
+    assert graphed.generate_all(prompts, 6) == eager.generate_all(prompts, 6)
+    prompts = [prompts[1], prompts[0]]
+    assert graphed.generate_all(prompts, 6) == eager.generate_all(prompts, 6)
