@@ -331,7 +331,7 @@ def rope_rows_interleaved_to_hf(w: torch.Tensor, n_heads: int) -> torch.Tensor:
     return w.reshape(n_heads, d, 2, cols).transpose(1, 2).reshape(rows, cols)
 
 
-def _fuse(r: GGUFReader, names: Iterable[str], heads: Sequence[Optional[int]], k_want: int):
+def _fuse(r: GGUFReader, names: Iterable[str], heads: Sequence[Optional[int]], k_want: int, layout: str = "x86"):
     """I2_S tensors `names` (q/k with their head count for the rotary row order, None otherwise) ->
     (packed [N, k/4] int8, weight_scale bf16 [4])."""
     parts = []
@@ -340,28 +340,30 @@ def _fuse(r: GGUFReader, names: Iterable[str], heads: Sequence[Optional[int]], k
         if k != k_want:
             raise GGUFError(f"{name}: {k} columns, {k_want} expected")
         if h is not None:
-            w = rope_rows_hf_to_interleaved(i2s.i2s_unpack(codes, n, k), h).contiguous()
-            codes = i2s.i2s_pack(w)
+            w = rope_rows_hf_to_interleaved(i2s.i2s_unpack(codes, n, k, layout), h).contiguous()
+            codes = i2s.i2s_pack(w, layout)
         parts.append((codes, scale, n))
-    return i2s.i2s_to_int2(parts, k_want)
+    return i2s.i2s_to_int2(parts, k_want, layout)
 
 
-def gguf_to_int2_state(r: GGUFReader, args: Optional[ModelArgs] = None, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+def gguf_to_int2_state(r: GGUFReader, args: Optional[ModelArgs] = None, dtype=torch.bfloat16,
+                       layout: str = "x86") -> Dict[str, torch.Tensor]:
     """The state dict `decoder.Transformer(args)` loads, from a GGUF file of the
     bitnet-b1.58 architecture whose seven projections per block are I2_S tensors.  Embedding and norms
     are cast to `dtype`; `output.weight` is the file's own when it has one, else the embedding (tied,
-    as gpu/convert_safetensors.py:88-91 does)."""
+    as gpu/convert_safetensors.py:88-91 does).  `layout` names the I2_S byte layout of the build that
+    wrote the file (`i2s.I2S_LAYOUTS`; the file itself does not record it)."""
     a = args or model_args_from_gguf(r)
     st: Dict[str, torch.Tensor] = {}
     for layer in range(a.n_layers):
         b, p = f"blk.{layer}.", f"layers.{layer}."
-        packed, scale = _fuse(r, [b + "attn_q.weight", b + "attn_k.weight", b + "attn_v.weight"], [a.n_heads, a.n_kv_heads, None], a.dim)
+        packed, scale = _fuse(r, [b + "attn_q.weight", b + "attn_k.weight", b + "attn_v.weight"], [a.n_heads, a.n_kv_heads, None], a.dim, layout)
         st[p + "attention.wqkv.weight"], st[p + "attention.wqkv.weight_scale"] = packed, scale
-        packed, scale = _fuse(r, [b + "attn_output.weight"], [None], a.dim)
+        packed, scale = _fuse(r, [b + "attn_output.weight"], [None], a.dim, layout)
         st[p + "attention.wo.weight"], st[p + "attention.wo.weight_scale"] = packed, scale
-        packed, scale = _fuse(r, [b + "ffn_gate.weight", b + "ffn_up.weight"], [None, None], a.dim)
+        packed, scale = _fuse(r, [b + "ffn_gate.weight", b + "ffn_up.weight"], [None, None], a.dim, layout)
         st[p + "feed_forward.w13.weight"], st[p + "feed_forward.w13.weight_scale"] = packed, scale
-        packed, scale = _fuse(r, [b + "ffn_down.weight"], [None], a.ffn_dim)
+        packed, scale = _fuse(r, [b + "ffn_down.weight"], [None], a.ffn_dim, layout)
         st[p + "feed_forward.w2.weight"], st[p + "feed_forward.w2.weight_scale"] = packed, scale
         st[p + "attention_norm.weight"] = r.plain(b + "attn_norm.weight").to(dtype)
         st[p + "ffn_norm.weight"] = r.plain(b + "ffn_norm.weight").to(dtype)
@@ -374,7 +376,7 @@ def gguf_to_int2_state(r: GGUFReader, args: Optional[ModelArgs] = None, dtype=to
 
 
 def int2_state_to_gguf(state: Dict[str, torch.Tensor], args: ModelArgs, path: str, name: str = "bitnet-amd export",
-                       embed_dtype=torch.float16, i2s_type: int = I2_S_TYPE) -> None:
+                       embed_dtype=torch.float16, i2s_type: int = I2_S_TYPE, layout: str = "x86") -> None:
     """The inverse: a packed decoder state dict -> a GGUF file with I2_S projections (q/k rows back in
     Hugging Face order), fp32 norms and an fp16 embedding, as the reference's converter lays a model
     out (convert-hf-to-gguf-bitnet.py:1120-1190).  No tokenizer metadata is written."""
@@ -393,10 +395,10 @@ def int2_state_to_gguf(state: Dict[str, torch.Tensor], args: ModelArgs, path: st
 
     def parts(key, rows, heads):
         out = []
-        for (codes, scale), n, h in zip(i2s.int2_to_i2s(state[key].cpu(), state[key.replace("weight", "weight_scale")].cpu(), rows), rows, heads):
+        for (codes, scale), n, h in zip(i2s.int2_to_i2s(state[key].cpu(), state[key.replace("weight", "weight_scale")].cpu(), rows, layout), rows, heads):
             k = state[key].shape[1] * 4
             if h is not None:
-                codes = i2s.i2s_pack(rope_rows_interleaved_to_hf(i2s.i2s_unpack(codes, n, k), h).contiguous())
+                codes = i2s.i2s_pack(rope_rows_interleaved_to_hf(i2s.i2s_unpack(codes, n, k, layout), h).contiguous(), layout)
             out.append((codes, scale, n, k))
         return out
 

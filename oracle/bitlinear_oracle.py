@@ -445,6 +445,33 @@ def i2s_unpack_x86(packed: np.ndarray, n: int, k: int) -> np.ndarray:
     return (q.reshape(n, k).astype(np.int16) - 1).astype(np.int8)
 
 
+def i2s_pack_loops(w: np.ndarray, layout: str) -> np.ndarray:
+    """The three I2_S byte layouts of quantize_i2_s, restated as its own loops
+    (small cases only): "x86" = blocks of 128 elements of the flat stream, element
+    j of a block -> byte 32 * block + j % 32 at shift 6 - 2 * (j / 32)
+    (ggml-bitnet-mad.cpp:80-88); "neon" = blocks of 64, byte 16 * block + j % 16
+    at shift 6 - 2 * (j / 16) (:177-186); "rows4" = the x86 build without
+    activation-parallel kernels: byte (r / 4) * K + c holds rows 4g..4g+3 of
+    column c at shifts 6, 4, 2, 0 (:121-141).  Returns uint8 [N * K / 4]."""
+    w = np.asarray(w)
+    n, k = w.shape
+    q = (w.astype(np.int16) + 1).astype(np.uint8).reshape(-1)
+    out = np.zeros(n * k // 4, dtype=np.uint8)
+    if layout in ("x86", "neon"):
+        blk, grp = (128, 32) if layout == "x86" else (64, 16)
+        assert (n * k) % blk == 0
+        for i in range(n * k // blk):
+            for j in range(blk):
+                out[i * grp + j % grp] |= q[i * blk + j] << (6 - 2 * (j // grp))
+        return out
+    assert layout == "rows4" and n % 4 == 0
+    for rg in range(n // 4):
+        for c in range(k):
+            for r in range(4):
+                out[rg * k + c] |= q[(rg * 4 + r) * k + c] << (6 - 2 * r)
+    return out
+
+
 def i2s_vec_dot(packed: np.ndarray, y: np.ndarray, n: int, k: int) -> np.ndarray:
     """What ggml_vec_dot_i2_i8_s returns per weight row (as float in the
     reference, ggml-bitnet-mad.cpp:292-293): sum_k q[k]*y[k] with the
