@@ -1,7 +1,7 @@
 """BitNet-b1.58-2B-shaped decoder on top of the BitLinear library: the caller
 of the hot path (gpu/model.py:87-296 and the decode loop of
-gpu/generate.py:159-213, 264-288 of the reference), kept to what a greedy
-decode benchmark needs.
+gpu/generate.py:159-213, 217-304 of the reference): the model, the captured
+prompt pass and decode step, and the generation loop on token ids.
 
 Same module tree and parameter names as the reference (``layers.N.attention.
 {wqkv,wo,attn_sub_norm}``, ``layers.N.feed_forward.{w13,w2,ffn_sub_norm}``,
@@ -12,6 +12,7 @@ plain torch ops are used: RMSNorm and RoPE are closed forms, attention is
 softmax(QK^T/sqrt(d))V in fp32 over the cache.  One decode step is captured in
 a HIP graph and replayed per token, as the reference does with CUDA graphs.
 """
+import time
 from dataclasses import dataclass
 from typing import List, Optional, Tuple
 
@@ -657,7 +658,7 @@ class Generator:
     @torch.no_grad()
     def generate_all(self, prompts, gen_length: int, use_sampling: bool = False, temperature: float = 0.7,
                      top_p: float = 0.95, eos_id: Optional[int] = None, pad_id: int = 1,
-                     rng: Optional[torch.Generator] = None):
+                     rng: Optional[torch.Generator] = None, timings: Optional[dict] = None):
         """FastGen.generate_all of the reference (gpu/generate.py:217-304) on token
         ids: `prompts` is one list of ids per sequence of the batch (lengths may
         differ; padded with pad_id, the reference's 1); the whole batch is
@@ -667,7 +668,11 @@ class Generator:
         are out or, with eos_id, until any sequence has produced it.  Every
         answer is cut behind its first eos_id.  Greedy steps replay the captured
         graph of the whole step; a sampled step runs the same kernels and draws
-        with torch between them (`rng` makes the draws reproducible)."""
+        with torch between them (`rng` makes the draws reproducible).  A dict
+        passed as `timings` receives what the reference's Stats phases report
+        (gpu/stats.py, gpu/generate.py:243-288): prefill_s, decode_s,
+        decode_tokens (steps x sequences) and decode_tokens_per_s; it costs two
+        device synchronisations."""
         if len(prompts) != self.batch:
             raise ValueError(f"generate_all: {len(prompts)} prompts for a generator of batch {self.batch}")
         if any(len(q) < 1 for q in prompts):
@@ -683,9 +688,15 @@ class Generator:
             probs = torch.softmax(logits / temperature, dim=-1)
             return top_p_sample(probs, top_p, rng).view(-1)
 
+        if timings is not None:
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
         first, logits, lens = self._prefill_ragged(prompts, pad_id, use_sampling)
         if use_sampling:
             first = draw(logits)
+        if timings is not None:
+            torch.cuda.synchronize()
+            t_prefill = time.perf_counter()
         out = [first.view(1, -1)]
         stop = eos_id is not None and bool((first == eos_id).any())
         if gen_length > 1 and not stop:
@@ -715,6 +726,12 @@ class Generator:
                 if self.fused:
                     self.attn_ws.check()
         tokens = torch.cat(out, dim=0).t().tolist()  # [B][steps]
+        if timings is not None:
+            torch.cuda.synchronize()
+            t_end = time.perf_counter()
+            steps = len(tokens[0]) - 1
+            timings.update(prefill_s=t_prefill - t_start, decode_s=t_end - t_prefill, decode_tokens=steps * self.batch,
+                           decode_tokens_per_s=(steps * self.batch / (t_end - t_prefill)) if steps else 0.0)
         answers = []
         for ans in tokens:
             if eos_id is not None and eos_id in ans:

@@ -768,7 +768,10 @@ def test_generate_all_stops_at_the_end_token_and_trims_the_answers():
     # take a token that sequence 1 produces at step 5 as the end token
     eos = full[1][5]
     first_hit = min(min(a.index(eos) for a in full if eos in a), 15)
-    cut = gen.generate_all(prompts, 16, eos_id=eos)
+    timings = {}
+    cut = gen.generate_all(prompts, 16, eos_id=eos, timings=timings)
+    assert timings["decode_tokens"] == 2 * (len(max(cut, key=len)) - 1) or timings["decode_tokens"] == 2 * first_hit
+    assert timings["prefill_s"] > 0 and timings["decode_s"] > 0 and timings["decode_tokens_per_s"] > 0
     for a, f in zip(cut, full):
         want = f[: first_hit + 1]           # the loop ends after the first step in which any sequence hit it
         if eos in want:
