@@ -403,7 +403,31 @@ def latency_floor(lib, shapes, layers, dev, n_timed=20):
     out["load_only_us"]["mean_of_the_four"] = round(tot_floor / len(shapes), 3)
     out["load_only_chain_GBps"] = round(step_bytes / (tot_floor * n_layers) / 1e3, 1)
     out["load_only_chain_frac_of_hbm_peak"] = round(step_bytes / (tot_floor * n_layers) / 1e3 / HBM_PEAK_GBPS, 4)
+    # what handing a flag from one workgroup to another inside a launch costs (two workgroups of one launch pass a
+    # counter back and forth with relaxed device-scope accesses): the price of any producer -> consumer step that
+    # would replace a kernel boundary
+    flags = torch.zeros(128, dtype=torch.int32, device=dev)
+    gave_up = torch.zeros(1, dtype=torch.int32, device=dev)
+    rounds = 2000
+    trips = {}
+    for label, (wa, wb) in {"same_xcd (workgroups 0 and 8)": (0, 8), "next_xcd (0 and 1)": (0, 1), "far_xcd (0 and 4)": (0, 4)}.items():
+        best = None
+        for _ in range(3):
+            flags.zero_()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            assert lib.bitlinear_probe_flag_roundtrip(_p(flags), wa, wb, rounds, _p(gave_up), None) == 0
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / rounds
+            best = us if best is None else min(best, us)
+        trips[label] = round(best, 3)
+    assert int(gave_up[0]) == 0, "a flag never arrived"
+    out["flag_round_trip_us"] = trips
     out["note"] = (
+        "flag_round_trip = bitlinear_probe_flag_roundtrip (launch duration / 2000 round trips, one launch: its own start "
+        "and end weigh less than a nanosecond per trip); "
         "load_only = bitlinear_probe_weight_stream: the streaming kernel's grid, 16-byte loads and software pipeline with "
         "the activation operand, the decode, the MFMAs and the output removed; the chain figure is what 120 such launches "
         "per step would stream: the ceiling of any per-call kernel in a dependent chain on this machine"

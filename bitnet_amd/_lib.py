@@ -92,6 +92,7 @@ SIGNATURES = {
     "bitlinear_probe_empty": (_c_int, [_c_int, _c_int, _c_ptr]),
     "bitlinear_probe_weight_stream": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "bitlinear_probe_mfma_i8": (_c_int, [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr]),
+    "bitlinear_probe_flag_roundtrip": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
 }
 
 

@@ -2916,9 +2916,43 @@ extern "C" {
 // nothing, and when it only requests a matrix's bytes with the streaming kernel's access pattern.
 __global__ void probe_empty_kernel() {}
 
+// Two workgroups of one launch hand a counter back and forth through device memory: workgroup wa stores round r
+// into its word and polls the other's word until it reads r, workgroup wb polls first and then stores.  Stores and
+// loads are relaxed device-scope accesses (write-through, read past the caches), the cheapest form in which one
+// workgroup can see another's data inside a launch.  Every poll is bounded: a side that runs out sets *gave_up
+// and both sides stop after their own bound.
+__global__ void probe_flag_roundtrip_kernel(uint32_t* flags, int wa, int wb, int rounds, int spin_limit, int* gave_up) {
+    const int w = blockIdx.x;
+    if (threadIdx.x != 0 || (w != wa && w != wb)) return;
+    uint32_t* mine = flags + (w == wa ? 0 : 64);      // 256 bytes apart: different cache lines
+    uint32_t* theirs = flags + (w == wa ? 64 : 0);
+    bool bad = false;
+    for (int r = 1; r <= rounds && !bad; ++r) {
+        if (w == wa) __hip_atomic_store(mine, (uint32_t)r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int spins = 0;
+        while (__hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != (uint32_t)r)
+            if (++spins > spin_limit) {
+                bad = true;
+                break;
+            }
+        if (w != wa && !bad) __hip_atomic_store(mine, (uint32_t)r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (bad) __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 int bitlinear_probe_empty(int blocks, int threads, void* stream) {
     if (blocks < 1 || threads < 1 || threads > 1024) return BITLINEAR_ERR_ARG;
     hipLaunchKernelGGL(probe_empty_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream);
+    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+}
+
+int bitlinear_probe_flag_roundtrip(uint32_t* flags, int wg_a, int wg_b, int rounds, int* gave_up, void* stream) {
+    if (!flags || !gave_up) return BITLINEAR_ERR_NULL;
+    if (wg_a < 0 || wg_b < 0 || wg_a == wg_b || wg_a > 4095 || wg_b > 4095 || rounds < 1 || rounds > (1 << 20)) return BITLINEAR_ERR_ARG;
+    const int blocks = (wg_a > wg_b ? wg_a : wg_b) + 1;
+    // both workgroups must be resident at once: one wave each, far below what the machine holds
+    hipLaunchKernelGGL(probe_flag_roundtrip_kernel, dim3(blocks), dim3(64), 0, (hipStream_t)stream, flags, wg_a, wg_b, rounds,
+                       1 << 20, gave_up);
     return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
 }
 

@@ -3,7 +3,8 @@
  * (the reference has no counterpart): bench.py uses them to measure, in the same
  * run and launch style as its headline, what a kernel launch costs on this
  * machine when the kernel does nothing, when it only requests a matrix's bytes,
- * and what the matrix pipe sustains on the operand values of this workload.  Same conventions as include/bitlinear_hip.h: device pointers owned by
+ * what the matrix pipe sustains on the operand values of this workload, and what handing a flag from one
+ * workgroup to another costs.  Same conventions as include/bitlinear_hip.h: device pointers owned by
  * the caller, no allocation, no synchronisation, launches on the given stream.
  */
 #ifndef BITLINEAR_PROBES_H
@@ -43,6 +44,19 @@ int bitlinear_probe_weight_stream(const int8_t* const* packed, int count, int N,
  * never written (may be NULL).  Returns 0, 3 or 4 as above.
  */
 int bitlinear_probe_mfma_i8(int mode, int iters, uint32_t* sink, long long* ops, void* stream);
+
+/*
+ * One launch in which workgroups wg_a and wg_b (indices within the launch,
+ * 0..4095, different) hand a counter back and forth `rounds` (1..2^20) times
+ * through two words of `flags` (device memory, at least 128 uint32, zeroed by
+ * the caller before every call) with relaxed device-scope stores and loads:
+ * launch duration / rounds is the round trip of a flag between two workgroups,
+ * i.e. twice what one hand-over inside a launch costs.  Workgroups go to the
+ * XCDs round-robin by index, so wg_b = wg_a + 8 lands on the same XCD and
+ * wg_b = wg_a + 1 on the next.  Every wait is bounded; *gave_up (device int,
+ * zeroed by the caller) becomes 1 if one ran out.  Returns a BITLINEAR_* code.
+ */
+int bitlinear_probe_flag_roundtrip(uint32_t* flags, int wg_a, int wg_b, int rounds, int* gave_up, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1266,3 +1266,24 @@ def test_kernel_test_harness_reports_the_reference_lines():
     assert "torch BF16: " in lines[1] and len(lines) == 6
     assert all(r["w2a8_graph_us"] > 0 and r["bf16_graph_us"] > 0 for r in res)
     assert len(kernel_test.REFERENCE_SHAPES) == 8
+
+
+def test_flag_round_trip_probe_completes_and_checks_its_arguments():
+    """bitlinear_probe_flag_roundtrip (the bench's hand-over leg): both workgroups see every round, on the same
+    XCD and across XCDs; bad arguments are refused before any launch."""
+    import ctypes
+
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    lib = _lib.load_library()
+    dev = torch.device("cuda")
+    flags = torch.zeros(128, dtype=torch.int32, device=dev)
+    gave_up = torch.zeros(1, dtype=torch.int32, device=dev)
+    for wa, wb in ((0, 8), (0, 1), (5, 2)):
+        flags.zero_()
+        assert lib.bitlinear_probe_flag_roundtrip(P(flags), wa, wb, 300, P(gave_up), None) == 0
+        torch.cuda.synchronize()
+        assert int(gave_up[0]) == 0
+        assert int(flags[0]) == 300 and int(flags[64]) == 300  # both sides reached the last round
+    assert lib.bitlinear_probe_flag_roundtrip(P(flags), 3, 3, 10, P(gave_up), None) == 4
+    assert lib.bitlinear_probe_flag_roundtrip(P(flags), 0, 1, 0, P(gave_up), None) == 4
+    assert lib.bitlinear_probe_flag_roundtrip(None, 0, 1, 10, P(gave_up), None) == 2
