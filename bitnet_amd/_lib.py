@@ -48,6 +48,16 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
          _c_int, _c_ptr],
     ),
+    "bitlinear_forward_bf16_seg": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.POINTER(_c_int), _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+         _c_ptr],
+    ),
+    "bitlinear_norm_forward_bf16_seg": (
+        _c_int,
+        [_c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_ptr, _c_ptr, ctypes.POINTER(_c_int), _c_int, _c_ptr, _c_ptr, _c_ptr,
+         _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    ),
     "bitnet_attn_decode": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,

@@ -190,15 +190,35 @@ class BitLinearKernel(nn.Module):
     weight: torch.Tensor
     weight_scale: torch.Tensor
 
-    def __init__(self, in_features: int, out_features: int, bias: bool = False, quant_mode: int = QUANT_COMPILED):
+    def __init__(self, in_features: int, out_features: int, bias: bool = False, quant_mode: int = QUANT_COMPILED,
+                 seg_ends=None):
+        """seg_ends (not in the reference, opt-in): the output-row boundaries of
+        the sub-tensors a fused weight was assembled from, e.g. (2560, 3200,
+        3840) for wqkv.  Row n then takes weight_scale[j] of the segment it
+        lies in -- the layout gpu/convert_checkpoint.py:42-50 stores -- instead
+        of the reference kernel's equal slots n // (N // ws_num)
+        (bitnet_kernels.h:80), which hand q rows 1280..2559 the k scale."""
         super().__init__()
         if bias:
             raise ValueError("BitLinearKernel has no bias")
         self.in_features = in_features
         self.out_features = out_features
         self.quant_mode = quant_mode
+        self.set_segments(seg_ends)
         self.weight = nn.Parameter(torch.zeros(out_features, in_features // 4, dtype=torch.int8), requires_grad=False)
         self.weight_scale = nn.Parameter(torch.zeros(4, dtype=torch.bfloat16), requires_grad=False)
+
+    def set_segments(self, seg_ends) -> None:
+        """Switch between the reference's equal-slot rule (None) and explicit
+        output-row segments for the weight scales."""
+        if seg_ends is None:
+            self.seg_ends, self._seg_c = None, None
+            return
+        ends = tuple(int(e) for e in seg_ends)
+        if not 1 <= len(ends) <= 4 or ends[-1] != self.out_features or any(b <= a for a, b in zip((0,) + ends, ends)):
+            raise ValueError(f"seg_ends {ends}: 1 to 4 strictly increasing row boundaries ending at out_features")
+        self.seg_ends = ends
+        self._seg_c = (ctypes.c_int * len(ends))(*ends)
 
     def quant_input(self, input):
         return quant_input(input, self.quant_mode)
@@ -219,6 +239,13 @@ class BitLinearKernel(nn.Module):
         if M == 0:
             return out
         lib = _lib.load_library()
+        if self.seg_ends is not None:
+            st = lib.bitlinear_forward_bf16_seg(
+                _ptr(input), _ptr(self.weight), _ptr(out), _ptr(self.weight_scale), self._seg_c, len(self.seg_ends),
+                _ptr(q), _ptr(s), M, N, K, self.quant_mode, _stream_ptr(),
+            )
+            _lib.check(st, f"bitlinear_forward_bf16_seg(M={M}, N={N}, K={K})")
+            return out
         st = lib.bitlinear_forward_bf16(
             _ptr(input), _ptr(self.weight), _ptr(out), _ptr(self.weight_scale), _ptr(q), _ptr(s), M, N, K,
             self.quant_mode, _stream_ptr(),

@@ -1713,9 +1713,11 @@ constexpr int kSoloMaxUPW = 8;  // at most 8 k-steps (512 k = 64 vectors of 8 va
 template <int UPW, int VROW, int MT, bool COOP, int PRO, bool RES, int RPW>
 __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     // parameter order: what stands between the kernel's entry and its first loads comes first
-    // (the weight scales' slots are runs of slot_rows output rows each, the reference's rule n / (N / ws_num):
-    // one integer among the leading arguments instead of a table behind them)
-    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, int slot_rows,
+    // (the weight scales' slots are at most eight runs of slot_rows output rows each, run j reading entry
+    // (slot_map >> 3 j) & 7 of ws: the reference's rule n / (N / ws_num) is the identity map, a fused q/k/v
+    // matrix with its true segments of 2560 / 640 / 640 rows is six runs of 640 reading 0 0 0 0 1 2; two
+    // integers among the leading arguments instead of a table behind them, the map in the upper bits of rb_map)
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int rb_map, int S, int slot_rows,
     const uint16_t* __restrict__ aux, const uint16_t* __restrict__ ws, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ residual, float eps, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
     int32_t* __restrict__ acc_out) {
@@ -1724,6 +1726,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
     __shared__ __attribute__((aligned(16))) int red[MT == 1 ? kSoloRedSlots : kMaxWaves][256];                    // a wave's partial 16 x 16 tiles, [row block * S + k slice]
     __shared__ uint32_t wmax[kMaxWaves][MT];                                                // COOP: a wave's slice maximum per token
     __shared__ double wsq[PRO ? kMaxWaves : 1][MT];                                         // PRO 1, 2: a wave's slice sum of squares per token
+    const int RB = rb_map & 0xff;                      // row blocks per workgroup
+    const uint32_t slot_map = (uint32_t)rb_map >> 8;   // run j of slot_rows output rows reads ws[(slot_map >> 3 j) & 7]
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1787,7 +1791,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
         slot_first += n_first >= j * slot_rows ? 1 : 0;
         slot_last += n_last >= j * slot_rows ? 1 : 0;
     }
-    const uint16_t wsb_first = ws[slot_first];
+    const uint16_t wsb_first = ws[(slot_map >> (3 * slot_first)) & 7u];
     const int nthreads = 64 * RB * S;
     uint16_t e_res[kFusedMaxRB];
     if (RES) {
@@ -1910,7 +1914,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
 #pragma unroll
             for (int mm = 1; mm < MT; ++mm) sv_ = m == mm ? sf[mm] : sv_;
             uint16_t wsb = wsb_first;
-            if (slot_first != slot_last) wsb = ws[n / slot_rows];  // uniform branch, rare
+            if (slot_first != slot_last) wsb = ws[(slot_map >> (3 * (n / slot_rows))) & 7u];  // uniform branch, rare
             uint16_t o = f32_to_bf16_rne((float)sum / sv_ * bf16_to_f32(wsb));
             if (RES) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
             if (out) out[(size_t)m * N + n] = o;
@@ -1930,10 +1934,12 @@ __global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_kernel(
 // wave's row blocks.  One barrier, behind the products, as in bitlinear_solo_kernel.
 template <int UPW, int RPW, bool RES>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_solo_kernel(
-    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int RB, int S, int slot_rows,
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int rb_map, int S, int slot_rows,
     const uint16_t* __restrict__ s, const uint16_t* __restrict__ ws, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ residual, int32_t* __restrict__ acc_out) {
     __shared__ __attribute__((aligned(16))) int red[kSoloRedSlots][256];  // partial 16 x 16 tiles, [row block * S + k slice]
+    const int RB = rb_map & 0xff;                      // row blocks per workgroup
+    const uint32_t slot_map = (uint32_t)rb_map >> 8;   // run j of slot_rows output rows reads ws[(slot_map >> 3 j) & 7]
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1973,7 +1979,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_solo_kernel(
         slot_first += n_first >= j * slot_rows ? 1 : 0;
         slot_last += n_last >= j * slot_rows ? 1 : 0;
     }
-    const uint16_t wsb_first = ws[slot_first];
+    const uint16_t wsb_first = ws[(slot_map >> (3 * slot_first)) & 7u];
     const uint16_t e_sb = s[(tid & 15) < M ? (tid & 15) : M - 1];  // every output slot of a thread belongs to token tid % 16
     const int nthreads = 64 * RB * S;
     uint16_t e_res[kFusedMaxRB];
@@ -2033,7 +2039,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_solo_kernel(
             for (int k = 0; k < S; ++k) sum += red[tb * S + k][t & 255];
             if (acc_out) acc_out[(size_t)m * N + n] = sum;  // uniform: parity tests only
             uint16_t wsb = wsb_first;
-            if (slot_first != slot_last) wsb = ws[n / slot_rows];  // uniform branch, rare
+            if (slot_first != slot_last) wsb = ws[(slot_map >> (3 * (n / slot_rows))) & 7u];  // uniform branch, rare
             uint16_t o = f32_to_bf16_rne((float)sum / sf * bf16_to_f32(wsb));
             if (RES) o = f32_to_bf16_rne(bf16_to_f32(e_res[r]) + bf16_to_f32(o));
             if (out) out[(size_t)m * N + n] = o;
@@ -2100,6 +2106,37 @@ int set_status(int st) {
 struct ShapeWs {
     int n, k, ws_num;
 };
+
+// The weight-scale segments as the kernels with two leading integers take them: at most eight runs of
+// slot_rows output rows, run j reading ws[(map >> 3 j) & 7].  Every boundary must be a multiple of the run
+// length (their greatest common divisor); a map that needs more than eight runs goes to the kernels that
+// take the whole table.
+struct SlotRule {
+    int slot_rows;
+    uint32_t map;
+    bool ok;
+};
+SlotRule slot_rule(const ScaleMap& smap, int N) {
+    auto gcd = [](int a, int b) {
+        while (b) {
+            const int t = a % b;
+            a = b;
+            b = t;
+        }
+        return a;
+    };
+    int g = N;
+    for (int j = 0; j + 1 < smap.nseg; ++j) g = gcd(g, smap.ends[j]);
+    SlotRule r = {g, 0u, g > 0 && N / g <= 8};
+    if (!r.ok) return r;
+    for (int run = 0; run < 8; ++run) {
+        const int n = run * g < N ? run * g : N - 1;
+        int seg = 0;
+        while (seg < smap.nseg - 1 && n >= smap.ends[seg]) ++seg;
+        r.map |= (uint32_t)seg << (3 * run);
+    }
+    return r;
+}
 // (N, K) -> ws_num of the reference's template instances (bitnet_kernels.cu:4-33)
 const ShapeWs kShapeTable[] = {
     {3840, 2560, 3},  {2560, 2560, 1},  {13824, 2560, 2}, {2560, 6912, 1},  {4800, 3200, 6},
@@ -2434,14 +2471,14 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
     const dim3 grid((blocks16 + pl.rb * pl.rpw - 1) / (pl.rb * pl.rpw), 1, 1);
     const dim3 block(64 * pl.rb * pl.s, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
-    // equal slots only (what the forward entry points use): rows per slot
-    const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
-    for (int j = 0; j + 1 < smap.nseg; ++j)
-        if (smap.ends[j] != (j + 1) * slot_rows) return BITLINEAR_ERR_ARG;
+    const SlotRule rule = slot_rule(smap, N);
+    if (!rule.ok) return BITLINEAR_ERR_ARG;
+    const int slot_rows = rule.slot_rows;
+    const int rb_map = pl.rb | (int)(rule.map << 8);
     if (pro != 0 && (!pl.coop || !norm_weight)) return BITLINEAR_ERR_ARG;
     g_last_kernel = pro == 0 ? "bitlinear_solo_kernel" : (pro == 1 ? "bitlinear_solo_kernel<norm>" : "bitlinear_solo_kernel<gate+norm>");
 #define BITLINEAR_LAUNCH_SOLO_W(U, V, T, C, P, R, W)                                                                      \
-    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C, P, R, W>), grid, block, 0, stream, x, wq, M, N, K, pl.rb, pl.s, \
+    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C, P, R, W>), grid, block, 0, stream, x, wq, M, N, K, rb_map, pl.s, \
                        slot_rows, norm_weight, ws, out, residual, eps, q_out, s_out, acc_out)
 #define BITLINEAR_LAUNCH_SOLO_P(U, V, T, C, P, R) BITLINEAR_LAUNCH_SOLO_W(U, V, T, C, P, R, 1)
 #define BITLINEAR_LAUNCH_SOLO(U, V, T, C) BITLINEAR_LAUNCH_SOLO_P(U, V, T, C, 0, false)
@@ -2557,12 +2594,13 @@ int launch_prod_solo(const int8_t* act, const int8_t* packed, uint16_t* out, int
     const dim3 grid((blocks16 + pl.rpw - 1) / pl.rpw, 1, 1);
     const dim3 block(64 * pl.s, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
-    const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
-    for (int j = 0; j + 1 < smap.nseg; ++j)
-        if (smap.ends[j] != (j + 1) * slot_rows) return BITLINEAR_ERR_ARG;  // equal slots only
+    const SlotRule rule = slot_rule(smap, N);
+    if (!rule.ok) return BITLINEAR_ERR_ARG;
+    const int slot_rows = rule.slot_rows;
+    const int rb_map = 1 | (int)(rule.map << 8);
     g_last_kernel = "gemv_i2_solo_kernel";
 #define BITLINEAR_LAUNCH_PS(U, W, R)                                                                               \
-    hipLaunchKernelGGL((gemv_i2_solo_kernel<U, W, R>), grid, block, 0, stream, act, wq, M, N, K, 1, pl.s, slot_rows, \
+    hipLaunchKernelGGL((gemv_i2_solo_kernel<U, W, R>), grid, block, 0, stream, act, wq, M, N, K, rb_map, pl.s, slot_rows, \
                        s, ws, out, residual, acc_out)
 #define BITLINEAR_LAUNCH_PS_W(U, W)         \
     if (residual) BITLINEAR_LAUNCH_PS(U, W, true); \
@@ -2817,10 +2855,7 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
                                                             (N / 16) < 1024);
     if (prod_solo_wanted && t_tune.path != 1 && t_tune.path != 2 && M <= 16) {
         const ProdPlan pp = plan_prod_solo(M, N, K);
-        bool equal = true;
-        const int slot_rows = smap.nseg > 1 ? smap.ends[0] : N;
-        for (int j = 0; j + 1 < smap.nseg; ++j) equal = equal && smap.ends[j] == (j + 1) * slot_rows;
-        if (pp.ok && equal)
+        if (pp.ok && slot_rule(smap, N).ok)
             return launch_prod_solo(act, packed, out, acc_out, out ? s : (const uint16_t*)packed, out ? ws : (const uint16_t*)packed,
                                     smap, M, N, K, pp, stream, residual);
     }
@@ -3174,23 +3209,30 @@ int bitlinear_int8xint2_grouped(const bitlinear_problem* problems, int count, vo
     return set_status(BITLINEAR_OK);
 }
 
+// seg_ends[0 .. nseg) -> the kernels' table: strictly increasing, the last one N
+static int segment_map(const int* seg_ends, int nseg, int N, ScaleMap* sm) {
+    if (!seg_ends) return BITLINEAR_ERR_NULL;
+    if (nseg < 1 || nseg > kMaxSeg) return BITLINEAR_ERR_ARG;
+    sm->nseg = nseg;
+    int prev = 0;
+    for (int j = 0; j < kMaxSeg; ++j) {
+        if (j < nseg) {
+            if (seg_ends[j] <= prev || seg_ends[j] > N) return BITLINEAR_ERR_ARG;
+            prev = seg_ends[j];
+        }
+        sm->ends[j] = (j < nseg) ? seg_ends[j] : N;
+    }
+    return prev == N ? BITLINEAR_OK : BITLINEAR_ERR_ARG;
+}
+
 int bitlinear_int8xint2_seg(const int8_t* input0, const int8_t* input1, uint16_t* output0, const uint16_t* s,
                             const uint16_t* ws, const int* seg_ends, int nseg, int M, int N, int K, void* stream) {
     refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!input0 || !input1 || !output0 || !s || !ws || !seg_ends) return set_status(BITLINEAR_ERR_NULL);
-    if (nseg < 1 || nseg > kMaxSeg) return set_status(BITLINEAR_ERR_ARG);
     ScaleMap sm;
-    sm.nseg = nseg;
-    int prev = 0;
-    for (int j = 0; j < kMaxSeg; ++j) {
-        if (j < nseg) {
-            if (seg_ends[j] <= prev || seg_ends[j] > N) return set_status(BITLINEAR_ERR_ARG);
-            prev = seg_ends[j];
-        }
-        sm.ends[j] = (j < nseg) ? seg_ends[j] : N;
-    }
-    if (prev != N) return set_status(BITLINEAR_ERR_ARG);
+    const int st = segment_map(seg_ends, nseg, N, &sm);
+    if (st != BITLINEAR_OK) return set_status(st);
     return set_status(launch_gemv(input0, input1, output0, nullptr, s, ws, sm, M, N, K, (hipStream_t)stream));
 }
 
@@ -3256,16 +3298,22 @@ static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t*
     return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
 }
 
+// seg_ends == nullptr: the reference's equal slots (bitnet_kernels.h:80); otherwise the caller's segments
 static int forward_impl(const uint16_t* x, const int8_t* packed, uint16_t* output0, int32_t* acc_out, const uint16_t* ws,
-                        int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+                        int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream,
+                        const int* seg_ends = nullptr, int nseg = 0) {
     refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !packed || !output0 || !ws) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
     if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)q_ws)) & 15u) return set_status(BITLINEAR_ERR_ARG);
-    const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    if (seg_ends) {
+        const int st = segment_map(seg_ends, nseg, N, &sm);
+        if (st != BITLINEAR_OK) return set_status(st);
+    }
     // up to four tokens: the kernel whose waves quantize their own slices
-    if (mode == 0 && t_tune.path == 0 && t_tune.solo != 5 && M <= kSoloMaxTokens) {
+    if (mode == 0 && t_tune.path == 0 && t_tune.solo != 5 && M <= kSoloMaxTokens && slot_rule(sm, N).ok) {
         const SoloPlan sp = plan_solo(M, N, K);
         if (sp.ok && (t_tune.solo >= 1 || solo_wanted(M, N, K)))
             return set_status(launch_solo(x, packed, output0, acc_out, ws, sm, q_ws, s_ws, M, N, K, sp, (hipStream_t)stream));
@@ -3288,6 +3336,13 @@ static int forward_impl(const uint16_t* x, const int8_t* packed, uint16_t* outpu
 int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
                            int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
     return forward_impl(x, packed, output0, nullptr, ws, q_ws, s_ws, M, N, K, mode, stream);
+}
+
+int bitlinear_forward_bf16_seg(const uint16_t* x, const int8_t* packed, uint16_t* output0, const uint16_t* ws,
+                               const int* seg_ends, int nseg, int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode,
+                               void* stream) {
+    if (!seg_ends) return set_status(BITLINEAR_ERR_NULL);
+    return forward_impl(x, packed, output0, nullptr, ws, q_ws, s_ws, M, N, K, mode, stream, seg_ends, nseg);
 }
 
 // The array's name is only a handle on the host: its device address is looked up once per device
@@ -3331,18 +3386,42 @@ int bitlinear_forward_bf16_acc_i32(const uint16_t* x, const int8_t* packed, int3
     return forward_impl(x, packed, output0, acc_out, ws, q_ws, s_ws, M, N, K, mode, stream);
 }
 
+static int norm_forward_impl(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu, const int8_t* packed,
+                             const uint16_t* ws, const uint16_t* residual, uint16_t* output0, int8_t* q_ws, uint16_t* s_ws,
+                             int M, int N, int K, int mode, void* stream, const int* seg_ends, int nseg);
+
 int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu,
                                 const int8_t* packed, const uint16_t* ws, const uint16_t* residual, uint16_t* output0,
                                 int8_t* q_ws, uint16_t* s_ws, int M, int N, int K, int mode, void* stream) {
+    return norm_forward_impl(x, norm_weight, eps, glu, packed, ws, residual, output0, q_ws, s_ws, M, N, K, mode, stream,
+                             nullptr, 0);
+}
+
+int bitlinear_norm_forward_bf16_seg(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu,
+                                    const int8_t* packed, const uint16_t* ws, const int* seg_ends, int nseg,
+                                    const uint16_t* residual, uint16_t* output0, int8_t* q_ws, uint16_t* s_ws, int M, int N,
+                                    int K, int mode, void* stream) {
+    if (!seg_ends) return set_status(BITLINEAR_ERR_NULL);
+    return norm_forward_impl(x, norm_weight, eps, glu, packed, ws, residual, output0, q_ws, s_ws, M, N, K, mode, stream,
+                             seg_ends, nseg);
+}
+
+static int norm_forward_impl(const uint16_t* x, const uint16_t* norm_weight, float eps, int glu, const int8_t* packed,
+                             const uint16_t* ws, const uint16_t* residual, uint16_t* output0, int8_t* q_ws, uint16_t* s_ws,
+                             int M, int N, int K, int mode, void* stream, const int* seg_ends, int nseg) {
     refresh_tuning();
     if (!shape_ok(M, N, K)) return set_status(BITLINEAR_ERR_SHAPE);
     if (!x || !norm_weight || !packed || !ws || !output0) return set_status(BITLINEAR_ERR_NULL);
     if (mode != 0 && mode != 1) return set_status(BITLINEAR_ERR_ARG);
     if ((((uintptr_t)x) | ((uintptr_t)packed) | ((uintptr_t)norm_weight) | ((uintptr_t)q_ws)) & 15u)
         return set_status(BITLINEAR_ERR_ARG);
-    const ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    ScaleMap sm = equal_slots(N, bitlinear_ws_num(N, K));
+    if (seg_ends) {
+        const int st = segment_map(seg_ends, nseg, N, &sm);
+        if (st != BITLINEAR_OK) return set_status(st);
+    }
     // up to four tokens: the kernel whose waves prepare their own slices
-    if (mode == 0 && t_tune.path == 0 && t_tune.solo != 5 && M <= kSoloMaxTokens) {
+    if (mode == 0 && t_tune.path == 0 && t_tune.solo != 5 && M <= kSoloMaxTokens && slot_rule(sm, N).ok) {
         const SoloPlan sp = plan_solo(M, N, K, glu ? 2 : 1, residual != nullptr);
         if (sp.ok && (t_tune.solo >= 1 || solo_norm_wanted(M, N, K, glu ? 2 : 1)))
             return set_status(launch_solo(x, packed, output0, nullptr, ws, sm, nullptr, nullptr, M, N, K, sp,

@@ -34,6 +34,9 @@ class ModelArgs:
     ffn_dim: int = 6912
     norm_eps: float = 1e-5
     rope_theta: float = 500000.0
+    # not in the reference: give every row of the fused wqkv / w13 products the scale of the sub-tensor it
+    # came from (what convert_checkpoint.py:42-50 stores) instead of the reference kernel's equal slots
+    segment_scales: bool = False
 
 
 class RMSNorm(nn.Module):
@@ -242,6 +245,14 @@ def norm_bitlinear(x, norm: "RMSNorm", lin: BitLinearKernel, glu: bool = False, 
     out = torch.empty(M, lin.out_features, dtype=torch.bfloat16, device=x.device)
     q_ws = torch.empty(M, K, dtype=torch.int8, device=x.device)
     s_ws = torch.empty(M, dtype=torch.bfloat16, device=x.device)
+    if lin.seg_ends is not None:
+        st = _lib.load_library().bitlinear_norm_forward_bf16_seg(
+            _ptr(x), _ptr(norm.weight), norm.eps, 1 if glu else 0, _ptr(lin.weight), _ptr(lin.weight_scale),
+            lin._seg_c, len(lin.seg_ends), _ptr(residual) if residual is not None else None, _ptr(out), _ptr(q_ws),
+            _ptr(s_ws), M, lin.out_features, K, lin.quant_mode, _stream_ptr(),
+        )
+        _lib.check(st, f"bitlinear_norm_forward_bf16_seg(M={M}, N={lin.out_features}, K={lin.in_features})")
+        return out
     st = _lib.load_library().bitlinear_norm_forward_bf16(
         _ptr(x), _ptr(norm.weight), norm.eps, 1 if glu else 0, _ptr(lin.weight), _ptr(lin.weight_scale),
         _ptr(residual) if residual is not None else None, _ptr(out), _ptr(q_ws), _ptr(s_ws), M, lin.out_features, K,
@@ -257,7 +268,8 @@ class Attention(nn.Module):
         self.head_dim = args.dim // args.n_heads
         self.n_heads = args.n_heads
         self.n_kv_heads = args.n_kv_heads
-        self.wqkv = BitLinearKernel(args.dim, (args.n_heads + 2 * args.n_kv_heads) * self.head_dim)
+        nq, nk = args.n_heads * self.head_dim, args.n_kv_heads * self.head_dim
+        self.wqkv = BitLinearKernel(args.dim, nq + 2 * nk, seg_ends=(nq, nq + nk, nq + 2 * nk) if args.segment_scales else None)
         self.wo = BitLinearKernel(args.n_heads * self.head_dim, args.dim)
         self.attn_sub_norm = RMSNorm(args.dim, args.norm_eps)
 
@@ -287,7 +299,8 @@ class Attention(nn.Module):
 class FeedForward(nn.Module):
     def __init__(self, args: ModelArgs):
         super().__init__()
-        self.w13 = BitLinearKernel(args.dim, 2 * args.ffn_dim)
+        self.w13 = BitLinearKernel(args.dim, 2 * args.ffn_dim,
+                                   seg_ends=(args.ffn_dim, 2 * args.ffn_dim) if args.segment_scales else None)
         self.w2 = BitLinearKernel(args.ffn_dim, args.dim)
         self.ffn_sub_norm = RMSNorm(args.ffn_dim, args.norm_eps)
 

@@ -239,6 +239,30 @@ int bitlinear_norm_forward_bf16(const uint16_t* x, const uint16_t* norm_weight,
                                 int M, int N, int K, int mode, void* stream);
 
 /*
+ * bitlinear_forward_bf16 and bitlinear_norm_forward_bf16 with the weight
+ * scales assigned by explicit output-row segments, as bitlinear_int8xint2_seg
+ * does for the plain product: rows [seg_ends[j-1], seg_ends[j]) use ws[j]
+ * (seg_ends host array, strictly increasing, seg_ends[nseg-1] == N,
+ * 1 <= nseg <= 8, every boundary a multiple of 16).  This is how
+ * gpu/convert_checkpoint.py:42-50 lays the scales of a fused matrix out: wqkv
+ * stores [s_q, s_k, s_v, 0] for segments of 2560 / 640 / 640 rows, which the
+ * reference kernel's equal-thirds rule (bitnet_kernels.h:80) does not follow.
+ * Opt-in: the plain entries keep the reference's rule bit for bit.  Same
+ * kernels, launch shapes and arithmetic as the plain entries.
+ */
+int bitlinear_forward_bf16_seg(const uint16_t* x, const int8_t* packed,
+                               uint16_t* output0, const uint16_t* ws,
+                               const int* seg_ends, int nseg,
+                               int8_t* q_ws, uint16_t* s_ws,
+                               int M, int N, int K, int mode, void* stream);
+int bitlinear_norm_forward_bf16_seg(const uint16_t* x, const uint16_t* norm_weight,
+                                    float eps, int glu, const int8_t* packed,
+                                    const uint16_t* ws, const int* seg_ends, int nseg,
+                                    const uint16_t* residual, uint16_t* output0,
+                                    int8_t* q_ws, uint16_t* s_ws,
+                                    int M, int N, int K, int mode, void* stream);
+
+/*
  * Kernel / launch-shape override for tuning runs and tests.  Process-wide;
  * results never depend on it.
  *   kernel 0: built-in choice (other arguments ignored)

@@ -377,12 +377,18 @@ def residual_add_bf16(res_bits: np.ndarray, o_bits: np.ndarray) -> np.ndarray:
     return f32_to_bf16_bits((bf16_bits_to_f32(res_bits) + bf16_bits_to_f32(o_bits)).astype(np.float32))
 
 
-def norm_bitlinear(x_bits, g_bits, eps, w, ws_bits, glu=False, residual_bits=None, mode=QUANT_COMPILED, ws_num=None):
-    """[gate ->] RMSNorm -> quantizer -> product -> epilogue [-> residual add]."""
+def norm_bitlinear(x_bits, g_bits, eps, w, ws_bits, glu=False, residual_bits=None, mode=QUANT_COMPILED, ws_num=None,
+                   seg_ends=None):
+    """[gate ->] RMSNorm -> quantizer -> product -> epilogue [-> residual add];
+    with seg_ends the weight scales follow the true segments
+    (bitlinear_int8xint2_seg) instead of the equal slots."""
     h = squared_relu_glu_bf16(x_bits) if glu else x_bits
     y = rmsnorm_bf16(h, g_bits, eps)
     q, s_bits = quant_input(y, mode)
-    _, out = bitlinear_int8xint2(q, w, s_bits, ws_bits, ws_num)
+    if seg_ends is not None:
+        _, out = bitlinear_int8xint2_seg(q, w, s_bits, ws_bits, seg_ends)
+    else:
+        _, out = bitlinear_int8xint2(q, w, s_bits, ws_bits, ws_num)
     return residual_add_bf16(residual_bits, out) if residual_bits is not None else out
 
 

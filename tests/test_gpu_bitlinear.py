@@ -208,6 +208,77 @@ def test_qkv_scale_slots_follow_the_reference_rule_and_seg_variant():
     assert not np.array_equal(want, want_seg)
 
 
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 8, 16, 40, 130])
+@pytest.mark.parametrize("n,k,ends", [
+    (3840, 2560, (2560, 3200, 3840)),   # wqkv as convert_checkpoint.py:42-50 lays its scales out: six runs of 640 rows
+    (13824, 2560, (6912, 13824)),       # w13: the segments coincide with the reference's equal halves
+    (3840, 2560, (16, 3824, 3840)),     # boundaries whose common divisor leaves more than eight runs: the table kernels
+    (2560, 6912, (640, 2560)),
+    (1040, 3200, (1040,)),
+])
+def test_forward_entries_with_segment_scales(n, k, ends, m):
+    """bitlinear_forward_bf16_seg and bitlinear_norm_forward_bf16_seg (with and without residual): row n takes the
+    weight scale of the segment it lies in.  Bit for bit against the oracle's segmented product behind the oracle's
+    quantizer / norm, at decode, batched-decode and prompt sizes; where the segments are the reference's equal slots
+    the plain entry gives the same bits, elsewhere it must not."""
+    import ctypes
+
+    lib = _lib.load_library()
+    rng = np.random.default_rng(n + 3 * k + m + len(ends))
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    xb = o.f32_to_bf16_bits((rng.standard_normal((m, k)) * 1.9).astype(np.float32))
+    gb = o.f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(k)).astype(np.float32))
+    rb = o.f32_to_bf16_bits(rng.standard_normal((m, n)).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    q, s_bits = o.quant_input(xb, o.QUANT_COMPILED)
+    _, want = o.bitlinear_int8xint2_seg(q, w, s_bits, ws_bits, ends)
+    pk, wsd = _packed_dev(w), dev_bf16(ws_bits)
+    mod = bitlinear.BitLinearKernel(k, n, seg_ends=ends).cuda()
+    mod.weight.data, mod.weight_scale.data = pk, wsd
+    _assert_bits_equal(host_bits(mod(dev_bf16(xb))), want, f"forward, segments {ends}")
+    plain = bitlinear.BitLinearKernel(k, n).cuda()
+    plain.weight.data, plain.weight_scale.data = pk, wsd
+    equal_rule = np.array_equal(np.searchsorted(np.asarray(ends), np.arange(n), side="right"),
+                                o.ws_slot(n, o.ws_num_for_shape(n, k)))
+    assert np.array_equal(host_bits(plain(dev_bf16(xb))), want) == equal_rule
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    ends_c = (ctypes.c_int * len(ends))(*ends)
+    for res in (None, rb):
+        want_n = o.norm_bitlinear(xb, gb, 1e-5, w, ws_bits, residual_bits=res, seg_ends=ends)
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        q_ws = torch.empty(m, k, dtype=torch.int8, device="cuda")
+        s_ws = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+        r = dev_bf16(res) if res is not None else None
+        x, g = dev_bf16(xb), dev_bf16(gb)
+        st = lib.bitlinear_norm_forward_bf16_seg(P(x), P(g), 1e-5, 0, P(pk), P(wsd), ends_c, len(ends), P(r), P(out), P(q_ws),
+                                                 P(s_ws), m, n, k, 0, None)
+        torch.cuda.synchronize()
+        assert st == 0
+        _assert_bits_equal(host_bits(out), want_n, f"norm forward, segments {ends}, residual {res is not None}")
+
+
+def test_segment_entries_refuse_bad_segment_lists():
+    import ctypes
+
+    lib = _lib.load_library()
+    n, k, m = 64, 128, 1
+    x = torch.zeros(m, k, dtype=torch.bfloat16, device="cuda")
+    pk = torch.zeros(n, k // 4, dtype=torch.int8, device="cuda")
+    ws = torch.ones(4, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    for ends in [(32, 48), (48, 32, 64), (0, 64), tuple(range(8, 80, 8))]:
+        ends_c = (ctypes.c_int * len(ends))(*ends)
+        st = lib.bitlinear_forward_bf16_seg(P(x), P(pk), P(out), P(ws), ends_c, len(ends), None, None, m, n, k, 0, None)
+        assert st == 4, ends
+        st = lib.bitlinear_norm_forward_bf16_seg(P(x), P(x), 1e-5, 0, P(pk), P(ws), ends_c, len(ends), None, P(out), None,
+                                                 None, m, n, k, 0, None)
+        assert st == 4, ends
+    assert lib.bitlinear_forward_bf16_seg(P(x), P(pk), P(out), P(ws), None, 1, None, None, m, n, k, 0, None) == 2
+    with pytest.raises(ValueError):
+        bitlinear.BitLinearKernel(k, n, seg_ends=(32, 48))
+
+
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("m,k", [(1, 2560), (1, 6912), (16, 2560), (5, 27648), (3, 8), (2, 10240)])
 def test_quantizer_bit_exact(mode, m, k):

@@ -824,3 +824,186 @@ def test_captured_prompt_pass_equals_the_launch_by_launch_one():
     assert graphed.generate_all(prompts, 6) == eager.generate_all(prompts, 6)
     prompts = [prompts[1], prompts[0]]
     assert graphed.generate_all(prompts, 6) == eager.generate_all(prompts, 6)
+
+
+# ---------------------------------------------------------------------------
+# A converted Hugging Face checkpoint through the decoder (gpu/convert_safetensors.py:43-93,
+# gpu/convert_checkpoint.py:29-32, 42-77)
+# ---------------------------------------------------------------------------
+HF_ARGS = decoder.ModelArgs(dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=320, ffn_dim=768, segment_scales=True)
+
+
+def _hf_checkpoint(args, seed):
+    """Synthetic tensors under the Hugging Face names, bf16 like the published master weights; q, k and v
+    projections of clearly different magnitude, so that their three weight scales differ by factors."""
+    g = torch.Generator().manual_seed(seed)
+    hd = args.dim // args.n_heads
+    r = lambda std, *shape: (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+    st = {}
+    for layer in range(args.n_layers):
+        b = f"model.layers.{layer}."
+        st[b + "self_attn.q_proj.weight"] = r(0.02, args.n_heads * hd, args.dim)
+        st[b + "self_attn.k_proj.weight"] = r(0.06, args.n_kv_heads * hd, args.dim)
+        st[b + "self_attn.v_proj.weight"] = r(0.009, args.n_kv_heads * hd, args.dim)
+        st[b + "self_attn.o_proj.weight"] = r(0.02, args.dim, args.n_heads * hd)
+        st[b + "input_layernorm.weight"] = 1 + r(0.1, args.dim)
+        st[b + "post_attention_layernorm.weight"] = 1 + r(0.1, args.dim)
+        st[b + "self_attn.attn_sub_norm.weight"] = 1 + r(0.1, args.dim)
+        st[b + "mlp.ffn_sub_norm.weight"] = 1 + r(0.1, args.ffn_dim)
+        st[b + "mlp.gate_proj.weight"] = r(0.03, args.ffn_dim, args.dim)
+        st[b + "mlp.up_proj.weight"] = r(0.015, args.ffn_dim, args.dim)
+        st[b + "mlp.down_proj.weight"] = r(0.02, args.dim, args.ffn_dim)
+    st["model.embed_tokens.weight"] = r(0.5, args.vocab_size, args.dim)
+    st["model.norm.weight"] = 1 + r(0.1, args.dim)
+    return st
+
+
+def _hf_convention_logits(st, args, ids):
+    """The model the checkpoint describes, evaluated the way the Hugging Face side of the reference's converter
+    sees it, in plain torch: projections kept apart and in their original row order, rotary embedding on the two
+    halves of a head (rotate_half), every BitLinear as the reference's fp module (activations snapped to the int8
+    grid, gpu/model.py:77-85, times weights ternarised and dequantised per tensor, gpu/convert_checkpoint.py:29-32),
+    sub-norms and squared-ReLU gate as gpu/model.py:159-160, 195-196.  fp32 arithmetic, rounded to bf16 where the
+    decoder's tensors are bf16.  ids [B, T] -> logits fp32 [B, T, vocab]."""
+    dev = ids.device
+    bf = torch.bfloat16
+    hd = args.dim // args.n_heads
+    rep = args.n_heads // args.n_kv_heads
+    B, T = ids.shape
+    w = {k: v.to(dev) for k, v in st.items()}
+
+    def rms(x, g):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + args.norm_eps) * g.float()).to(bf)
+
+    def deq(t):  # convert_checkpoint.py:29-32, in the checkpoint's dtype
+        s = 1.0 / t.abs().mean().clamp_(min=1e-5)
+        return ((t * s).round().clamp(-1, 1) / s).float()
+
+    def bitlinear_fp(x, t):  # gpu/model.py:77-85
+        xf = x.float()
+        s = 127 / xf.abs().max(dim=-1, keepdim=True).values.clamp_(min=1e-5)
+        return (((xf * s).round().clamp(-128, 127) / s) @ deq(t).T).to(bf)
+
+    inv = 1.0 / (args.rope_theta ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
+    ang = torch.outer(torch.arange(T, device=dev, dtype=torch.float32), inv)
+    cos = torch.cat([ang.cos(), ang.cos()], dim=-1)[None, :, None, :]  # [1, T, 1, hd]: frequency i at i and i + hd/2
+    sin = torch.cat([ang.sin(), ang.sin()], dim=-1)[None, :, None, :]
+
+    def rope_half(x):  # x [B, T, heads, hd]
+        xf = x.float()
+        x1, x2 = xf[..., : hd // 2], xf[..., hd // 2 :]
+        return (xf * cos + torch.cat([-x2, x1], dim=-1) * sin).to(bf)
+
+    h = w["model.embed_tokens.weight"][ids]  # [B, T, dim] bf16
+    causal = torch.ones(T, T, dtype=torch.bool, device=dev).tril()
+    for layer in range(args.n_layers):
+        b = f"model.layers.{layer}."
+        x = rms(h, w[b + "input_layernorm.weight"])
+        q = rope_half(bitlinear_fp(x, w[b + "self_attn.q_proj.weight"]).view(B, T, args.n_heads, hd))
+        k = rope_half(bitlinear_fp(x, w[b + "self_attn.k_proj.weight"]).view(B, T, args.n_kv_heads, hd))
+        v = bitlinear_fp(x, w[b + "self_attn.v_proj.weight"]).view(B, T, args.n_kv_heads, hd)
+        k = k.repeat_interleave(rep, dim=2).float()  # query head j reads kv head j // rep
+        v = v.repeat_interleave(rep, dim=2).float()
+        sc = torch.einsum("bthd,bshd->bhts", q.float(), k) * hd ** -0.5
+        sc = sc.masked_fill(~causal[None, None], float("-inf"))
+        o = torch.einsum("bhts,bshd->bthd", torch.softmax(sc, dim=-1), v).reshape(B, T, args.dim).to(bf)
+        h = (h.float() + bitlinear_fp(rms(o, w[b + "self_attn.attn_sub_norm.weight"]), w[b + "self_attn.o_proj.weight"]).float()).to(bf)
+        x = rms(h, w[b + "post_attention_layernorm.weight"])
+        gate = bitlinear_fp(x, w[b + "mlp.gate_proj.weight"])
+        up = bitlinear_fp(x, w[b + "mlp.up_proj.weight"])
+        inner = ((torch.relu(gate.float()) ** 2).to(bf).float() * up.float()).to(bf)
+        h = (h.float() + bitlinear_fp(rms(inner, w[b + "mlp.ffn_sub_norm.weight"]), w[b + "mlp.down_proj.weight"]).float()).to(bf)
+    return rms(h, w["model.norm.weight"]).float() @ w["model.embed_tokens.weight"].float().T
+
+
+def _load_converted(path, args):
+    with torch.device("cuda"):
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            model = decoder.Transformer(args)
+        finally:
+            torch.set_default_dtype(prev)
+    model.load_state_dict(torch.load(path, weights_only=True), strict=True)
+    return model
+
+
+def test_converted_hf_checkpoint_runs_through_the_decoder_like_the_hf_convention_model(tmp_path):
+    """Row (f3) on the device: synthetic Hugging Face tensors -> convert_hf_checkpoint (rotary row permutation,
+    q|k|v and gate|up fusing, per-sub-tensor ternarisation, four-slot scales, packing) -> strict load into the
+    decoder -> prompt pass and decode step through the library's int8 kernels with the segment scale rule.  The
+    yardstick never sees a fused, permuted or packed tensor: it evaluates the unfused projections with half-split
+    rotary embedding and the reference's fp BitLinear.  Attention scores are invariant under the permutation
+    (q and k are permuted alike within a head), and the int8 path differs from the fp module only in where
+    roundings fall (same integer products; tests/test_gpu_bitlinear.py::test_fp_path_agrees_with_the_int8_path
+    derives the per-call bound), so the logits agree up to the amplification of those roundings by the later
+    quantizers: a few percent of the logits' norm.  A wrong row order, segment boundary or scale slot moves them
+    by tens of percent -- the control at the end runs the same file with the reference kernel's slot rule
+    n // (N // ws_num) (bitnet_kernels.h:80; one slot for a shape outside its table, so k and v rows are scaled
+    by s_q) and must land far outside the bound."""
+    from safetensors.torch import save_file
+
+    from bitnet_amd import checkpoint
+
+    args = HF_ARGS
+    st = _hf_checkpoint(args, seed=11)
+    src = str(tmp_path / "model.safetensors")
+    save_file(st, src)
+    path = checkpoint.convert_hf_checkpoint(src, str(tmp_path / "out"), args)
+    model = _load_converted(path, args)
+    for lr in model.layers:  # the three scales of a fused wqkv really differ, else the control below proves nothing
+        s3 = lr.attention.wqkv.weight_scale.float()
+        assert float(s3[1] / s3[0]) > 2.0 and float(s3[0] / s3[2]) > 1.5 and float(s3[3]) == 0.0
+
+    dev = torch.device("cuda")
+    B, T, S = 2, 48, 64
+    g = torch.Generator(device="cuda").manual_seed(12)
+    ids = torch.randint(0, args.vocab_size, (B, T + 1), generator=g, device=dev)
+    want = _hf_convention_logits(st, args, ids)  # [B, T + 1, V]
+
+    @torch.no_grad()
+    def run(m):
+        cos, sin = decoder.rope_tables(args.dim // args.n_heads, S, args.rope_theta, dev)
+        cache = m.make_cache(B, S, dev)
+        hid = m.prefill_hidden_fused(ids[:, :T].contiguous(), cache, cos, sin)  # quantizer kernels + int8 MFMA GEMM
+        prompt_logits = m.output(m.norm(hid)).float()
+        ws = decoder.AttnWorkspace(B, args.n_heads, args.n_kv_heads, 8, dev)
+        pos = torch.full((B, 1), T, device=dev)
+        step_logits = m.forward_decode_fused(ids[:, T:].contiguous(), pos, cache, cos, sin, ws)  # one-kernel forwards
+        ws.check()
+        # the unfused glue (BitLinearKernel.forward per projection) on the same prompt
+        glue = m.forward_tokens(ids[:, :T].contiguous(), torch.arange(T, device=dev)[None].expand(B, T).contiguous(),
+                                m.make_cache(B, S, dev), cos, sin)
+        torch.cuda.synchronize()
+        return torch.cat([prompt_logits, step_logits], dim=1), glue
+
+    rel = lambda a, b: float((a - b).norm() / b.norm())
+    got, glue = run(model)
+    assert bool(torch.isfinite(got).all())
+    err_prompt, err_step, err_glue = rel(got[:, :T], want[:, :T]), rel(got[:, T:], want[:, T:]), rel(glue, want[:, :T])
+    bound = 0.035  # measured 0.017-0.020 over three seeds
+    assert err_prompt < bound and err_step < bound and err_glue < bound, (err_prompt, err_step, err_glue)
+    top = want.topk(2, dim=-1).values
+    clear = (top[..., 0] - top[..., 1]) > 0.15 * want.std()
+    assert int(clear.sum()) > 10
+    assert torch.equal(got.argmax(-1)[clear], want.argmax(-1)[clear])
+
+    # control: the same file through the reference kernel's slot rule
+    import dataclasses
+
+    thirds = _load_converted(path, dataclasses.replace(args, segment_scales=False))
+    got3, _ = run(thirds)
+    assert rel(got3, want) > 2 * bound, rel(got3, want)  # measured 0.094-0.112
+
+    # control: a converter that forgot the rotary row permutation of q and k (convert_safetensors.py:43-47)
+    state = checkpoint.hf_to_model_state(st, args)
+    hd = args.dim // args.n_heads
+    for layer in range(args.n_layers):
+        b = f"model.layers.{layer}.self_attn."
+        state[f"layers.{layer}.attention.wqkv.weight"] = torch.cat(
+            [st[b + "q_proj.weight"], st[b + "k_proj.weight"], st[b + "v_proj.weight"]], dim=0)
+    bad = str(tmp_path / "unpermuted.pt")
+    torch.save(checkpoint.model_state_to_int2(state, args), bad)
+    got_bad, _ = run(_load_converted(bad, args))
+    assert rel(got_bad, want) > 2 * bound, rel(got_bad, want)
