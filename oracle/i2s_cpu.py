@@ -20,12 +20,41 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+_path = LIB_PATH
+_build_note = "-O3 -mavx2 -fopenmp (built beforehand)"
+
+
+def use_native_build() -> str:
+    """For timing runs: rebuild the library on THIS host with -O3 -march=native (what the reference's own
+    harness uses, utils/test_gemm_kernel.sh:392-397) next to the portable build and load that one from now on.
+    Falls back to the portable build when no compiler is at hand.  Returns a note saying which build is loaded."""
+    global _lib, _path, _build_note
+    native = os.path.join(_DIR, "_build", "libi2s_oracle_native.so")
+    try:
+        res = subprocess.run(
+            ["make", "-C", _DIR, "-B", "OUT=_build/libi2s_oracle_native.so",
+             "CFLAGS=-O3 -march=native -fopenmp -fPIC -shared -Wall -Wextra"],
+            capture_output=True, text=True, timeout=120,
+        )
+        ok = res.returncode == 0 and os.path.exists(native)
+    except (OSError, subprocess.SubprocessError):
+        ok = False
+    if ok:
+        try:
+            ctypes.CDLL(native)
+        except OSError:
+            ok = False
+    if ok:
+        _lib, _path, _build_note = None, native, "-O3 -march=native -fopenmp (built on this host)"
+    return _build_note
+
+
 def load():
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
+        if not os.path.exists(_path):
             build()
-        lib = ctypes.CDLL(LIB_PATH)
+        lib = ctypes.CDLL(_path)
         vp, i64, ci, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
         lib.i2s_pack_row.argtypes = [vp, vp, i64]
         lib.i2s_pack_row.restype = None
