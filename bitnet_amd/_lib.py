@@ -84,7 +84,6 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     ),
     "bitnet_attn_decode_set_threads": (_c_int, [_c_int]),
-    "bitnet_attn_decode_set_kernel": (_c_int, [_c_int]),
     "bitnet_lm_head_greedy": (
         _c_int,
         [_c_ptr, _c_ptr, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -97,6 +96,7 @@ SIGNATURES = {
     "bitnet_lm_head_workgroups": (_c_int, [_c_int]),
     "bitnet_lm_head_set_kernel": (_c_int, [_c_int]),
     "bitlinear_set_tuning": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
+    "bitlinear_plan_name": (_c_int, [_c_int, _c_int, _c_int, _c_int, ctypes.c_char_p, _c_int]),
     "bitlinear_int8xint2_grouped": (_c_int, [_c_ptr, _c_int, _c_ptr]),
     # include/bitlinear_probes.h
     "bitlinear_probe_empty": (_c_int, [_c_int, _c_int, _c_ptr]),
@@ -152,6 +152,15 @@ def load_library(path: str = None) -> ctypes.CDLL:
     if path is None:
         _lib = lib
     return lib
+
+
+def plan_name(entry: int, M: int, N: int, K: int) -> str:
+    """bitlinear_plan_name: the kernels (template arguments, grid, block, LDS) a call would launch; needs no GPU."""
+    buf = ctypes.create_string_buffer(1024)
+    st = load_library().bitlinear_plan_name(entry, M, N, K, buf, len(buf))
+    if st != 0:
+        raise BitLinearLibraryError(f"bitlinear_plan_name(entry={entry}, M={M}, N={N}, K={K}): status {st}")
+    return buf.value.decode()
 
 
 def check(status: int, what: str) -> None:

@@ -22,6 +22,7 @@
 
 #include <hip/hip_runtime.h>
 #include <mutex>
+#include <string>
 #include <type_traits>
 #include <stdint.h>
 #include <stdio.h>
@@ -115,144 +116,9 @@ __device__ __forceinline__ int scale_slot_uniform(const ScaleMap& smap, int n) {
     return slot;
 }
 
-// ---------------------------------------------------------------------------
-// Decode kernel, M <= 4 tokens: one wave owns a 16-row block over all of K
-// ---------------------------------------------------------------------------
-// A lane loads 16 bytes (dwordx4): four packed words = rows 4q..4q+3 of one
-// 16-k chunk; the wave's 64 lanes cover 1 KB contiguous = 16 rows x 256 k.
-// Word i of every lane is the A operand of MFMA i (i = 0..3), which therefore
-// sees row 4q+i at A-row index p = 4*sigma + q with k-chunk 4g + sigma
-// (g = lane / 16).  The B operand puts token m's chunk 4g + sigma' at column
-// p' = 4*sigma' + m.  Entry (p, p') of the 16x16 result is a true partial dot
-// product exactly when sigma == sigma'; those entries sit in lanes 20*G + m
-// (G = sigma), register q, and the four G parts are added at the end.  The
-// off-diagonal entries are never read.  No cross-wave reduction, no workgroup
-// barrier after the weight stream.
+// Up to this many tokens a product goes through the kernels that keep the token rows in LDS or registers per
+// wave (the staged and the streaming kernel); beyond, through the kernels that split the tokens over MFMA columns
 constexpr int kDecodeMaxTokens = 4;
-constexpr int kDecodeMaxWaves = 4;
-constexpr int kDecodeMaxLdsBytes = 48 * 1024;
-
-template <int R>
-__global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
-    const int8_t* __restrict__ act, const v4u* __restrict__ wq, int M, int N, int K, int nwaves,
-    uint16_t* __restrict__ out, int32_t* __restrict__ acc_out, const uint16_t* __restrict__ s,
-    const uint16_t* __restrict__ ws, ScaleMap smap) {
-    __shared__ int red[kDecodeMaxWaves * 256];
-    extern __shared__ __attribute__((aligned(16))) int8_t lds_act[];  // [M][K]
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int rb = blockIdx.x * nwaves + wave;  // 16-row block of this wave
-    const bool rows_ok = rb < (N >> 4);
-    const int g = lane >> 4;
-    const int sg = (lane >> 2) & 3;  // sigma (A side) / sigma' (B side)
-    const int q = lane & 3;          // row quad (A side) / token (B side)
-    const int chunk = 4 * g + sg;    // 16-k chunk inside a 256-k step
-    const int steps = (K + 255) >> 8;
-
-    // 16-byte group of (row quad q, chunk): tile chunk/2, half chunk&1
-    const int grp = (chunk >> 1) * 8 + (q >> 1) * 4 + (chunk & 1) * 2 + (q & 1);
-    const v4u* wp = wq + (size_t)(rows_ok ? rb : 0) * (K >> 2) + grp;
-
-    // epilogue operands, fetched early as raw bits (see the split-K kernel)
-    const int e_row = lane >> 2;
-    const int e_m = lane & 3;
-    const int e_n = rb * 16 + e_row;
-    uint16_t e_sb = 0, e_wsb = 0;
-    if (out) {
-        e_sb = s[e_m < M ? e_m : M - 1];
-        e_wsb = ws[scale_slot(smap, rows_ok ? e_n : 0)];
-    }
-
-    const int tokB = q < M ? q : M - 1;  // columns of tokens >= M are never read
-    const int8_t* bp = lds_act + (size_t)tokB * K + chunk * 16;
-
-    v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0}, acc3 = {0, 0, 0, 0};
-    v4i accb = {0, 0, 0, 0};
-    const int neg2w = (int)0xFEFEFEFEu;
-    const v4i neg2 = {neg2w, neg2w, neg2w, neg2w};
-
-    // Software pipeline over K: R 1-KB steps per round, the next round's loads
-    // issued before this round's MFMAs, so a wave always has R to 2R KB in flight.
-    v4u w0[R], w1[R];
-    auto load_round = [&](v4u(&w)[R], int base) {
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
-            int st = base + j;
-            // clamped into the row block: a step (or the part of the last step) past K is ignored when used
-            st = (st < steps && (st * 256 + chunk * 16) < K) ? st : 0;
-            w[j] = __builtin_nontemporal_load(wp + (size_t)st * 64);
-        }
-    };
-    auto use_round = [&](const v4u(&w)[R], int base) {
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
-            const int st = base + j;
-            const bool live = rows_ok && st < steps && (st * 256 + chunk * 16) < K;
-            const int stc = st < steps ? st : steps - 1;
-            const int kc = (stc * 256 + chunk * 16) < K ? stc * 256 : 0;
-            v4i b = *(const v4i*)(bp + (size_t)kc);
-            if (!live) b = v4i{0, 0, 0, 0};
-            const uint32_t wd[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
-            v4i a[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                a[i].x = (int)(wd[i] & 0x03030303u);
-                a[i].y = (int)((wd[i] >> 2) & 0x03030303u);
-                a[i].z = (int)((wd[i] >> 4) & 0x03030303u);
-                a[i].w = (int)((wd[i] >> 6) & 0x03030303u);
-            }
-            acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[1], b, acc1, 0, 0, 0);
-            acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[2], b, acc2, 0, 0, 0);
-            acc3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[3], b, acc3, 0, 0, 0);
-            accb = __builtin_amdgcn_mfma_i32_16x16x64_i8(neg2, b, accb, 0, 0, 0);
-        }
-    };
-    load_round(w0, 0);
-    if (steps > R) load_round(w1, R);
-    {
-        // activations -> LDS while the weight loads are in flight
-        const int nvec = (M * K) >> 4;
-        for (int i = threadIdx.x; i < nvec; i += nwaves * 64)
-            *(v4i*)(lds_act + (size_t)i * 16) = *(const v4i*)(act + (size_t)i * 16);
-        lds_barrier();
-    }
-    for (int base = 0; base < steps; base += 2 * R) {
-        use_round(w0, base);
-        if (base + 2 * R < steps) load_round(w0, base + 2 * R);
-        if (base + R < steps) {
-            use_round(w1, base + R);
-            if (base + 3 * R < steps) load_round(w1, base + 3 * R);
-        }
-    }
-
-    // result lane 16G + p' holds A-rows 4G + r (r = register): diagonal <=> sigma' == G
-    int* myred = red + wave * 256;
-    if (sg == g) {
-        int* dst = myred + g * 64 + q;  // [G][row][token], token = q here
-        const int r0[4] = {acc0.x, acc1.x, acc2.x, acc3.x};
-        const int r1[4] = {acc0.y, acc1.y, acc2.y, acc3.y};
-        const int r2[4] = {acc0.z, acc1.z, acc2.z, acc3.z};
-        const int r3[4] = {acc0.w, acc1.w, acc2.w, acc3.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {  // register r of MFMA i is row 4r + i
-            dst[(0 + i) * 4] = r0[i] + accb.x;
-            dst[(4 + i) * 4] = r1[i] + accb.y;
-            dst[(8 + i) * 4] = r2[i] + accb.z;
-            dst[(12 + i) * 4] = r3[i] + accb.w;
-        }
-    }
-    // same wave wrote and reads: LDS operations of a wave complete in order
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (rows_ok && e_m < M) {
-        const int sum = myred[lane] + myred[64 + lane] + myred[128 + lane] + myred[192 + lane];
-        if (acc_out) acc_out[(size_t)e_m * N + e_n] = sum;
-        if (out) out[(size_t)e_m * N + e_n] = f32_to_bf16_rne((float)sum / bf16_to_f32(e_sb) * bf16_to_f32(e_wsb));
-    }
-}
 
 // ---------------------------------------------------------------------------
 // Streaming kernel (M <= 4 tokens): waves that own whole 16-row blocks and never meet
@@ -263,9 +129,13 @@ __global__ __launch_bounds__(kDecodeMaxWaves * 64) void gemv_i2_decode_kernel(
 // pipeline that does not stop at item boundaries: a ring of D 16-byte weight loads per lane (D KB per
 // wave, the lanes of one load covering 1 KB = 16 rows x 256 k), each slot re-requested for the next
 // round of k-steps -- or for the first round of the wave's next row block -- right after the MFMAs
-// that consumed it.  The operand scheme is the decode kernel's: the four words of a lane's 16 bytes
-// are rows 4q..4q+3 of one 16-k chunk and feed four MFMAs whose B operand carries token m's chunk at
-// column 4 * sigma + m, so only the diagonal blocks of the results are read.  The problem's int8
+// that consumed it.  Operand scheme: a lane loads 16 bytes = four packed words = rows 4q..4q+3 of one
+// 16-k chunk (the wave's 64 lanes cover 1 KB contiguous = 16 rows x 256 k).  Word i of every lane is the A
+// operand of MFMA i (i = 0..3), which therefore sees row 4q+i at A-row index p = 4*sigma + q with k-chunk
+// 4g + sigma (g = lane / 16).  The B operand puts token m's chunk 4g + sigma' at column p' = 4*sigma' + m.
+// Entry (p, p') of the 16x16 result is a true partial dot product exactly when sigma == sigma': those
+// entries sit in lanes 20*G + m (G = sigma), register q, and the four G parts are added at the end; the
+// off-diagonal entries are never read.  The problem's int8
 // activation rows are copied into LDS once per workgroup (requested before the weights, so that they
 // are not queued behind them: loads return in the order of their requests), with sum(a) per token
 // taken on the way (it removes the +2 of the stored codes); after that single barrier no wave waits
@@ -2060,8 +1930,7 @@ thread_local const char* g_last_kernel = "none";
 struct Tuning {
     int waves = 0;
     int upw = 0;
-    int decode_waves = 0;
-    int path = 0;  // 0 = built-in choice, 1 = decode kernel, 2 = split-K kernel, 3 = fused shape, 4 = never fuse, 5 = GEMM tile
+    int path = 0;  // 0 = built-in choice, 2 = split-K kernel, 3 = fused shape, 4 = never fuse, 5 = GEMM tile
     int fused[3] = {1, 10, 4};
     int prefill_big = 0;
     int prefill_band = 0;  // row tiles per band of the prefill GEMM's tile order, 0 = built-in choice
@@ -2087,16 +1956,99 @@ void refresh_tuning() {
 }
 
 using bitnet_host::OncePerDevice;
-// Row blocks from which ONE call goes through the streaming kernel (measured at M = 1: 55296 x 5120, 3456
-// row blocks: 12.7 us against 13.3 with the LDS-staged kernel's many small workgroups, at 4 tokens 13.0
-// against 15.4; 20480 x 3200, 1280 row blocks: 6.5 against 5.0 -- with few row blocks per CU the waves
-// that split K finish earlier).  Grouped calls take it from two problems on.
+// ---------------------------------------------------------------------------
+// Every crossover of the dispatch code below, in one place.  Each value is where two kernels (or two launch
+// shapes of one kernel) measured level on an MI355X, per call from a HIP graph of dependent launches over
+// distinct weights; the figures that set it stand beside it.  bitlinear_plan_name() reports what these rules
+// choose for a given (entry, M, N, K); tests/test_dispatch_plan.py pins the choice over a grid of shapes, so
+// that a changed value shows up as a changed row of that table.
+// ---------------------------------------------------------------------------
+namespace dispatch {
+// --- which kernel -----------------------------------------------------------
+// tokens above which the product is the MFMA GEMM instead of a GEMV kernel (the GEMV kernels hold at most 16
+// tokens: one MFMA column block)
+constexpr int kPrefillMinTokens = 16;
+// 16 < M <= this: GEMM or split-K GEMV by the estimate in launch_gemv (fitted to the 2B shapes; above it the
+// GEMM is always ahead)
+constexpr int kSplitKMaxTokens = 256;
+// row blocks (N / 16) from which ONE product at up to 4 tokens goes through the streaming kernel: 55296 x 5120
+// (3456 blocks) 12.7 us against 13.3 with the staged kernel's many small workgroups, at 4 tokens 13.0 against
+// 15.4; 20480 x 3200 (1280 blocks) 6.5 against 5.0: with few row blocks per CU the waves that split K finish earlier
 constexpr int kStreamMinBlocks = 2048;
-constexpr int kPrefillMinTokens = 16;  // above this the MFMA GEMM takes over from the split-K kernel
-constexpr int kPrefillFewTiles = 330;   // up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles
-constexpr int kPrefillSplit2Tiles = 320;  // up to this many 32 x 128 tiles two groups of waves split a tile's K,
-constexpr int kPrefillSplit4Tiles = 200;  // up to this many, and a long K, four
+// row blocks from which the product without staging (gemv_i2_solo_kernel) is ahead of the staged kernel at up to
+// 4 tokens: 13824 x 2560 (864 blocks) 4.46 -> 4.19 us; 3840 x 2560 (240) 2.89 staged against 2.95, 2560 x 6912 (160)
+// 3.65 against 4.06.  Above 4 tokens it is ahead at every 2B shape (3840 x 2560 at 8 tokens 3.40 -> 3.34, 2560 x 6912
+// 4.90 -> 4.71), and the staged kernel only stays where a workgroup shares the rows between row blocks (same bound)
+constexpr int kManyBlocks = 432;
+// ... and up to here: from 1024 row blocks on the staged kernel's many small workgroups stay ahead (20480 x 3200:
+// 5.0 us against 5.9) until the streaming kernel takes over
+constexpr int kSmallWorkgroupBlocks = 1024;
+// row blocks from which a wave of the two kernels without a shared prologue takes four row blocks instead of two
+// (13824 x 2560: 4.80 -> 4.46 us forward; product at 8 tokens 4.67 -> 4.62, at 16 5.78 -> 5.15)
+constexpr int kFourRowBlocksPerWave = 864;
+// activation elements (M * K) up to which the forward call is ONE kernel in which every workgroup quantizes the
+// block again; above, quantizer kernel + product kernel (8 x 2560 = 20480: 5.9-6.2 us fused against 5.6 as two
+// kernels; 16 x 2560: 9.7 against 6.1)
+constexpr int kFuseMaxElems = 16384;
+// the same with a norm (and gate) in the prologue (K = 2560: 3 tokens 5.2 us fused against 5.5, 4 tokens 6.5
+// against 5.7; K = 6912: 2 tokens 7.4 against 6.7)
+constexpr int kFuseMaxElemsNorm = 9216;
+// bitlinear_solo_kernel (every wave prepares its own slice) instead of the shared-prologue kernel: one token up
+// to this K (3840 x 2560 3.40 -> 3.18 us, 2560 x 2560 3.33 -> 3.13, 13824 x 2560 5.03 -> 4.81, 2560 x 6912
+// 4.56 -> 4.31) ...
+constexpr int kSoloMaxK = 8192;
+// ... two to four tokens above this K (2560 x 6912: two tokens 5.61 -> 5.21, four 6.81 -> 6.61; at K = 2560 four
+// tokens 4.16 -> 4.59, not taken), two tokens also below kManyBlocks row blocks (3.86 -> 3.69, 3.75 -> 3.62;
+// 13824 x 2560 5.14 -> 6.07, not taken); with a norm in front only at one token up to this K (3840 x 2560
+// 3.95 -> 3.80, 13824 x 2560 5.44 -> 5.16; 2560 x 6912 with gate and residual 5.87 -> 6.12, not taken)
+constexpr int kSoloLongRowK = 4096;
+// rows from which the norm + quantizer kernel of a prompt runs a wave per row (norm + product at K = 2560:
+// 32.2 -> 30.1 us at 2048 rows, 53.6 -> 48.7 at 4096; below 0.2-0.9 us behind)
+constexpr int kNormRowsPerWaveMinRows = 1024;
+// --- prefill GEMM: tile and k-split by the number of tiles ------------------
+// up to this many 64 x 128 tiles the GEMM uses 32 x 128 tiles (M = 128: 11.4 -> 9.0 us at 3840 x 2560, 21.5 -> 16.4
+// at 2560 x 6912); beyond, 64 x 256 (level or ahead from here on: 2560 x 6912 at M = 1536 31.7 -> 29.2)
+constexpr int kPrefillFewTiles = 330;
+// wide matrices at prompt sizes take the 64 x 256 tile whatever the count
+constexpr int kPrefillWideN = 8192, kPrefillWideMinTokens = 512;
+// up to this many 32 x 128 tiles two groups of waves split a tile's K (M = 128, K = 2560: 9.0 -> 8.0 us), ...
+constexpr int kPrefillSplit2Tiles = 320;
+// ... up to this many, and from this K on, four (K = 6912: 16.6 -> 13.1 -> 12.6 us with two and four)
+constexpr int kPrefillSplit4Tiles = 200;
 constexpr int kPrefillSplit4MinK = 5120;
+// about one tile per CU (more than half the CUs, at most all 256): 64 x 128 tiles with two k-groups (2560 x 6912
+// at M = 512 19.1 -> 17.3 us) and 64 x 256 tiles with two k-groups (2560 x 6912 at M = 1024 25.9 -> 23.4)
+constexpr int kPrefillOnePerCuMin = 128, kPrefillOnePerCuMax = 256;
+// a little more than one round of 64 x 256 tiles (three per CU): one round of 128 x 256 tiles (two per CU) instead
+// (13824 x 2560 at M = 1024: 864 tiles, 46.5 -> 42.3 us)
+constexpr int kPrefillRound64 = 768, kPrefillRound128 = 1024;
+}  // namespace dispatch
+using namespace dispatch;
+
+// Planning calls (bitlinear_plan_name): the entry points' own dispatch code runs, and every launch is recorded --
+// the kernel with its template arguments, grid, block and dynamic LDS -- instead of issued.  Nothing touches a device.
+struct PlanLog {
+    bool active = false;
+    std::string text;
+};
+thread_local PlanLog t_plan;
+void plan_note(const char* kernel, dim3 grid, dim3 block, size_t lds) {
+    char buf[96];
+    snprintf(buf, sizeof(buf), " grid=(%u,%u,%u) block=%u lds=%zu", grid.x, grid.y, grid.z, block.x, lds);
+    if (!t_plan.text.empty()) t_plan.text += " + ";
+    // the kernel as written at the launch site, without the parentheses that protect its commas
+    std::string k(kernel);
+    if (k.size() >= 2 && k.front() == '(' && k.back() == ')') k = k.substr(1, k.size() - 2);
+    t_plan.text += k + buf;
+}
+#define BL_LAUNCH(KERNEL, GRID, BLOCK, LDS, STREAM, ...)                           \
+    do {                                                                           \
+        if (t_plan.active)                                                         \
+            plan_note(#KERNEL, GRID, BLOCK, LDS);                                  \
+        else                                                                       \
+            hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, STREAM, __VA_ARGS__);     \
+    } while (0)
+int launch_status() { return (t_plan.active || hipGetLastError() == hipSuccess) ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH; }
 
 int set_status(int st) {
     g_status = st;
@@ -2170,7 +2122,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
     const dim3 block(waves * 64, 1, 1);
     const uint32_t* wq = (const uint32_t*)packed;
 #define BITLINEAR_LAUNCH(U)                                                                                  \
-    hipLaunchKernelGGL(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, M, N, K, waves, out, acc_out, s, ws, smap, residual)
+    BL_LAUNCH(gemv_i2_mfma_kernel<U>, grid, block, 0, stream, act, wq, M, N, K, waves, out, acc_out, s, ws, smap, residual)
     switch (upw) {
         case 1: BITLINEAR_LAUNCH(1); break;
         case 2: BITLINEAR_LAUNCH(2); break;
@@ -2178,28 +2130,7 @@ int launch_splitk(const int8_t* act, const int8_t* packed, uint16_t* out, int32_
         default: BITLINEAR_LAUNCH(8); break;
     }
 #undef BITLINEAR_LAUNCH
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
-}
-
-int launch_decode(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
-                  const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream) {
-    const int steps = (K + 255) / 256;
-    int waves = 4;
-    g_last_kernel = "gemv_i2_decode_kernel";
-    if (t_tune.decode_waves > 0) waves = t_tune.decode_waves;
-    const int blocks16 = N / 16;
-    const dim3 grid((blocks16 + waves - 1) / waves, 1, 1);
-    const dim3 block(waves * 64, 1, 1);
-    const size_t lds = (size_t)M * K;
-    const v4u* wq = (const v4u*)packed;
-#define BITLINEAR_LAUNCH(R)                                                                                     \
-    hipLaunchKernelGGL(gemv_i2_decode_kernel<R>, grid, block, lds, stream, act, wq, M, N, K, waves, out, acc_out, s, ws, smap)
-    // R steps (1 KB each per wave) per round, two rounds in flight
-    if (steps <= 4) BITLINEAR_LAUNCH(2);
-    else if (steps <= 10) BITLINEAR_LAUNCH(5);
-    else BITLINEAR_LAUNCH(8);
-#undef BITLINEAR_LAUNCH
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    return launch_status();
 }
 
 // Launch shape of the fused kernel: RB 16-row blocks per workgroup, S waves
@@ -2214,13 +2145,7 @@ struct FusedPlan {
 // pre-quantized variant raises its limit (see raise_fused_lds).
 constexpr size_t kFusedLdsPlain = 58u * 1024u;
 constexpr size_t kFusedLdsRaised = 144u * 1024u;
-// Above this many activation elements the quantizer (and what precedes it)
-// runs once in a kernel of its own instead of in every workgroup.
-constexpr int kFuseMaxElems = 16384;
-// The same with a norm (and gate) in front of the quantizer: the prologue is heavier, the crossover
-// earlier (measured at K = 2560: 3 tokens 5.2 us fused against 5.5, 4 tokens 6.5 against 5.7; at
-// K = 6912: 2 tokens 7.4 against 6.7).
-constexpr int kFuseMaxElemsNorm = 9216;
+// (kFuseMaxElems / kFuseMaxElemsNorm, the activation block up to which a forward call stays one kernel: dispatch table)
 
 FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
     FusedPlan pl = {1, 1, 4, 1, false};
@@ -2232,7 +2157,7 @@ FusedPlan plan_fused(int M, int N, int K, int pro = 0) {
         pl.rb = t_tune.fused[0];
         pl.s = t_tune.fused[1];
         pl.upw = t_tune.fused[2];
-    } else if (N / 16 >= 1024 && M <= 4) {
+    } else if (N / 16 >= kSmallWorkgroupBlocks && M <= kDecodeMaxTokens) {
         // Many row blocks (N >= 16384) and few tokens: the matrix is large enough to be bandwidth-bound, and what
         // measured best there is many small workgroups (four or five waves per row block, several
         // workgroups per CU covering each other's latencies) that walk K in two to four rounds:
@@ -2333,7 +2258,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
                                                "bitlinear_fused_kernel<gate+norm>", "bitlinear_fused_kernel<staged int8>"};
     g_last_kernel = kFusedNames[pro];
 #define BITLINEAR_LAUNCH_UVPR(U, V, P, R)                                                                            \
-    hipLaunchKernelGGL((bitlinear_fused_kernel<U, V, P, R>), grid, block, lds, stream, x, wq, M, N, K, pl.rb, pl.s,  \
+    BL_LAUNCH((bitlinear_fused_kernel<U, V, P, R>), grid, block, lds, stream, x, wq, M, N, K, pl.rb, pl.s,  \
                        mode, 1.0f / (float)(K / (pro == 3 ? 16 : 8)), pro == 3 ? ex.act_scale : ex.norm_weight, out, ws, \
                        smap, q_out, s_out, ex)
 #define BITLINEAR_LAUNCH_UVP(U, V, P)              \
@@ -2347,7 +2272,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
         case 1: BITLINEAR_LAUNCH_UVP(U, V, 1); break;               \
         case 2: BITLINEAR_LAUNCH_UVP(U, V, 2); break;               \
         default:                                                    \
-            if (lds > 48u * 1024u) {                                \
+            if (lds > 48u * 1024u && !t_plan.active) {              \
                 const hipError_t e = ex.residual ? raise_fused_lds<U, V, true>() : raise_fused_lds<U, V, false>(); \
                 if (e != hipSuccess) return BITLINEAR_ERR_LAUNCH;   \
             }                                                       \
@@ -2372,7 +2297,7 @@ int launch_fused(const uint16_t* x, const int8_t* packed, uint16_t* out, const u
 #undef BITLINEAR_LAUNCH_UV
 #undef BITLINEAR_LAUNCH_UVP
 #undef BITLINEAR_LAUNCH_UVPR
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    return launch_status();
 }
 
 // Launch shape of bitlinear_solo_kernel: every wave multiplies exactly UPW (<= 8) k-steps, so S * UPW
@@ -2390,9 +2315,9 @@ struct SoloPlan {
 // waves; 5.24 with every wave scanning the 13.8 KB row); two tokens 3.86 -> 3.69 / 3.75 -> 3.62 / 5.14 -> 6.07
 // (not taken) / 5.61 -> 5.21; four tokens 4.16 -> 4.59 (not taken) and 6.81 -> 6.61 at K = 6912.
 bool solo_wanted(int M, int N, int K) {
-    if (M == 1) return K <= 8192;
-    if (K > 4096) return true;  // long rows, two to four tokens
-    return M == 2 && (N / 16) < 432;
+    if (M == 1) return K <= kSoloMaxK;
+    if (K > kSoloLongRowK) return true;  // long rows, two to four tokens
+    return M == 2 && (N / 16) < kManyBlocks;
 }
 
 // The same with an RMSNorm (pro 1) or gate + RMSNorm (pro 2) in front: measured against the shared-prologue kernel
@@ -2402,7 +2327,7 @@ bool solo_norm_wanted(int M, int N, int K, int pro) {
     // measured at one token (shared-prologue kernel -> this one): 3840 x 2560 3.95 -> 3.80 us, 2560 x 2560 with
     // the residual 3.91 -> 3.80, 13824 x 2560 5.44 -> 5.16; 2560 x 6912 with the gate and the residual 5.87 -> 6.12
     // (not taken); two to four tokens 4.7 -> 4.9 and worse (not taken)
-    return M == 1 && pro == 1 && K <= 4096;
+    return M == 1 && pro == 1 && K <= kSoloLongRowK;
 }
 
 SoloPlan plan_solo(int M, int N, int K, int pro = 0, bool has_res = false) {
@@ -2429,10 +2354,10 @@ SoloPlan plan_solo(int M, int N, int K, int pro = 0, bool has_res = false) {
         const int blocks16 = N / 16;
         pl.rb = 1;
         const int order_few[4] = {5, 7, 8, 4}, order_many[4] = {8, 7, 5, 4};
-        const int* order = blocks16 >= 432 ? order_many : order_few;
+        const int* order = blocks16 >= kManyBlocks ? order_many : order_few;
         pl.upw = 0;
         for (int i = 0; i < 4; ++i)
-            if ((units + order[i] - 1) / order[i] <= ((blocks16 >= 432 || units > 64) ? kMaxWaves : 10)) {
+            if ((units + order[i] - 1) / order[i] <= ((blocks16 >= kManyBlocks || units > 64) ? kMaxWaves : 10)) {
                 pl.upw = order[i];
                 break;
             }
@@ -2441,9 +2366,9 @@ SoloPlan plan_solo(int M, int N, int K, int pro = 0, bool has_res = false) {
         // one token and many row blocks: waves of five k-steps that take two or four row blocks each, so that a
         // slice is prepared once for all of them (13824 x 2560: 4.80 -> 4.46 us; with the RMSNorm in front 5.44,
         // the shared-prologue kernel's time, -> 5.16)
-        if (M == 1 && pro <= 1 && !has_res && blocks16 >= 432 && (units + 4) / 5 <= 16 && (pl.coop || pl.vrow == 5)) {
+        if (M == 1 && pro <= 1 && !has_res && blocks16 >= kManyBlocks && (units + 4) / 5 <= 16 && (pl.coop || pl.vrow == 5)) {
             const int s5 = (units + 4) / 5;
-            int rpw = blocks16 >= 864 ? 4 : 2;
+            int rpw = blocks16 >= kFourRowBlocksPerWave ? 4 : 2;
             while (rpw > 1 && (rpw * s5 > kSoloRedSlots || rpw > s5)) --rpw;
             if (rpw > 1) {
                 pl.upw = 5;
@@ -2478,7 +2403,7 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
     if (pro != 0 && (!pl.coop || !norm_weight)) return BITLINEAR_ERR_ARG;
     g_last_kernel = pro == 0 ? "bitlinear_solo_kernel" : (pro == 1 ? "bitlinear_solo_kernel<norm>" : "bitlinear_solo_kernel<gate+norm>");
 #define BITLINEAR_LAUNCH_SOLO_W(U, V, T, C, P, R, W)                                                                      \
-    hipLaunchKernelGGL((bitlinear_solo_kernel<U, V, T, C, P, R, W>), grid, block, 0, stream, x, wq, M, N, K, rb_map, pl.s, \
+    BL_LAUNCH((bitlinear_solo_kernel<U, V, T, C, P, R, W>), grid, block, 0, stream, x, wq, M, N, K, rb_map, pl.s, \
                        slot_rows, norm_weight, ws, out, residual, eps, q_out, s_out, acc_out)
 #define BITLINEAR_LAUNCH_SOLO_P(U, V, T, C, P, R) BITLINEAR_LAUNCH_SOLO_W(U, V, T, C, P, R, 1)
 #define BITLINEAR_LAUNCH_SOLO(U, V, T, C) BITLINEAR_LAUNCH_SOLO_P(U, V, T, C, 0, false)
@@ -2495,7 +2420,7 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
             if (pl.rpw == 2) { BITLINEAR_LAUNCH_SOLO_RW(5, 2); } else if (pl.rpw == 3) { BITLINEAR_LAUNCH_SOLO_RW(5, 3); } else { BITLINEAR_LAUNCH_SOLO_RW(5, 4); }
         }
 #undef BITLINEAR_LAUNCH_SOLO_RW
-        return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+        return launch_status();
     }
     // norm / gate prologues: the exchanging variant only, with or without the residual epilogue
 #define BITLINEAR_LAUNCH_SOLO_N(U, T)                                        \
@@ -2517,7 +2442,7 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
             case 7: BITLINEAR_LAUNCH_SOLO_NU(7); break;
             default: BITLINEAR_LAUNCH_SOLO_NU(8); break;
         }
-        return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+        return launch_status();
     }
 #define BITLINEAR_LAUNCH_SOLO_U(U)                                      \
     if (pl.coop) {                                                      \
@@ -2547,7 +2472,7 @@ int launch_solo(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t*
 #undef BITLINEAR_LAUNCH_SOLO
 #undef BITLINEAR_LAUNCH_SOLO_P
 #undef BITLINEAR_LAUNCH_SOLO_W
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    return launch_status();
 }
 
 // Launch shape of gemv_i2_solo_kernel (up to 16 tokens): one row block per group of S waves, UPW k-steps per wave
@@ -2578,7 +2503,7 @@ ProdPlan plan_prod_solo(int M, int N, int K) {
         pl.s = (units + pl.upw - 1) / pl.upw;
         // measured at 13824 x 2560: up to four tokens two row blocks per wave (4.19 / 4.22 / 4.33 us at one / two /
         // four tokens, 4.39 / 4.41 / 4.49 with four), from eight tokens on four (4.62 against 4.67; 5.15 against 5.78 at 16)
-        if (blocks16 >= 432) pl.rpw = (blocks16 >= 864 && M > 4) ? 4 : 2;
+        if (blocks16 >= kManyBlocks) pl.rpw = (blocks16 >= kFourRowBlocksPerWave && M > kDecodeMaxTokens) ? 4 : 2;
     }
     if (t_tune.solo_rpw >= 1) pl.rpw = t_tune.solo_rpw;
     if (pl.rpw == 3) pl.rpw = 2;
@@ -2600,7 +2525,7 @@ int launch_prod_solo(const int8_t* act, const int8_t* packed, uint16_t* out, int
     const int rb_map = 1 | (int)(rule.map << 8);
     g_last_kernel = "gemv_i2_solo_kernel";
 #define BITLINEAR_LAUNCH_PS(U, W, R)                                                                               \
-    hipLaunchKernelGGL((gemv_i2_solo_kernel<U, W, R>), grid, block, 0, stream, act, wq, M, N, K, rb_map, pl.s, slot_rows, \
+    BL_LAUNCH((gemv_i2_solo_kernel<U, W, R>), grid, block, 0, stream, act, wq, M, N, K, rb_map, pl.s, slot_rows, \
                        s, ws, out, residual, acc_out)
 #define BITLINEAR_LAUNCH_PS_W(U, W)         \
     if (residual) BITLINEAR_LAUNCH_PS(U, W, true); \
@@ -2618,7 +2543,7 @@ int launch_prod_solo(const int8_t* act, const int8_t* packed, uint16_t* out, int
 #undef BITLINEAR_LAUNCH_PS_U
 #undef BITLINEAR_LAUNCH_PS_W
 #undef BITLINEAR_LAUNCH_PS
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    return launch_status();
 }
 
 int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
@@ -2631,7 +2556,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // the large tile double-buffers 2 x 128 rows x 272 bytes = 68 KiB of LDS (so do four groups of the
     // small one): above the 64 KiB a kernel gets without asking (a host-side attribute, set once per process)
     static OncePerDevice lds_limit_raised;
-    const hipError_t lds_err = lds_limit_raised.run([] {
+    const hipError_t lds_err = t_plan.active ? hipSuccess : lds_limit_raised.run([] {
         hipError_t e = hipFuncSetAttribute((const void*)gemm_i2_prefill_kernel<4, 2, 1>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 128 * kPfRowBytes);
         if (e == hipSuccess)
@@ -2655,11 +2580,11 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // (beyond the few-tile range the wide tile: against 64 x 128 it measured level or ahead from 330 tiles on --
     // 2560 x 6912 at M = 1536 31.7 -> 29.2 us, 2560 x 2560 there 14.3 -> 13.6, elsewhere within 2 %)
     const long long wide_tiles = (long long)((N + 255) / 256) * ((M + 63) / 64);
-    int tile = ((N >= 8192 && M >= 512) || narrow_tiles > kPrefillFewTiles) ? 2 : 4;
+    int tile = ((N >= kPrefillWideN && M >= kPrefillWideMinTokens) || narrow_tiles > kPrefillFewTiles) ? 2 : 4;
     // 64 x 256 tiles run three workgroups per CU (768 at a time), 128 x 256 tiles two (512): with a little more than
     // one full round of the former, one round of the latter finishes earlier (13824 x 2560 at M = 1024: 864 tiles,
     // 46.5 -> 42.3 us; 3840 x 2560 at M = 4096: 960 tiles, 45.1 -> 44.1)
-    if (tile == 2 && wide_tiles > 768 && wide_tiles <= 1024) tile = 1;
+    if (tile == 2 && wide_tiles > kPrefillRound64 && wide_tiles <= kPrefillRound128) tile = 1;
     if (t_tune.path == 5) tile = t_tune.prefill_big;
     // groups of waves that split a tile's K between them (small tiles only): while the small tiles
     // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
@@ -2674,15 +2599,15 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // between half a tile and about one tile of 64 x 128 per CU: those tiles, with two groups of waves each
     // (2560 x 6912: M = 512 19.1 -> 17.3 us, M = 640 20.5 -> 17.7, M = 768 22.1 -> 20.0; 2560 x 2560: M = 640
     // 10.2 -> 9.5; 3840 x 2560: M = 384 10.0 -> 9.5, M = 512 9.7 -> 9.3)
-    if (t_tune.path != 5 && tile == 4 && narrow_tiles > 128 && narrow_tiles <= 256) {
+    if (t_tune.path != 5 && tile == 4 && narrow_tiles > kPrefillOnePerCuMin && narrow_tiles <= kPrefillOnePerCuMax) {
         tile = 0;
         ks = 2;
     }
     // about one 64 x 256 tile per CU: those tiles, two groups of waves each (2560 x 6912: M = 1024 25.9 -> 23.4 us,
     // M = 1536 29.2 -> 27.9; 13824 x 2560 at M = 256 15.8 -> 14.3; 2560 x 2560 at M = 1280 13.6 -> 13.1; with 320
     // tiles 42.6 -> 49.4: not taken; at K = 2560 the 32 x 128 tiles stay ahead up to 330 of the 64 x 128 kind)
-    if (t_tune.path != 5 && (tile == 2 || (tile == 4 && K >= kPrefillSplit4MinK)) && wide_tiles > 128 && wide_tiles <= 256 &&
-        narrow_tiles > 256) {
+    if (t_tune.path != 5 && (tile == 2 || (tile == 4 && K >= kPrefillSplit4MinK)) && wide_tiles > kPrefillOnePerCuMin &&
+        wide_tiles <= kPrefillOnePerCuMax && narrow_tiles > kPrefillOnePerCuMax) {
         tile = 2;
         ks = 2;
     }
@@ -2714,7 +2639,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     if (seg_cols > 65535 || (units + 7) / 8 > 65535) return BITLINEAR_ERR_SHAPE;
     const dim3 grid(8 * band, seg_cols, (units + 7) / 8);
 #define BITLINEAR_LAUNCH_PF(MT_, NT_, KS_)                                                                          \
-    hipLaunchKernelGGL((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
+    BL_LAUNCH((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
                        act, wq, M, N, K, units, cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual)
     if (tile == 4) {
         if (ks == 4) {
@@ -2740,7 +2665,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
         BITLINEAR_LAUNCH_PF(2, 1, 1);
     }
 #undef BITLINEAR_LAUNCH_PF
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    return launch_status();
 }
 
 // Streaming kernel: applicability and launch.  D (loads in flight per lane) is chosen so that the
@@ -2793,9 +2718,9 @@ int launch_stream(const StreamProblem* probs, int nprob, int M, int N, int K, co
     g_last_kernel = "gemv_i2_stream_kernel";
 #define BITLINEAR_LAUNCH_STREAM(DD)                                                                      \
     if (compute)                                                                                         \
-        hipLaunchKernelGGL((gemv_i2_stream_kernel<DD, true>), grid, block, lds, stream, a, sink);        \
+        BL_LAUNCH((gemv_i2_stream_kernel<DD, true>), grid, block, lds, stream, a, sink);        \
     else                                                                                                 \
-        hipLaunchKernelGGL((gemv_i2_stream_kernel<DD, false>), grid, block, lds, stream, a, sink)
+        BL_LAUNCH((gemv_i2_stream_kernel<DD, false>), grid, block, lds, stream, a, sink)
     switch (depth) {
         case 4: BITLINEAR_LAUNCH_STREAM(4); break;
         case 6: BITLINEAR_LAUNCH_STREAM(6); break;
@@ -2805,7 +2730,7 @@ int launch_stream(const StreamProblem* probs, int nprob, int M, int N, int K, co
         default: BITLINEAR_LAUNCH_STREAM(5); break;
     }
 #undef BITLINEAR_LAUNCH_STREAM
-    return hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH;
+    return launch_status();
 }
 
 int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
@@ -2819,7 +2744,7 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
         // run once per 16 tokens and re-reading the weights from L2 (about 1.45 TB/s measured),
         // finishes earlier.  Both estimates in microseconds, fitted to measurements at the 2B shapes.
         bool gemm = true;
-        if (M <= 256 && t_tune.path == 0) {
+        if (M <= kSplitKMaxTokens && t_tune.path == 0) {
             const double groups = (M + 15) / 16;
             const double splitk_us = 3.5 + groups * ((double)N * K / 4.0) / 1.45e6;
             const double tiles = ((N + 127) / 128) * (double)((M + 63) / 64);
@@ -2851,9 +2776,9 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // at sixteen; 2560 x 6912: 4.90 -> 4.71 and 6.11 -> 5.89); elsewhere the staged kernel stays (2.89 against 2.95
     // at 3840 x 2560 and 3.65 against 4.06 at 2560 x 6912, one token)
     // (from 1024 row blocks on the staged kernel's many small workgroups stay: 20480 x 3200 5.0 us against 5.9)
-    const bool prod_solo_wanted = t_tune.prod_solo == 1 || (t_tune.prod_solo == 0 && t_tune.staged == 0 && ((N / 16) >= 432 || M > kDecodeMaxTokens) &&
-                                                            (N / 16) < 1024);
-    if (prod_solo_wanted && t_tune.path != 1 && t_tune.path != 2 && M <= 16) {
+    const bool prod_solo_wanted = t_tune.prod_solo == 1 || (t_tune.prod_solo == 0 && t_tune.staged == 0 && ((N / 16) >= kManyBlocks || M > kDecodeMaxTokens) &&
+                                                            (N / 16) < kSmallWorkgroupBlocks);
+    if (prod_solo_wanted && t_tune.path != 2 && M <= 16) {
         const ProdPlan pp = plan_prod_solo(M, N, K);
         if (pp.ok && slot_rule(smap, N).ok)
             return launch_prod_solo(act, packed, out, acc_out, out ? s : (const uint16_t*)packed, out ? ws : (const uint16_t*)packed,
@@ -2862,23 +2787,17 @@ int launch_gemv(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t*
     // (The accumulator export takes the same kernel choice as the drop-in call, so what the parity
     // tests read is what the drop-in entry computes.  Without an output there are no scales: the
     // kernel's unconditional scale requests then go to an address that exists.)
-    if (t_tune.staged != 2 && t_tune.path != 1 && t_tune.path != 2) {
+    if (t_tune.staged != 2 && t_tune.path != 2) {
         const FusedPlan pl = plan_fused(M, N, K, 3);
         // measured: up to 4 tokens staging always wins (2.8-4.5 us against 3.1-5.1 at the 2B shapes);
         // beyond, it pays once a workgroup shares the rows between two or more row blocks
-        const bool wanted = t_tune.staged == 1 || M <= kDecodeMaxTokens || (N / 16) >= 432;
+        const bool wanted = t_tune.staged == 1 || M <= kDecodeMaxTokens || (N / 16) >= kManyBlocks;
         if (pl.ok && wanted)
             return launch_fused((const uint16_t*)act, packed, out, out ? ws : (const uint16_t*)packed, smap, nullptr,
                                 nullptr, FusedExtras{nullptr, residual, 0.0f, 0, out ? s : (const uint16_t*)packed, acc_out},
                                 M, N, K, 0, pl, stream);
     }
-    if (residual) return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
-    const bool decode_fits = M <= kDecodeMaxTokens && (size_t)M * K <= (size_t)kDecodeMaxLdsBytes;
-    // The one-wave-per-row-block kernel pays off once there are enough row
-    // blocks to fill every SIMD; below that, splitting K across waves wins.
-    const bool many_rows = (N / 16) >= 512;
-    if (decode_fits && t_tune.path != 2 && (many_rows || t_tune.path == 1)) return launch_decode(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
-    return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream);
+    return launch_splitk(act, packed, out, acc_out, s, ws, smap, M, N, K, stream, residual);
 }
 
 ScaleMap equal_slots(int N, int ws_num) {
@@ -3051,7 +2970,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.decode_waves = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = g.prod_solo = 0;
+        g.path = g.waves = g.upw = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = g.prod_solo = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -3095,12 +3014,6 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         g.solo = a;
         g.solo_s = b;
         g.solo_upw = c;
-        return set_status(BITLINEAR_OK);
-    }
-    if (kernel == 1) {
-        if (a < 1 || a > kDecodeMaxWaves) return set_status(BITLINEAR_ERR_ARG);
-        g.path = 1;
-        g.decode_waves = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 2) {
@@ -3277,7 +3190,7 @@ static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t*
         const int per_lane = (K / 8 + 63) / 64;
         const dim3 grid((M + 3) / 4, 1, 1), block(256, 1, 1);
 #define BITLINEAR_LAUNCH_QR(MODE_, V_) \
-    hipLaunchKernelGGL((quant_absmax_rows_kernel<MODE_, V_>), grid, block, 0, (hipStream_t)stream, x, q, s, M, K, rowsum)
+    BL_LAUNCH((quant_absmax_rows_kernel<MODE_, V_>), grid, block, 0, (hipStream_t)stream, x, q, s, M, K, rowsum)
 #define BITLINEAR_LAUNCH_QR_V(V_)          \
     if (mode == 0) BITLINEAR_LAUNCH_QR(0, V_); \
     else BITLINEAR_LAUNCH_QR(1, V_)
@@ -3286,16 +3199,16 @@ static int quant_absmax_impl(const uint16_t* x, int8_t* q, uint16_t* s, int32_t*
         else { BITLINEAR_LAUNCH_QR_V(8); }
 #undef BITLINEAR_LAUNCH_QR_V
 #undef BITLINEAR_LAUNCH_QR
-        return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
+        return set_status(launch_status());
     }
     int threads = kQuantThreads;
     while (threads < kQuantMaxThreads && K > threads * kQuantRegVecs * 8) threads *= 2;
     const dim3 grid(M, 1, 1), block(threads, 1, 1);
     if (mode == 0)
-        hipLaunchKernelGGL(quant_absmax_kernel<0>, grid, block, 0, (hipStream_t)stream, x, q, s, K, rowsum);
+        BL_LAUNCH(quant_absmax_kernel<0>, grid, block, 0, (hipStream_t)stream, x, q, s, K, rowsum);
     else
-        hipLaunchKernelGGL(quant_absmax_kernel<1>, grid, block, 0, (hipStream_t)stream, x, q, s, K, rowsum);
-    return set_status(hipGetLastError() == hipSuccess ? BITLINEAR_OK : BITLINEAR_ERR_LAUNCH);
+        BL_LAUNCH(quant_absmax_kernel<1>, grid, block, 0, (hipStream_t)stream, x, q, s, K, rowsum);
+    return set_status(launch_status());
 }
 
 // seg_ends == nullptr: the reference's equal slots (bitnet_kernels.h:80); otherwise the caller's segments
@@ -3439,24 +3352,24 @@ static int norm_forward_impl(const uint16_t* x, const uint16_t* norm_weight, flo
     if (K > kPreThreads * kPreVecs * 8) return set_status(BITLINEAR_ERR_SHAPE);
     // very many rows, no gate, short rows: a wave per row (norm + product at K = 2560: 32.2 -> 30.1 us at 2048 rows,
     // 53.6 -> 48.7 at 4096; below 1024 rows 0.2-0.9 us behind, with the gate at K = 6912 4-7 us behind: not taken)
-    if (M >= 1024 && !glu && K <= 8 * 64 * 8) {
+    if (M >= kNormRowsPerWaveMinRows && !glu && K <= 8 * 64 * 8) {
         const int per_lane = (K / 8 + 63) / 64;
         const dim3 rgrid((M + 3) / 4, 1, 1), rblock(256, 1, 1);
 #define BITLINEAR_LAUNCH_NR(P, V) \
-    hipLaunchKernelGGL((norm_quant_rows_kernel<P, V>), rgrid, rblock, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, M, K, mode)
+    BL_LAUNCH((norm_quant_rows_kernel<P, V>), rgrid, rblock, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, M, K, mode)
 #define BITLINEAR_LAUNCH_NR_V(V) BITLINEAR_LAUNCH_NR(1, V)
         if (per_lane <= 2) { BITLINEAR_LAUNCH_NR_V(2); }
         else if (per_lane <= 5) { BITLINEAR_LAUNCH_NR_V(5); }
         else { BITLINEAR_LAUNCH_NR_V(8); }
 #undef BITLINEAR_LAUNCH_NR_V
 #undef BITLINEAR_LAUNCH_NR
-        if (hipGetLastError() != hipSuccess) return set_status(BITLINEAR_ERR_LAUNCH);
+        if (launch_status() != BITLINEAR_OK) return set_status(BITLINEAR_ERR_LAUNCH);
         return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream, residual));
     }
     const dim3 grid(M, 1, 1), block(kPreThreads, 1, 1);
     const int per_thread = (K / 8 + kPreThreads - 1) / kPreThreads;
 #define BITLINEAR_LAUNCH_PRE(P, V) \
-    hipLaunchKernelGGL((norm_quant_kernel<P, V>), grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode)
+    BL_LAUNCH((norm_quant_kernel<P, V>), grid, block, 0, (hipStream_t)stream, x, norm_weight, eps, q_ws, s_ws, K, mode)
 #define BITLINEAR_LAUNCH_PRE_V(V)    \
     if (glu)                         \
         BITLINEAR_LAUNCH_PRE(2, V);  \
@@ -3473,8 +3386,34 @@ static int norm_forward_impl(const uint16_t* x, const uint16_t* norm_weight, flo
     }
 #undef BITLINEAR_LAUNCH_PRE_V
 #undef BITLINEAR_LAUNCH_PRE
-    if (hipGetLastError() != hipSuccess) return set_status(BITLINEAR_ERR_LAUNCH);
+    if (launch_status() != BITLINEAR_OK) return set_status(BITLINEAR_ERR_LAUNCH);
     return set_status(launch_gemv(q_ws, packed, output0, nullptr, s_ws, ws, sm, M, N, K, (hipStream_t)stream, residual));
+}
+
+int bitlinear_plan_name(int entry, int M, int N, int K, char* buf, int buflen) {
+    if (!buf || buflen < 1) return set_status(BITLINEAR_ERR_NULL);
+    buf[0] = 0;
+    if (entry < 0 || entry > 4) return set_status(BITLINEAR_ERR_ARG);
+    // operands of a planning call are never dereferenced, on the host or anywhere: any aligned address does
+    uint16_t* const h = reinterpret_cast<uint16_t*>((uintptr_t)0x100000);
+    int8_t* const b = reinterpret_cast<int8_t*>((uintptr_t)0x100000);
+    t_plan.active = true;
+    t_plan.text.clear();
+    int st = BITLINEAR_OK;
+    switch (entry) {
+        case 0:
+            bitlinear_int8xint2(b, b, h, h, h, M, N, K, nullptr);
+            st = g_status;
+            break;
+        case 1: st = forward_impl(h, b, h, nullptr, h, b, h, M, N, K, 0, nullptr); break;
+        default:
+            st = norm_forward_impl(h, h, 1e-5f, entry == 4 ? 1 : 0, b, h, entry >= 3 ? h : nullptr, h, b, h, M, N, K, 0, nullptr,
+                                   nullptr, 0);
+            break;
+    }
+    t_plan.active = false;
+    snprintf(buf, (size_t)buflen, "%s", t_plan.text.c_str());
+    return set_status(st);
 }
 
 }  // extern "C"

@@ -1,20 +1,9 @@
-// Decode-step attention for the BitNet decoder: rotary embedding of q and k,
-// KV-cache write and grouped-query attention of one new token per sequence,
-// in one kernel.  It is the caller-side glue between the wqkv and wo BitLinear
-// calls (gpu/model.py:128-157 of the reference, which uses xformers'
-// rope_padded and flash attention there); a floating-point kernel, checked
-// against a torch fp32 restatement within a stated tolerance.
-//
-// One workgroup per (kv head, sequence, split of the cached positions): the
-// g = n_heads / n_kv_heads query heads that share the kv head are processed
-// together so every cached K / V row is read once; splitting the positions
-// over several workgroups spreads the cache read over as many CUs (one CU
-// alone pulls well under 100 GB/s).  With more than one split every workgroup
-// leaves (unnormalised output, max, sum of exponentials) in a workspace and
-// the last one to finish -- an atomic counter per (sequence, kv head), reset
-// by that last workgroup -- merges them.  Phases: (1) rope + cache write, rotated q kept in LDS as
-// bf16; (2) scores with bf16 MFMA, 16 cached positions per wave and step; (3) softmax per head; (4) P.V with the positions split
-// over the waves and combined through LDS.
+// Host entry points of the decode-step attention (rotary embedding of q and k, KV-cache write and
+// grouped-query attention of one new token per sequence, in one kernel: the caller-side glue between
+// the wqkv and wo BitLinear calls, gpu/model.py:128-157 of the reference, which uses xformers'
+// rope_padded and flash attention there; the kernel itself lives in attn_prefill.hip), and the final
+// RMSNorm + bf16 LM head + greedy token.  Floating-point kernels, checked against torch fp32
+// restatements within stated tolerances.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -70,324 +59,7 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
 // Workspace record of one (sequence, kv head, split): G heads x (128 unnormalised outputs,
 // running maximum, sum of exponentials)
 constexpr int kRecFloats = kHeadDim + 2;
-constexpr int kMaxSplits = 8;
-
-template <int G>  // query heads per kv head
-__global__ __launch_bounds__(kAttnMaxThreads) void attn_decode_kernel(
-    const uint16_t* __restrict__ qkv, uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
-    const int64_t* __restrict__ positions, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    uint16_t* __restrict__ out, float* workspace, int* counters, int S, int span, int n_heads, int n_kv_heads) {
-    extern __shared__ float sc[];  // [G][span] scores, then probabilities; then part[nwaves][G][kHeadDim]
-    __shared__ __attribute__((aligned(16))) uint16_t qb[G][kHeadDim];  // rotated q as bf16
-    __shared__ __attribute__((aligned(16))) uint16_t knew[kHeadDim];   // rotated k of the new token
-    __shared__ __attribute__((aligned(16))) uint16_t vnew[kHeadDim];
-    __shared__ float red_m[G], red_l[G];
-    __shared__ int is_last;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // on the scalar unit: loops over a wave's positions are uniform
-    const int nthreads = blockDim.x;
-    const int nwaves = nthreads >> 6;
-    const int kvh = blockIdx.x;
-    const int b = blockIdx.y;
-    const int sp = blockIdx.z;
-    const int nsplit = gridDim.z;
-    const int row_elems = (n_heads + 2 * n_kv_heads) * kHeadDim;
-    const uint16_t* row = qkv + (size_t)b * row_elems;
-    const size_t cache_row = (size_t)n_kv_heads * kHeadDim;  // elements between positions
-    uint16_t* ck = cache_k + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
-    uint16_t* cv = cache_v + ((size_t)b * S * n_kv_heads + kvh) * kHeadDim;
-    const int c = lane & 15, g4 = lane >> 4;
-    // Cached rows are read through buffer descriptors that span this (sequence, kv head)'s rows:
-    // 32-bit byte offsets with the uniform part formed on the scalar unit, and a row past the end
-    // of the cache is out of range and reads as zero (such rows are ignored anyway), so no index
-    // needs clamping.
-    const int row_bytes = n_kv_heads * kHeadDim * 2;  // bytes between positions
-    const int cache_bytes = (S - 1) * row_bytes + kHeadDim * 2;
-    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)ck, 0, cache_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cv, 0, cache_bytes, 0x00020000);
-    const int k_lane_off = c * row_bytes + g4 * 16;  // K: lane = (position c of a block of 16, 16-byte piece g4 of a 64-byte step)
-    const int v_lane_off = lane * 4;                 // V: lane = dims 2 * lane, 2 * lane + 1 of one position
-    // This split owns positions [lo, lo + span): a fixed slice of the cache, whatever the current
-    // position is, so its rows can be requested before the position is known.  span % 16 == 0.
-    const int lo = sp * span;
-    // Behind the scores: one 4 KB region per wave.  During P.V it stages the wave's 16 V rows of a
-    // round (so that the loop over them need not be unrolled), afterwards it holds the wave's partial
-    // outputs [G][128] for the reduction over the waves.
-    constexpr int kWaveRegion = 1024;  // floats
-    float* part = sc + (size_t)G * span;
-    uint32_t* vst = (uint32_t*)part + wave * kWaveRegion;
-
-    // The kernel is a chain of memory round trips of a microsecond or more each, so everything
-    // that does not depend on anything else is requested first and at once: the position, this
-    // token's q / k / v, and the first round of cached K and V rows of the slice (row indices
-    // clamped to the cache; rows past the current position are ignored later, the row of the new
-    // token itself is patched in from LDS).
-    constexpr int R = 2;   // blocks of 16 positions per wave and round (K)
-    constexpr int U = 16;  // positions per wave and round (V)
-    constexpr int kItems = (G + 2) * (kHeadDim / 2);           // (head, pair) items of phase 1
-    constexpr int kIters = (kItems + kAttnMinThreads - 1) / kAttnMinThreads;
-    uint32_t praw[kIters];
-#pragma unroll
-    for (int u = 0; u < kIters; ++u) {
-        const int it = tid + u * nthreads;
-        const int hh = it / (kHeadDim / 2);
-        const int i = it - hh * (kHeadDim / 2);
-        const int src = hh < G ? (kvh * G + hh) * kHeadDim : (hh == G ? (n_heads + kvh) : (n_heads + n_kv_heads + kvh)) * kHeadDim;
-        praw[u] = *(const uint32_t*)(row + (it < kItems ? src + 2 * i : 0));
-    }
-    v4u kb[R][4];
-    // Rows beyond this split's slice belong to other splits: their requests get an offset past the
-    // end of the descriptor instead, which costs no memory access (with eight waves a round covers
-    // 256 K rows and 128 V rows, a slice is often 96 or fewer).
-    constexpr int kPastEnd = 0x7fff0000;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int blk = wave * 16 + r * nwaves * 16;
-        const int off = blk < span ? k_lane_off + (lo + blk) * row_bytes : kPastEnd;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) kb[r][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
-    }
-    uint32_t vr[U];
-#pragma unroll
-    for (int j = 0; j < U; ++j) {
-        const int rel = wave + j * nwaves;
-        vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, rel < span ? v_lane_off + (lo + rel) * row_bytes : kPastEnd, 0, 0);
-    }
-    // A position outside the cache would index the rope tables and the cache rows out of range;
-    // the host cannot see this device-side value, so it is clamped here (the result for such a
-    // sequence is then meaningless, but nothing outside the buffers is touched).
-    const int64_t p_raw = positions[b];
-    const int p = __builtin_amdgcn_readfirstlane(p_raw < 0 ? 0 : (p_raw >= (int64_t)S ? S - 1 : (int)p_raw));
-    const int hi = (lo + span) < (p + 1) ? (lo + span) : (p + 1);  // this split's positions are [lo, hi)
-    const bool owns_new = p >= lo && p < lo + span;
-    // Splits whose slice starts beyond the current position have nothing to do and take no part in
-    // the combination: nact splits are active (the comparison chain is p / span + 1 without a
-    // division), and a single active split writes the output itself.  They leave after the first
-    // barrier, not here: a branch on the position in front of phase 1 would make the compiler move
-    // the cache-row loads above behind it, i.e. behind the wait for the position, and serialise two
-    // memory round trips.
-    int nact = 1;
-#pragma unroll
-    for (int k = 1; k < kMaxSplits; ++k) nact += (k < nsplit && p >= k * span) ? 1 : 0;
-    const bool active = sp < nact;
-
-    // (1) rope on adjacent pairs, in fp32, results rounded to bf16.  Every split needs q; the
-    // split that holds position p also rotates k, keeps k and v of the new token in LDS and
-    // writes them to the cache.
-#pragma unroll
-    for (int u = 0; u < kIters; ++u) {
-        const int it = tid + u * nthreads;
-        const int hh = it / (kHeadDim / 2);
-        const int i = it - hh * (kHeadDim / 2);
-        if (it < kItems && active) {
-            if (hh <= G) {
-                if (hh < G || owns_new) {
-                    const float a = bf16f(praw[u] & 0xffffu), cc = bf16f(praw[u] >> 16);
-                    const float cs = cos_t[(size_t)p * (kHeadDim / 2) + i], sn = sin_t[(size_t)p * (kHeadDim / 2) + i];
-                    const uint32_t rot = (uint32_t)to_bf16(a * cs - cc * sn) | ((uint32_t)to_bf16(a * sn + cc * cs) << 16);
-                    if (hh < G) {
-                        *(uint32_t*)(&qb[hh][2 * i]) = rot;
-                    } else {
-                        *(uint32_t*)(&knew[2 * i]) = rot;
-                        *(uint32_t*)(ck + (size_t)p * cache_row + 2 * i) = rot;
-                    }
-                }
-            } else if (owns_new) {
-                *(uint32_t*)(&vnew[2 * i]) = praw[u];
-                *(uint32_t*)(cv + (size_t)p * cache_row + 2 * i) = praw[u];
-            }
-        }
-    }
-    __syncthreads();
-    if (!active) return;
-
-    // (2) scores with bf16 MFMA 16x16x32 (products of bf16 values are exact in fp32, sums are
-    // fp32): A = the rotated q rows (heads, zero rows beyond G), B = 16 cached positions; a lane
-    // supplies 8 consecutive dims (lane / 16 picks which 8 of a 32-dim step) of row / position
-    // lane % 16, i.e. one 16-byte piece of a K row.  Four steps cover the 128 dims.
-    const float scale = 0.08838834764831845f;  // 128^-0.5
-    {
-        v8bf qa[4];
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            uint4 t = make_uint4(0, 0, 0, 0);
-            if (c < G) t = *(const uint4*)(&qb[c][kk * 32 + g4 * 8]);
-            qa[kk] = __builtin_bit_cast(v8bf, t);
-        }
-        for (int s0 = lo + wave * 16; s0 < hi; s0 += nwaves * 16 * R) {
-            if (s0 != lo + wave * 16) {  // later rounds of a long slice
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const int blk = s0 - lo + r * nwaves * 16;
-                    const int off = blk < span ? k_lane_off + (lo + blk) * row_bytes : kPastEnd;
-#pragma unroll
-                    for (int kk = 0; kk < 4; ++kk) kb[r][kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, off + kk * 64, 0, 0);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int s = s0 + r * nwaves * 16 + c;
-                v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int kk = 0; kk < 4; ++kk) {
-                    v4u kv = kb[r][kk];
-                    if (s == p) kv = *(const v4u*)(&knew[kk * 32 + g4 * 8]);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[kk], __builtin_bit_cast(v8bf, kv), acc, 0, 0, 0);
-                }
-                // result lane: position c, heads 4 * g4 + j in register j
-                if (s < hi) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (4 * g4 + j < G) sc[(size_t)(4 * g4 + j) * span + (s - lo)] = acc[j] * scale;
-                }
-            }
-        }
-    }
-    __syncthreads();
-
-    // (3) exp(score - max) over this split's positions, one head per wave at a time
-    for (int hh = wave; hh < G; hh += nwaves) {
-        float* srow = sc + (size_t)hh * span;
-        float mx = -INFINITY;
-        for (int s = lane; s < hi - lo; s += 64) mx = fmaxf(mx, srow[s]);
-        mx = wave_max_f32(mx);
-        float sum = 0.0f;
-        for (int s = lane; s < hi - lo; s += 64) {
-            const float e = __expf(srow[s] - mx);
-            srow[s] = e;
-            sum += e;
-        }
-        sum = wave_sum_f32(sum);
-        if (lane == 0) {
-            red_m[hh] = mx;
-            red_l[hh] = sum;
-        }
-    }
-    __syncthreads();
-
-    // (4) o[hh][d] = sum_s e[hh][s] * v[s][d]: every wave takes positions lo + wave, + W, ... for all G
-    // heads at once (a V row is read once), a lane owns dims 2*lane, 2*lane+1
-    float a0[G], a1[G];
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) a0[hh] = a1[hh] = 0.0f;
-    // Straight-line code that runs once costs instruction fetch on top of its execution (about
-    // twice as much per instruction as code in a loop), and 16 unrolled positions x G heads were
-    // the longest stretch of it in this kernel: the rows go through the wave's LDS region and a
-    // short loop walks them.
-    const int nw_shift = nwaves == 8 ? 3 : 2;  // nwaves is 4 or 8
-    for (int s0 = lo + wave; s0 < hi; s0 += nwaves * U) {
-        if (s0 != lo + wave) {
-#pragma unroll
-            for (int j = 0; j < U; ++j) {
-                const int rel = s0 - lo + j * nwaves;
-                vr[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(v_rsrc, rel < span ? v_lane_off + (lo + rel) * row_bytes : kPastEnd, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < U; ++j) vst[j * 64 + lane] = vr[j];
-        // same wave writes and reads: LDS operations of a wave complete in order
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const int left = (hi - s0 + nwaves - 1) >> nw_shift;  // positions of this wave from s0 on
-        const int cnt = left < U ? left : U;
-#pragma unroll 2
-        for (int j = 0; j < cnt; ++j) {
-            const int s = s0 + j * nwaves;
-            const uint32_t* src = s == p ? (const uint32_t*)vnew + lane : vst + j * 64 + lane;
-            const uint32_t pr = *src;
-            const float v0 = bf16f(pr & 0xffffu), v1 = bf16f(pr >> 16);
-#pragma unroll
-            for (int hh = 0; hh < G; ++hh) {
-                const float pw = sc[(size_t)hh * span + (s - lo)];
-                a0[hh] += pw * v0;
-                a1[hh] += pw * v1;
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) {
-        part[(size_t)wave * kWaveRegion + hh * kHeadDim + 2 * lane] = a0[hh];
-        part[(size_t)wave * kWaveRegion + hh * kHeadDim + 2 * lane + 1] = a1[hh];
-    }
-    __syncthreads();
-
-    uint16_t* orow = out + (size_t)b * n_heads * kHeadDim + (size_t)(kvh * G) * kHeadDim;
-    float* rec = workspace + ((size_t)(b * n_kv_heads + kvh) * nsplit) * G * kRecFloats;
-    for (int hh = wave; hh < G; hh += nwaves) {
-        float o0 = 0.0f, o1 = 0.0f;
-        for (int k = 0; k < nwaves; ++k) {
-            o0 += part[(size_t)k * kWaveRegion + hh * kHeadDim + 2 * lane];
-            o1 += part[(size_t)k * kWaveRegion + hh * kHeadDim + 2 * lane + 1];
-        }
-        if (nact == 1) {
-            const float is = 1.0f / red_l[hh];
-            *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
-        } else {
-            // device-coherent (write-through) stores: the record reaches the point where the other
-            // XCDs' loads see it without a writeback of this XCD's whole L2
-            float* r = rec + ((size_t)sp * G + hh) * kRecFloats;
-            __hip_atomic_store(r + 2 * lane, o0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(r + 2 * lane + 1, o1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (lane == 0) {
-                __hip_atomic_store(r + kHeadDim, red_m[hh], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // -inf: no positions
-                __hip_atomic_store(r + kHeadDim + 1, red_l[hh], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-    }
-    if (nact == 1) return;
-
-    // The last split of this (sequence, kv head) to finish combines the records.  The barrier
-    // waits until every thread's record stores have completed (they are write-through, so
-    // completed = visible device-wide); only then is the arrival counted, with a device-scope
-    // atomic, and the last arrival reads the records with device-coherent loads.  No L2-wide
-    // writeback or invalidate is involved.
-    // (the wait is spelled out: the arrival below must not be counted before this thread's
-    // write-through record stores are acknowledged)
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) {
-        const int done = __hip_atomic_fetch_add(&counters[b * n_kv_heads + kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = done == nact - 1;
-        if (is_last) __hip_atomic_store(&counters[b * n_kv_heads + kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    for (int hh = wave; hh < G; hh += nwaves) {
-        // all records' loads first (independent), then the merge
-        float mk[kMaxSplits], lk[kMaxSplits], p0[kMaxSplits], p1[kMaxSplits];
-#pragma unroll
-        for (int k = 0; k < kMaxSplits; ++k) {
-            const float* r = rec + ((size_t)(k < nact ? k : 0) * G + hh) * kRecFloats;
-            mk[k] = __hip_atomic_load(r + kHeadDim, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            lk[k] = __hip_atomic_load(r + kHeadDim + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            p0[k] = __hip_atomic_load(r + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            p1[k] = __hip_atomic_load(r + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int k = 0; k < kMaxSplits; ++k)
-            if (k < nact) mx = fmaxf(mx, mk[k]);
-        float l = 0.0f, o0 = 0.0f, o1 = 0.0f;
-#pragma unroll
-        for (int k = 0; k < kMaxSplits; ++k) {
-            if (k < nact && lk[k] > 0.0f) {
-                const float w = __expf(mk[k] - mx);
-                l += lk[k] * w;
-                o0 += w * p0[k];
-                o1 += w * p1[k];
-            }
-        }
-        const float is = 1.0f / l;
-        *(uint32_t*)(orow + hh * kHeadDim + 2 * lane) = (uint32_t)to_bf16(o0 * is) | ((uint32_t)to_bf16(o1 * is) << 16);
-    }
-}
-
+constexpr int kMaxSplits = 16;
 
 // ---------------------------------------------------------------------------
 // Final RMSNorm + bf16 LM head + greedy token (gpu/model.py:280-281 followed by
@@ -798,7 +470,6 @@ __global__ __launch_bounds__(kLmFinalThreads) void lm_head_final_kernel(const fl
 }  // namespace
 
 static std::atomic<int> g_attn_threads{0};
-static std::atomic<int> g_attn_kernel{0};  // 0 = built-in choice, 1 = score buffer in LDS + vector-pipe P.V, 2 = everything on the matrix pipe
 
 // in attn_prefill.hip
 int bitnet_attn_decode_flash_launch(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,
@@ -812,13 +483,6 @@ static std::atomic<int> g_attn_spin_limit{-1};  // polls of the merging workgrou
    merge of more than one split give up at once, which is how the failure path is tested) */
 extern "C" int bitnet_attn_decode_set_spin_limit(int polls) {
     g_attn_spin_limit = polls < 0 ? -1 : polls;
-    return 0;
-}
-
-/* tuning override for tests and measurements: which of the two decode-step attention kernels runs */
-extern "C" int bitnet_attn_decode_set_kernel(int which) {
-    if (which < 0 || which > 2) return 1;
-    g_attn_kernel = which;
     return 0;
 }
 
@@ -855,50 +519,22 @@ static int attn_decode_impl(const uint16_t* qkv, uint16_t* cache_k, uint16_t* ca
     if (n_heads % n_kv_heads) return 1;
     const int g = n_heads / n_kv_heads;
     if (g != 1 && g != 2 && g != 4 && g != 8) return 1;
-    const bool flash = g_attn_kernel != 1;  // the built-in choice is the matrix-pipe kernel
-    if (n_splits < 1 || n_splits > (flash ? 16 : kMaxSplits)) return 1;
+    if (n_splits < 1 || n_splits > kMaxSplits) return 1;
     if (!qkv || !cache_k || !cache_v || !positions || !cos_table || !sin_table || !out) return 2;
     if (n_splits > 1 && (!workspace || !counters)) return 2;
     if (((uintptr_t)workspace) & 7u) return 1;
-    // the kernels' 32-bit byte offsets into one sequence's cache (the first blocks requested may lie up to 4096 rows in)
+    // the kernel's 32-bit byte offsets into one sequence's cache (the first blocks requested may lie up to 4096 rows in)
     if ((size_t)((S > 4096 ? S : 4096) + 512) * n_kv_heads * kHeadDim * 2 >= ((size_t)1 << 31)) return 1;
-    const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // a split's share of the cache capacity (kernel 1: its fixed slice)
-    // Eight waves take a slice of up to 128 rows in one round of loads (four waves: 64 rows; a
-    // second round exposes a full memory round trip, about 1 us).  Measured: that wins while every
-    // workgroup has a CU of its own (up to 256 of them); beyond that two 512-thread workgroups
-    // share a CU badly (12.9 -> 16.8 us at 320 workgroups) and 256 threads are the better choice.
-    int threads = (span > 64 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
-    // the matrix-pipe kernel deals blocks of 32 rows to splits and waves: four waves cover a split's share of
-    // up to 128 rows of the capacity in one round (measured at 96 rows: 6.85 us with four waves, 7.12 with
-    // eight; at 272 rows 8.77 / 8.46)
-    if (flash) threads = (span > 128 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
+    const int span = ((S + n_splits - 1) / n_splits + 15) & ~15;  // a split's share of the cache capacity
+    // The kernel deals blocks of 32 rows to splits and waves: four waves cover a split's share of up to 128
+    // rows of the capacity in one round (measured at 96 rows: 6.85 us with four waves, 7.12 with eight; at 272
+    // rows 8.77 / 8.46).  Eight waves while every workgroup has a CU of its own (up to 256 of them); beyond
+    // that two 512-thread workgroups share a CU badly and 256 threads are the better choice.
+    int threads = (span > 128 && (long long)n_kv_heads * B * n_splits <= 256) ? 512 : 256;
     if (const int forced = g_attn_threads.load()) threads = forced;
-    if (flash)
-        return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, rope_rows, out, workspace,
-                                               counters, n_splits, threads, B, S, n_heads, n_kv_heads, g_attn_spin_limit.load(),
-                                               (hipStream_t)stream);
-    const size_t lds = ((size_t)g * span + (size_t)(threads / 64) * 1024) * sizeof(float);  // scores + one 4 KB region per wave
-    if (lds > 96u * 1024u) return 1;
-    const dim3 grid(n_kv_heads, B, n_splits), block(threads, 1, 1);
-#define BITNET_ATTN_LAUNCH(GG)                                                                                        \
-    {                                                                                                                 \
-        static bitnet_host::OncePerDevice raised; /* more than 64 KiB of dynamic LDS has to be asked for */          \
-        if (raised.run([] {                                                                                           \
-                return hipFuncSetAttribute((const void*)attn_decode_kernel<GG>,                                       \
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);                    \
-            }) != hipSuccess)                                                                                         \
-            return 3;                                                                                                 \
-        hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, block, lds, (hipStream_t)stream, qkv, cache_k, cache_v,      \
-                           positions, cos_table, sin_table, out, workspace, counters, S, span, n_heads, n_kv_heads);       \
-    }
-    switch (g) {
-        case 1: BITNET_ATTN_LAUNCH(1) break;
-        case 2: BITNET_ATTN_LAUNCH(2) break;
-        case 4: BITNET_ATTN_LAUNCH(4) break;
-        default: BITNET_ATTN_LAUNCH(8) break;
-    }
-#undef BITNET_ATTN_LAUNCH
-    return hipGetLastError() == hipSuccess ? 0 : 3;
+    return bitnet_attn_decode_flash_launch(qkv, cache_k, cache_v, positions, cos_table, sin_table, rope_rows, out, workspace,
+                                           counters, n_splits, threads, B, S, n_heads, n_kv_heads, g_attn_spin_limit.load(),
+                                           (hipStream_t)stream);
 }
 
 extern "C" int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v, const int64_t* positions,

@@ -263,11 +263,24 @@ int bitlinear_norm_forward_bf16_seg(const uint16_t* x, const uint16_t* norm_weig
                                     int M, int N, int K, int mode, void* stream);
 
 /*
+ * What the library would launch for a call, without launching it (host only:
+ * works without a GPU).  Runs the dispatch code of the entry point itself --
+ * entry 0: bitlinear_int8xint2, 1: bitlinear_forward_bf16 (mode 0, with
+ * workspaces), 2: bitlinear_norm_forward_bf16 (norm), 3: the same with a
+ * residual, 4: with gate and residual -- and writes into buf, for every kernel
+ * of the call in launch order and joined by " + ", the kernel with its template
+ * arguments, the grid, the workgroup size and the dynamic LDS bytes, e.g.
+ * "bitlinear_solo_kernel<5, 1, 1, true, 0, false, 1> grid=(160,1,1) block=512
+ * lds=0".  Returns the status the call itself would return for the shape.
+ * The current bitlinear_set_tuning overrides apply.  No counterpart in the
+ * reference, whose dispatch is a table of ten shapes (bitnet_kernels.cu:4-33).
+ */
+int bitlinear_plan_name(int entry, int M, int N, int K, char* buf, int buflen);
+
+/*
  * Kernel / launch-shape override for tuning runs and tests.  Process-wide;
  * results never depend on it.
  *   kernel 0: built-in choice (other arguments ignored)
- *   kernel 1: decode kernel where it applies (M <= 4, M*K <= 48 KiB) with
- *             a (1..4) 16-row blocks per workgroup
  *   kernel 2: split-K kernel always, a (1..16) waves per workgroup each
  *             keeping one to two rounds of b (1, 2, 4 or 8) 64-wide k-steps in flight
  *             (a = b = 0: the library's own launch shape)

@@ -31,19 +31,17 @@ extern "C" {
  *   workspace float [bitnet_attn_decode_workspace_floats(B, n_heads, n_kv_heads, n_splits)], 8-byte
  *            aligned and zero before the first call that uses it (the calls keep it consistent: every
  *            split's record carries the tag of the call that wrote it, and the tag advances per call)
- *   counters  int [B * n_kv_heads], zero before the first call (every call leaves them zero)
- *   n_splits  1..16 (1..8 with kernel 1) workgroups share the cache rows of one (sequence, kv head): blocks of
- *             32 rows dealt round-robin, so the rows up to the position are spread over all splits whatever
- *             the capacity S is (kernel 1: fixed slices of S / n_splits rows, of which those beyond the
- *             position cost almost nothing); with 1, workspace and counters may be NULL.  Calls that share
- *             a workspace must not overlap in time.  Fastest when B * n_kv_heads * n_splits <= 256 (one
- *             workgroup per CU: the kernel then runs eight waves per workgroup for long caches).
- * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8 (kernel 1 also needs
- * g * (S / n_splits + 16) * 4 bytes + 32 KiB <= 96 KiB of LDS for its scores).  Returns 0, or 1
- * (shape), 2 (null pointer), 3 (launch failed).  Scores and outputs on the bf16 matrix pipe with
- * fp32 accumulation, the probabilities rounded to bf16 in between (kernel 1: fp32 probabilities on
- * the vector pipe); results agree with an fp32 evaluation of the same formula to about 1e-2
- * relative on bf16 outputs.
+ *   counters  int [B * n_kv_heads]: kept in the signature for callers written against earlier versions; the
+ *             kernel does not use it (must be non-NULL when n_splits > 1)
+ *   n_splits  1..16 workgroups share the cache rows of one (sequence, kv head): blocks of 32 rows dealt
+ *             round-robin, so the rows up to the position are spread over all splits whatever the capacity
+ *             S is; with 1, workspace and counters may be NULL.  Calls that share a workspace must not
+ *             overlap in time.  Fastest when B * n_kv_heads * n_splits <= 256 (one workgroup per CU: the
+ *             kernel then runs eight waves per workgroup for long caches).
+ * head_dim must be 128, g = n_heads / n_kv_heads one of 1, 2, 4, 8.  Returns 0, or 1 (shape), 2 (null
+ * pointer), 3 (launch failed).  Scores and outputs on the bf16 matrix pipe with fp32 accumulation, the
+ * probabilities rounded to bf16 in between; results agree with an fp32 evaluation of the same formula to
+ * about 1e-2 relative on bf16 outputs.
  */
 int bitnet_attn_decode(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v,
                        const int64_t* positions, const float* cos_table,
@@ -114,12 +112,6 @@ int bitnet_attn_prefill(const uint16_t* q, const uint16_t* cache_k, const uint16
  * (256 or 512; 0 restores the built-in choice).  Results do not depend on it beyond the
  * order of fp32 additions.  Returns 0, or 1 for another value. */
 int bitnet_attn_decode_set_threads(int threads);
-
-/* Tuning override for tests and measurements: 0 = the library's choice of decode-step attention
- * kernel, 1 = scores in an LDS buffer and P.V on the vector pipe, 2 = scores, softmax and P.V in
- * registers with both products on the matrix pipe (probabilities rounded to bf16).  Returns 0, or
- * 1 for another value. */
-int bitnet_attn_decode_set_kernel(int which);
 
 /* Number of floats bitnet_attn_decode needs as workspace; -1 for bad arguments. */
 int bitnet_attn_decode_workspace_floats(int B, int n_heads, int n_kv_heads, int n_splits);

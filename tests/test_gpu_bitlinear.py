@@ -316,7 +316,7 @@ def test_result_independent_of_kernel_and_launch_shape():
             pk, ad = _packed_dev(w), dev_i8(a)
             want = o.acc_int32(a, w)
             settings = [(2, wv, u) for wv, u in [(1, 1), (2, 8), (3, 4), (7, 8), (16, 2), (16, 8), (5, 1)]]
-            settings += [(1, 1, 0), (1, 2, 0), (1, 3, 0), (1, 4, 0), (0, 0, 0)]
+            settings += [(0, 0, 0)]
             for setting in settings:
                 assert lib.bitlinear_set_tuning(*setting, 0) == 0
                 acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
@@ -327,19 +327,12 @@ def test_result_independent_of_kernel_and_launch_shape():
 
 @pytest.mark.parametrize("n,k", [(16, 64), (16, 128), (48, 192), (80, 320), (32, 3200), (1040, 256)])
 @pytest.mark.parametrize("m", [1, 2, 4])
-def test_decode_kernel_ragged_shapes(n, k, m):
+def test_default_kernels_on_ragged_shapes(n, k, m):
     """K not a multiple of 256 (partial last step) and row-block counts that
-    do not fill the last workgroup."""
-    lib = _lib.load_library()
+    do not fill the last workgroup, through whatever the library chooses."""
     w, a = _rand_case(n, k, m, seed=n + k + m)
-    want = o.acc_int32(a, w)
-    try:
-        for waves in (1, 3, 4):
-            assert lib.bitlinear_set_tuning(1, waves, 0, 0) == 0
-            acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
-            assert np.array_equal(acc.cpu().numpy(), want), waves
-    finally:
-        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    acc = bitlinear.bitnet_int8xint2_acc(dev_i8(a), _packed_dev(w))
+    assert np.array_equal(acc.cpu().numpy(), o.acc_int32(a, w))
 
 
 def _forward_raw(lib, xb, pk, ws_bits, m, n, k, mode, with_ws=True):

@@ -136,15 +136,13 @@ def _ulp(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return (mono(a) - mono(b)).abs()
 
 
-@pytest.mark.parametrize("which", [1, 2])
 @pytest.mark.parametrize("n_splits", [1, 3, 8])
 @pytest.mark.parametrize("B,S,nh,nkv", [(1, 641, 20, 5), (8, 200, 20, 5), (2, 64, 4, 1), (3, 1500, 8, 8), (2, 33, 16, 2)])
-def test_attention_decode_kernel_against_torch_fp32(B, S, nh, nkv, n_splits, which):
-    """Floating-point kernels: compared with the fp32 torch restatement (rope,
-    cache write, softmax(QK^T/sqrt(d))V).  Kernel 1 (fp32 probabilities, P.V on
-    the vector pipe): 2 bf16 ulp or 2e-3 absolute on the bf16 outputs (fp32
-    sums in a different order); kernel 2 (probabilities rounded to bf16 for the
-    matrix pipe): 3 ulp or 4e-3."""
+def test_attention_decode_kernel_against_torch_fp32(B, S, nh, nkv, n_splits):
+    """A floating-point kernel: compared with the fp32 torch restatement (rope,
+    cache write, softmax(QK^T/sqrt(d))V).  Its probabilities are rounded to
+    bf16 for the matrix pipe and its fp32 sums run in another order: 3 bf16 ulp
+    or 4e-3 absolute on the bf16 outputs."""
     hd = 128
     dev = torch.device("cuda")
     g = torch.Generator(device="cuda").manual_seed(B * 1000 + S)
@@ -171,28 +169,22 @@ def test_attention_decode_kernel_against_torch_fp32(B, S, nh, nkv, n_splits, whi
     mask = torch.arange(S, device=dev)[None, None, :] <= pos[:, None, None]
     want = att.attend(q, rk, rv, mask)[:, 0]
     ws = decoder.AttnWorkspace(B, nh, nkv, n_splits, dev) if n_splits > 1 else None
-    lib = _lib.load_library()
-    assert lib.bitnet_attn_decode_set_kernel(which) == 0
-    try:
-        got = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
-        torch.cuda.synchronize()
-        assert torch.equal(ck, rk) and torch.equal(cv, rv)  # cache rows written exactly
-        if ws is not None:
-            assert int(ws.counters.abs().sum()) == 0  # arrival counters reset by the last split
-            again = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)  # same cache row rewritten
-            assert torch.equal(again, got)
-        # the same call with the positions' cos | sin rows handed over: identical bits
-        emb = torch.randn(16, 64, generator=g, device=dev).to(torch.bfloat16)
-        toks = torch.randint(0, 16, (B,), generator=g, device=dev)
-        h0, rows = decoder.decode_step_begin(toks, pos, emb, cos, sin)
-        assert torch.equal(h0, emb[toks]) and torch.equal(rows, torch.cat([cos[pos], sin[pos]], dim=1))
-        ck2, cv2 = ck.clone(), cv.clone()
-        with_rows = decoder.attn_decode(xqkv, ck2, cv2, pos, cos, sin, nh, nkv, ws, rope_rows=rows)
-        torch.cuda.synchronize()
-        assert torch.equal(with_rows, got) and torch.equal(ck2, rk) and torch.equal(cv2, rv)
-    finally:
-        lib.bitnet_attn_decode_set_kernel(0)
-    ulps, tol = (2, 2e-3) if which == 1 else (3, 4e-3)
+    got = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(ck, rk) and torch.equal(cv, rv)  # cache rows written exactly
+    if ws is not None:
+        again = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)  # same cache row rewritten
+        assert torch.equal(again, got)
+    # the same call with the positions' cos | sin rows handed over: identical bits
+    emb = torch.randn(16, 64, generator=g, device=dev).to(torch.bfloat16)
+    toks = torch.randint(0, 16, (B,), generator=g, device=dev)
+    h0, rows = decoder.decode_step_begin(toks, pos, emb, cos, sin)
+    assert torch.equal(h0, emb[toks]) and torch.equal(rows, torch.cat([cos[pos], sin[pos]], dim=1))
+    ck2, cv2 = ck.clone(), cv.clone()
+    with_rows = decoder.attn_decode(xqkv, ck2, cv2, pos, cos, sin, nh, nkv, ws, rope_rows=rows)
+    torch.cuda.synchronize()
+    assert torch.equal(with_rows, got) and torch.equal(ck2, rk) and torch.equal(cv2, rv)
+    ulps, tol = 3, 4e-3
     bad = (_ulp(got, want) > ulps) & ((got.float() - want.float()).abs() > tol)
     assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance"
 
@@ -233,9 +225,8 @@ def test_attention_decode_long_cache_any_position(p, n_splits):
     assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance"
 
 
-@pytest.mark.parametrize("which", [1, 2])
 @pytest.mark.parametrize("n_splits", [1, 8])
-def test_attention_decode_ignores_rows_behind_the_position(n_splits, which):
+def test_attention_decode_ignores_rows_behind_the_position(n_splits):
     """Cache rows behind a sequence's position may never have been written:
     with NaNs there the output has the bits it has with finite values there."""
     B, S, nh, nkv, hd = 3, 300, 8, 2, 128
@@ -247,17 +238,12 @@ def test_attention_decode_ignores_rows_behind_the_position(n_splits, which):
     pos = torch.tensor([0, 37, 255], device=dev)
     cos, sin = decoder.rope_tables(hd, S, 500000.0, dev)
     ws = decoder.AttnWorkspace(B, nh, nkv, n_splits, dev) if n_splits > 1 else None
-    lib = _lib.load_library()
-    assert lib.bitnet_attn_decode_set_kernel(which) == 0
-    try:
-        want = decoder.attn_decode(xqkv, ck.clone(), cv.clone(), pos, cos, sin, nh, nkv, ws)
-        behind = torch.arange(S, device=dev)[None, :] > pos[:, None]
-        ck[behind] = float("nan")
-        cv[behind] = float("nan")
-        got = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
-        torch.cuda.synchronize()
-    finally:
-        lib.bitnet_attn_decode_set_kernel(0)
+    want = decoder.attn_decode(xqkv, ck.clone(), cv.clone(), pos, cos, sin, nh, nkv, ws)
+    behind = torch.arange(S, device=dev)[None, :] > pos[:, None]
+    ck[behind] = float("nan")
+    cv[behind] = float("nan")
+    got = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
+    torch.cuda.synchronize()
     assert not torch.isnan(got.float()).any()
     assert torch.equal(got, want)
     assert torch.isnan(ck[behind].float()).all() and torch.isnan(cv[behind].float()).all()
@@ -468,10 +454,9 @@ def test_attention_merge_that_gives_up_is_reported():
     assert torch.equal(fresh, good) and ws2.error() == 0
 
 
-@pytest.mark.parametrize("which", [1, 2])
-def test_attention_decode_clamps_positions_outside_the_cache(which):
+def test_attention_decode_clamps_positions_outside_the_cache():
     """A position outside [0, S) must not take any access outside the buffers:
-    the kernels clamp it.  Checked on outputs and buffers only: a position of
+    the kernel clamps it.  Checked on outputs and buffers only: a position of
     S + 1000 (or 2^40) behaves exactly like S - 1, a negative one like 0, and
     guard rows allocated around the cache keep their bytes."""
     B, S, nh, nkv, hd = 3, 96, 8, 2, 128
@@ -491,19 +476,14 @@ def test_attention_decode_clamps_positions_outside_the_cache(which):
         return k, v, flat_k, flat_v
 
     cos, sin = decoder.rope_tables(hd, S, 500000.0, dev)
-    lib = _lib.load_library()
-    assert lib.bitnet_attn_decode_set_kernel(which) == 0
-    try:
-        outs = []
-        for pos_list in ([S + 1000, -7, 1 << 40], [S - 1, 0, S - 1]):
-            k, v, ck, cv = caches()
-            pos = torch.tensor(pos_list, device=dev, dtype=torch.int64)
-            ws = decoder.AttnWorkspace(B, nh, nkv, 4, dev)
-            out = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
-            torch.cuda.synchronize()
-            outs.append((out, k, v))
-    finally:
-        lib.bitnet_attn_decode_set_kernel(0)
+    outs = []
+    for pos_list in ([S + 1000, -7, 1 << 40], [S - 1, 0, S - 1]):
+        k, v, ck, cv = caches()
+        pos = torch.tensor(pos_list, device=dev, dtype=torch.int64)
+        ws = decoder.AttnWorkspace(B, nh, nkv, 4, dev)
+        out = decoder.attn_decode(xqkv, ck, cv, pos, cos, sin, nh, nkv, ws)
+        torch.cuda.synchronize()
+        outs.append((out, k, v))
     (o_bad, k_bad, v_bad), (o_ok, k_ok, v_ok) = outs
     assert not torch.isnan(o_bad.float()).any()
     assert torch.equal(o_bad, o_ok)
