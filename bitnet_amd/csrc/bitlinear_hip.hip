@@ -892,6 +892,267 @@ void gemm_i2_prefill_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Prefill GEMM for the 64 x 256 (and 128 x 256) output tile once the machine is full: the same decomposition as
+// gemm_i2_prefill_kernel (four waves side by side along n, weights from global straight into the MFMA row
+// operand, activations through LDS), rebuilt around what the CU's vector-memory path costs.  Measured with a
+// loop of MFMAs and one kind of other instruction between them: vector, scalar and wait instructions are free
+// next to v_mfma_i32_32x32x32_i8, two 16-byte LDS reads per four MFMAs as well, but every vector-memory
+// instruction occupies the CU's one 64-byte-per-cycle load path for as long as its bytes take, a path all waves
+// of the CU share, and a wave stands still while its request is taken.  So:
+//  * the activation chunk goes from global memory straight into LDS (buffer_load ... lds, 1 KB per wave and
+//    instruction, no registers, no vector instructions; rows XOR-swizzled in 16-byte pieces so that the MFMA
+//    operand reads hit every bank once), three stages deep;
+//  * a lane fetches the words of its NT column tiles with ONE load per 32-k step: the wave's 32 * NT columns
+//    are 2 * NT row blocks of the packed layout, a lane takes NT consecutive words of a tile's run of eight
+//    (NT consecutive weight rows, one k-half) and word i feeds column tile i, which therefore holds every
+//    NT-th column; half (a quarter) as many weight requests as one word per column tile;
+//  * the stored codes c = w + 2 are expanded to bytes that read 64 * w -- xor with 0b10 gives w in two-bit two's
+//    complement, and a two-bit field at the top of a byte is that number times 64 -- so the accumulators are
+//    64 * sum(w * a) exactly (|.| <= 64 * 127 * K < 2^31 up to K = 262144), the +2 of the codes never enters,
+//    no row sums are collected and the epilogue starts with an exact shift;
+//  * with the interleaved column tiles a lane's accumulators of one register quad are 4 * NT consecutive output
+//    columns: 16-byte (NT = 2) or 32-byte stores per token instead of 8.
+// K must be a multiple of CK.
+constexpr int kPfxWaves = 4;
+template <int NT>
+struct PfxWords;
+template <>
+struct PfxWords<2> {
+    typedef uint32_t type __attribute__((ext_vector_type(2)));
+};
+template <>
+struct PfxWords<4> {
+    typedef uint32_t type __attribute__((ext_vector_type(4)));
+};
+// 16 bytes per lane from a buffer straight into LDS: lane l's piece lands at ldsp + 16 l (ldsp wave-uniform)
+__device__ __forceinline__ void load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, int8_t* ldsp, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)ldsp, 16, voff, soff, 0, 0);
+}
+
+template <int MT, int NT, int CK>
+__global__ __launch_bounds__(kPfxWaves * 64) __attribute__((amdgpu_waves_per_eu(MT * NT <= 4 ? 3 : 2)))
+void gemm_i2_prefill_dma_kernel(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int nunits, int cseg_shift,
+    int band, int seg_cols, const uint16_t* __restrict__ s, uint16_t* __restrict__ out, int32_t* __restrict__ acc_out,
+    const uint16_t* __restrict__ ws, ScaleMap smap, const uint16_t* __restrict__ residual) {
+    constexpr int TM = MT * 32;
+    constexpr int KSTEPS = CK / 32;
+    constexpr int PPR = CK / 16;             // 16-byte pieces per row and chunk
+    constexpr int RPI = 64 / PPR;            // rows one load instruction of a wave covers
+    constexpr int ROUNDS = TM / (RPI * kPfxWaves);  // load instructions per wave and stage
+    constexpr int SB = TM * CK;              // bytes per stage
+    constexpr int QR = 8 / NT;               // lanes per run of eight words
+    static_assert(NT == 2 || NT == 4, "two or four interleaved column tiles");
+    static_assert(TM % (RPI * kPfxWaves) == 0 && (CK == 128 || CK == 256), "stage shape");
+    extern __shared__ __attribute__((aligned(1024))) int8_t lds_x[];  // [3][TM][CK], rows swizzled in 16-byte pieces
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // workgroup -> tile: as gemm_i2_prefill_kernel (bands of row tiles per XCD, column segments)
+    const int row_tiles = (M + TM - 1) / TM;
+    const int col_tiles = (N + kPfxWaves * NT * 32 - 1) / (kPfxWaves * NT * 32);
+    const int unit = (blockIdx.x & 7) + 8 * blockIdx.z;
+    if (unit >= nunits) return;
+    const bool has_out = (cseg_shift >> 8) != 0;
+    cseg_shift &= 0xff;
+    const int col_tile = (unit & ((1 << cseg_shift) - 1)) * seg_cols + blockIdx.y;
+    const int row_tile = (unit >> cseg_shift) * band + (blockIdx.x >> 3);
+    if (row_tile >= row_tiles || col_tile >= col_tiles) return;
+    const int m0 = row_tile * TM;
+    const int n0 = (col_tile * kPfxWaves + wave) * NT * 32;
+    const int nl = lane & 31;
+    const int kc = lane >> 5;
+    const int nchunks = K / CK;
+
+    // rows past M lie beyond the activation descriptor: they arrive in LDS as zeros
+    const int rows_here = (M - m0) < TM ? (M - m0) : TM;
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(act + (size_t)m0 * K), 0, rows_here * K, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, (N >> 2) * K, 0x00020000);
+
+    // activation requests: instruction (r * 4 + wave) of a stage fills 1 KB of it = RPI rows; the lane at LDS
+    // piece p of row i fetches global piece p ^ (i & 7) (the row offset is part of the vector offset: the one
+    // the descriptor's range check sees)
+    const int arow = wave * RPI + lane / PPR;
+    const int akp = (lane % PPR) ^ (arow & 7);
+    int a_voff[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) a_voff[r] = (arow + r * kPfxWaves * RPI) * K + akp * 16;
+    auto load_stage = [&](int c, int st) {
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) load16_to_lds(a_rsrc, lds_x + st * SB + (r * kPfxWaves + wave) * 1024, a_voff[r], c * CK);
+    };
+    // weight requests (row blocks past N repeat the last one; their columns are never stored)
+    const int wb = nl / (2 * QR), wp = nl % (2 * QR), whi = wp / QR, wlo = NT * (wp % QR);
+    int w_voff;
+    {
+        int blk = (n0 >> 4) + wb;
+        blk = blk < (N >> 4) ? blk : (N >> 4) - 1;
+        w_voff = blk * K * 4 + (whi * 16 + kc * 8 + wlo) * 4;
+    }
+    const int last_step_off = ((K >> 5) - 1) * 128;
+    typedef typename PfxWords<NT>::type wvec_t;
+    auto load_words = [&](int c, int ks) -> wvec_t {
+        int so = (c * KSTEPS + ks) * 128;
+        so = so < last_step_off ? so : last_step_off;  // the step behind the last chunk re-reads the last one
+        if constexpr (NT == 2)
+            return __builtin_bit_cast(wvec_t, __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, w_voff, so, 0));
+        else
+            return __builtin_bit_cast(wvec_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, w_voff, so, 0));
+    };
+    // the scales of the lane's MT tokens (without output there are none: the request goes to an address that exists)
+    uint16_t s_raw[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + mt * 32 + nl;
+        s_raw[mt] = *(has_out ? s + (m < M ? m : M - 1) : (const uint16_t*)wq);
+    }
+
+    v16i acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0;
+
+    wvec_t wW[KSTEPS];
+    load_stage(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) wW[ks] = load_words(0, ks);
+    if (nchunks > 1) load_stage(1, 1);
+
+    // LDS read offsets: row nl, piece (2 ks + kc) ^ (nl & 7)
+    int a_rd[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) a_rd[ks] = nl * CK + (((ks * 2 + kc) ^ (nl & 7)) * 16);
+
+    auto expand = [&](uint32_t wd) -> v4i {
+        const uint32_t x = wd ^ 0xAAAAAAAAu;
+        v4i r;
+        r.x = (int)((x << 6) & 0xC0C0C0C0u);
+        r.y = (int)((x << 4) & 0xC0C0C0C0u);
+        r.z = (int)((x << 2) & 0xC0C0C0C0u);
+        r.w = (int)(x & 0xC0C0C0C0u);
+        return r;
+    };
+
+    // the first chunk: every wave waits for its own requests, then all meet
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); the other counters untouched
+    lds_barrier();
+
+    auto chunk_body = [&](int c, auto stc) {
+        constexpr int ST = decltype(stc)::value;
+        constexpr int SLOTS = MT * NT;
+        // stage (ST + 2) % 3 was read in chunk c - 1, which every wave has left (the barrier at its end)
+        if (c + 2 < nchunks) load_stage(c + 2, (ST + 2) % 3);
+        const int8_t* abuf = lds_x + ST * SB;
+        v4i aop[2][MT], bop[2][NT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) aop[0][mt] = *(const v4i*)(abuf + a_rd[0] + mt * 32 * CK);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) bop[0][nt] = expand(wW[0][nt]);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+#pragma unroll
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                const int mt = slot / NT, nt = slot % NT;
+                acc[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bop[cur][nt], aop[cur][mt], acc[mt][nt], 0, 0, 0);
+                if (ks + 1 < KSTEPS) {
+#pragma unroll
+                    for (int j = 0; j < MT; ++j)
+                        if (j % SLOTS == slot) aop[nxt][j] = *(const v4i*)(abuf + a_rd[ks + 1] + j * 32 * CK);
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        if ((MT + j) % SLOTS == slot) bop[nxt][j] = expand(wW[ks + 1][j]);
+                }
+                if (slot == SLOTS - 1) wW[ks] = load_words(c + 1, ks);  // expanded during the step before: re-request
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // the next chunk's activations (requested two chunks ago) are older than every request that may stay in
+        // flight: this chunk's re-requested words and the stage requested at its start
+        constexpr int kYounger = KSTEPS + ROUNDS;
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (kYounger & 15) | ((kYounger >> 4) << 14));
+        lds_barrier();
+    };
+    int c = 0;
+    for (; c + 3 <= nchunks; c += 3) {
+        chunk_body(c, std::integral_constant<int, 0>{});
+        chunk_body(c + 1, std::integral_constant<int, 1>{});
+        chunk_body(c + 2, std::integral_constant<int, 2>{});
+    }
+    if (c < nchunks) chunk_body(c, std::integral_constant<int, 0>{});
+    if (c + 1 < nchunks) chunk_body(c + 1, std::integral_constant<int, 1>{});
+
+    // Epilogue.  A lane holds token nl of row tile mt; register r of column tile nt is the weight row with
+    // operand index (r / 4) * 8 + kc * 4 + r % 4, i.e. column n0 + 16 b + 8 hi + lo + nt with that index split
+    // into (b, hi, lo) as in the weight requests: for one register quad the 4 * NT values over (r % 4, nt) are
+    // 4 * NT consecutive columns.  Division by the token's scale as in gemm_i2_prefill_kernel (reciprocal and
+    // one correction step: the bits of the IEEE divide for these integer numerators).
+    const int n_first = n0 < N ? n0 : N - 1;
+    const int n_last = (n0 + NT * 32 - 1) < N ? (n0 + NT * 32 - 1) : N - 1;
+    const int slot_first = scale_slot(smap, n_first);
+    const bool one_slot = slot_first == scale_slot(smap, n_last);
+    const float w1 = out ? bf16_to_f32(ws[slot_first]) : 1.0f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + mt * 32 + nl;
+        const float sv = has_out ? bf16_to_f32(s_raw[mt]) : 1.0f;
+        const float ri = 1.0f / sv;
+        if (m >= M) continue;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const int ridx = g4 * 8 + kc * 4;
+            const int n = n0 + 16 * (ridx / (2 * QR)) + 8 * ((ridx % (2 * QR)) / QR) + NT * (ridx % QR);
+            if (n >= N) continue;  // N % 16 == 0 and n % (4 * NT) == 0: the columns of a quad are in or out together
+            const size_t o = (size_t)m * N + n;
+            int sum[4 * NT];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    // column offset of (register j of the quad, column tile nt) from n
+                    const int col = NT == 2 ? 2 * j + nt : 8 * (j / 2) + 4 * (j % 2) + nt;
+                    sum[col] = acc[mt][nt][g4 * 4 + j] >> 6;  // exact: the accumulator is 64 * sum(w * a)
+                }
+            if (acc_out) {
+#pragma unroll
+                for (int v = 0; v < NT; ++v) *(v4i*)(acc_out + o + 4 * v) = v4i{sum[4 * v], sum[4 * v + 1], sum[4 * v + 2], sum[4 * v + 3]};
+            }
+            if (out) {
+                float h[4 * NT];
+#pragma unroll
+                for (int col = 0; col < 4 * NT; ++col) {
+                    const float a = (float)sum[col];
+                    const float q0 = a * ri;
+                    const float q = __builtin_fmaf(__builtin_fmaf(-q0, sv, a), ri, q0);
+                    h[col] = q * (one_slot ? w1 : bf16_to_f32(ws[scale_slot(smap, n + col)]));
+                }
+#pragma unroll
+                for (int v = 0; v < NT / 2; ++v) {
+                    uint4 ob = make_uint4(f32x2_to_bf16x2(h[8 * v], h[8 * v + 1]), f32x2_to_bf16x2(h[8 * v + 2], h[8 * v + 3]),
+                                          f32x2_to_bf16x2(h[8 * v + 4], h[8 * v + 5]), f32x2_to_bf16x2(h[8 * v + 6], h[8 * v + 7]));
+                    if (residual) {  // out = bf16(residual + bf16(result))
+                        const uint4 rv = *(const uint4*)(residual + o + 8 * v);
+                        const uint32_t a4[4] = {ob.x, ob.y, ob.z, ob.w}, r4[4] = {rv.x, rv.y, rv.z, rv.w};
+                        uint32_t o4[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            o4[j] = f32x2_to_bf16x2(__uint_as_float(r4[j] << 16) + __uint_as_float(a4[j] << 16),
+                                                    __uint_as_float(r4[j] & 0xffff0000u) + __uint_as_float(a4[j] & 0xffff0000u));
+                        ob = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+                    }
+                    *(uint4*)(out + o + 8 * v) = ob;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Per-token absmax quantizer: one workgroup per token row
 // ---------------------------------------------------------------------------
 constexpr int kQuantThreads = 256;
@@ -2585,7 +2846,18 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // one full round of the former, one round of the latter finishes earlier (13824 x 2560 at M = 1024: 864 tiles,
     // 46.5 -> 42.3 us; 3840 x 2560 at M = 4096: 960 tiles, 45.1 -> 44.1)
     if (tile == 2 && wide_tiles > kPrefillRound64 && wide_tiles <= kPrefillRound128) tile = 1;
-    if (t_tune.path == 5) tile = t_tune.prefill_big;
+    // the 64 x 256 tile goes through the kernel that brings the activations into LDS without registers and the
+    // weight words of two column tiles with one request (a layer's four GEMMs at M = 2048: 1.72 -> 1.92 POP/s on
+    // uniform random int8; 13824 x 2560 73.3 -> 64.8 us, 2560 x 6912 46.3 -> 42.2, at M = 4096 1.97 -> 2.20),
+    // given 128-k chunks that divide K and 16-byte aligned rows
+    bool dma = true;
+    if (t_tune.path == 5) {
+        tile = t_tune.prefill_big;
+        dma = tile == 5;
+        if (tile == 5) tile = 2;
+    }
+    const bool dma_fits = K % 128 == 0 && ((((uintptr_t)out) | ((uintptr_t)acc_out) | ((uintptr_t)residual)) & 15u) == 0 &&
+                          ((long long)M * K < (1ll << 31));
     // groups of waves that split a tile's K between them (small tiles only): while the small tiles
     // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
     // instruction stream, and more groups shorten it
@@ -2656,6 +2928,14 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     } else if (tile == 2) {
         if (ks == 2) {
             BITLINEAR_LAUNCH_PF(2, 2, 2);
+        } else if (dma && dma_fits) {
+            g_last_kernel = "gemm_i2_prefill_dma_kernel";
+            if (K % 256 == 0)
+                BL_LAUNCH((gemm_i2_prefill_dma_kernel<2, 2, 256>), grid, block, 3 * 64 * 256, stream, act, wq, M, N, K, units,
+                          cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual);
+            else
+                BL_LAUNCH((gemm_i2_prefill_dma_kernel<2, 2, 128>), grid, block, 3 * 64 * 128, stream, act, wq, M, N, K, units,
+                          cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual);
         } else {
             BITLINEAR_LAUNCH_PF(2, 2, 1);
         }
@@ -3043,7 +3323,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
-        if (a < 0 || a > 4 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 0 || a > 5 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
         g.path = 5;
         g.prefill_big = a;
         g.prefill_band = b;

@@ -31,7 +31,7 @@ def test_plan_rows_say_what_the_design_says():
     assert p(2, 1, 3840, 2560).startswith("bitlinear_solo_kernel<5, 1, 1, true, 1, false, 1>")
     two = p(1, 8, 3840, 2560).split(" + ")
     assert len(two) == 2 and two[0].startswith("quant_absmax_rows_kernel<0, 5>") and two[1].startswith("gemv_i2_solo_kernel<5, 1, false>")
-    assert "gemm_i2_prefill_kernel" in p(0, 17, 13824, 2560) and "gemm_i2_prefill_kernel<2, 2, 1>" in p(0, 2048, 13824, 2560)
+    assert "gemm_i2_prefill_kernel" in p(0, 17, 13824, 2560) and "gemm_i2_prefill_dma_kernel<2, 2, 256>" in p(0, 2048, 13824, 2560)
     assert p(0, 1, 55296, 5120).startswith("gemv_i2_stream_kernel<5, true>")
     assert p(0, 1, 20480, 3200).startswith("bitlinear_fused_kernel<")
 

@@ -544,7 +544,39 @@ def test_fused_forward_launch_shapes_and_null_workspaces():
         lib.bitlinear_set_tuning(0, 0, 0, 0)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("m,n,k", [(17, 48, 128), (33, 16, 256), (64, 272, 384), (65, 1040, 640), (100, 2560, 768), (128, 2560, 2560),
+                                   (129, 3840, 2560), (300, 1040, 3200), (512, 2560, 6912), (1000, 13824, 2560)])
+def test_prefill_gemm_through_the_direct_to_lds_kernel(m, n, k):
+    """gemm_i2_prefill_dma_kernel (activation chunks straight into LDS, one weight request per k-step for two
+    interleaved column tiles, codes expanded to 64 * w): forced for every shape with K % 128 == 0 -- one to 54
+    chunks of 128 or 256 k, chunk counts that leave 0, 1 and 2 chunks behind the loop's rounds of three, ragged
+    M and N, a last workgroup whose waves lie partly or wholly beyond N -- accumulators equal to the oracle's,
+    bf16 outputs (the reference's scale slots, and explicit segments cutting through a register quad's 8
+    columns) equal bit for bit.  (The residual epilogue: test_norm_forward_with_residual_beyond_decode_sizes.)"""
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=m + n + k)
+    s_bits = o.f32_to_bf16_bits(np.linspace(3.0, 90.0, m).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    acc_want, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    ends = [n] if n < 64 else [20, n // 2 + 4, n]  # boundaries inside a register quad's 8 columns
+    _, want_seg = o.bitlinear_int8xint2_seg(a, w, s_bits, ws_bits, ends)
+    ad, pk, sd, wsd = dev_i8(a), _packed_dev(w), dev_bf16(s_bits), dev_bf16(ws_bits)
+    try:
+        assert lib.bitlinear_set_tuning(5, 5, 0, 0) == 0
+        acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
+        name = bitlinear.last_kernel()
+        out = bitlinear.bitnet_int8xint2_linear(ad, pk, sd, wsd)
+        out_seg = bitlinear.bitnet_int8xint2_linear_seg(ad, pk, sd, wsd, ends)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert name == "gemm_i2_prefill_dma_kernel"
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    _assert_bits_equal(host_bits(out), want, "direct-to-LDS GEMM")
+    _assert_bits_equal(host_bits(out_seg), want_seg, f"direct-to-LDS GEMM, segments {ends}")
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("m,n,k", [(17, 48, 192), (64, 128, 64), (100, 272, 320), (128, 2560, 2560), (129, 3840, 2560),
                                    (300, 1040, 3200), (512, 2560, 6912)])
 def test_prefill_gemm_acc_bit_exact(m, n, k, tile):
@@ -620,7 +652,7 @@ def test_prefill_scaled_output_with_outliers(shape_id, m):
     mod.weight.data = _packed_dev(w)
     mod.weight_scale.data = dev_bf16(ws_bits)
     out = mod(dev_bf16(xb))
-    assert bitlinear.last_kernel() == "gemm_i2_prefill_kernel"
+    assert bitlinear.last_kernel() in ("gemm_i2_prefill_kernel", "gemm_i2_prefill_dma_kernel")
     _assert_bits_equal(host_bits(out), want, f"{sh.name} prefill M={m}")
     qd, sd = mod.quant_input(dev_bf16(xb))
     assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(host_bits(sd).reshape(-1), s_bits)
@@ -829,7 +861,7 @@ def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
     assert st != 0
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("m,n,k,glu", [(40, 2560, 2560, 0), (130, 3840, 2560, 0), (300, 2560, 6912, 1), (77, 48, 192, 1),
                                        (513, 1040, 640, 0), (1030, 64, 2560, 0), (1025, 272, 640, 0), (1024, 48, 4096, 0),
                                        (1026, 32, 6912, 1)])  # from 1024 rows on without the gate: a wave per row
