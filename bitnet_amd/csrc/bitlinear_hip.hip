@@ -2841,23 +2841,27 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // (beyond the few-tile range the wide tile: against 64 x 128 it measured level or ahead from 330 tiles on --
     // 2560 x 6912 at M = 1536 31.7 -> 29.2 us, 2560 x 2560 there 14.3 -> 13.6, elsewhere within 2 %)
     const long long wide_tiles = (long long)((N + 255) / 256) * ((M + 63) / 64);
+    // (the kernel that brings the activation chunks straight into LDS needs 128-k chunks that divide K and 16-byte
+    // aligned output rows)
+    const bool dma_fits = K % 128 == 0 && ((((uintptr_t)out) | ((uintptr_t)acc_out) | ((uintptr_t)residual)) & 15u) == 0;
     int tile = ((N >= kPrefillWideN && M >= kPrefillWideMinTokens) || narrow_tiles > kPrefillFewTiles) ? 2 : 4;
     // 64 x 256 tiles run three workgroups per CU (768 at a time), 128 x 256 tiles two (512): with a little more than
     // one full round of the former, one round of the latter finishes earlier (13824 x 2560 at M = 1024: 864 tiles,
     // 46.5 -> 42.3 us; 3840 x 2560 at M = 4096: 960 tiles, 45.1 -> 44.1)
-    if (tile == 2 && wide_tiles > kPrefillRound64 && wide_tiles <= kPrefillRound128) tile = 1;
+    // (with the direct-to-LDS kernel the 64 x 256 tiles stay: 13824 x 2560 at M = 1024 41.5 -> 39.8 us)
+    if (tile == 2 && wide_tiles > kPrefillRound64 && wide_tiles <= kPrefillRound128 && !dma_fits) tile = 1;
     // the 64 x 256 tile goes through the kernel that brings the activations into LDS without registers and the
     // weight words of two column tiles with one request (a layer's four GEMMs at M = 2048: 1.72 -> 1.92 POP/s on
     // uniform random int8; 13824 x 2560 73.3 -> 64.8 us, 2560 x 6912 46.3 -> 42.2, at M = 4096 1.97 -> 2.20),
     // given 128-k chunks that divide K and 16-byte aligned rows
     bool dma = true;
+    int dma_mt = 2;  // row tiles of 32 tokens per workgroup of that kernel: 64 x 256, or 32 x 256 / 128 x 256 when forced
     if (t_tune.path == 5) {
         tile = t_tune.prefill_big;
-        dma = tile == 5;
-        if (tile == 5) tile = 2;
+        dma = tile >= 5;
+        dma_mt = tile == 6 ? 1 : (tile == 7 ? 4 : 2);
+        if (tile >= 5) tile = tile == 7 ? 1 : (tile == 6 ? 8 : 2);  // 8: 32 x 256, a shape only that kernel has
     }
-    const bool dma_fits = K % 128 == 0 && ((((uintptr_t)out) | ((uintptr_t)acc_out) | ((uintptr_t)residual)) & 15u) == 0 &&
-                          ((long long)M * K < (1ll << 31));
     // groups of waves that split a tile's K between them (small tiles only): while the small tiles
     // leave SIMDs with one or two waves, a tile's chain of chunks runs at the speed of one wave's
     // instruction stream, and more groups shorten it
@@ -2878,17 +2882,27 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // about one 64 x 256 tile per CU: those tiles, two groups of waves each (2560 x 6912: M = 1024 25.9 -> 23.4 us,
     // M = 1536 29.2 -> 27.9; 13824 x 2560 at M = 256 15.8 -> 14.3; 2560 x 2560 at M = 1280 13.6 -> 13.1; with 320
     // tiles 42.6 -> 49.4: not taken; at K = 2560 the 32 x 128 tiles stay ahead up to 330 of the 64 x 128 kind)
+    // (with the direct-to-LDS kernel one group does as well or better: 13824 x 2560 at M = 256 17.1 -> 14.8 us,
+    // 2560 x 6912 at M = 1024 27.3 -> 27.0)
     if (t_tune.path != 5 && (tile == 2 || (tile == 4 && K >= kPrefillSplit4MinK)) && wide_tiles > kPrefillOnePerCuMin &&
         wide_tiles <= kPrefillOnePerCuMax && narrow_tiles > kPrefillOnePerCuMax) {
         tile = 2;
-        ks = 2;
+        ks = (dma_fits && K < kPrefillSplit4MinK) ? 1 : 2;  // (long rows keep the two groups: 2560 x 6912 at M = 1024 level)
     }
+    // between one and one and a half 64 x 256 tiles per CU a quarter of the CUs would get two tiles and the rest one:
+    // half-height tiles (32 x 256, the direct-to-LDS kernel only) spread evenly, at most three per CU (2560 x 2560 at
+    // M = 2048 21.3 -> 20.0 us, 2560 x 6912 43.5 -> 42.5, 3840 x 2560 at M = 1536 21.5 -> 21.1; from two tiles per CU
+    // on the full-height tiles are ahead again: 2560 x 2560 at M = 4096 30.7 against 32.1)
+    if (t_tune.path != 5 && tile == 2 && ks == 1 && dma_fits && wide_tiles > kPrefillOnePerCuMax &&
+        wide_tiles <= kPrefillOnePerCuMax + kPrefillOnePerCuMin)
+        tile = 8;
     if (t_tune.path == 5 && t_tune.prefill_ks > 0) ks = (tile == 4 || ((tile == 0 || tile == 2) && t_tune.prefill_ks == 2)) ? t_tune.prefill_ks : 1;
     if (K <= kPfChunk * (ks - 1)) ks = 1;  // fewer chunks than groups
     const dim3 block(kPfWaves * 64 * ks, 1, 1);
     // grid of 8 XCDs x bands per XCD x tiles per band (see the kernel); bands of up to 8 row
     // tiles, fewer when there are not enough row tiles to give every XCD a band
-    const int tm = tile == 1 ? 128 : (tile == 4 ? 32 : 64);
+    if (tile == 8 && !dma_fits) tile = 4;
+    const int tm = tile == 1 ? 128 : ((tile == 4 || tile == 8) ? 32 : 64);
     const int tn = (tile == 0 || tile == 4) ? 128 : (tile == 3 ? 512 : 256);
     const int row_tiles = (M + tm - 1) / tm, col_tiles = (N + tn - 1) / tn;
     int band = row_tiles / 8;
@@ -2913,7 +2927,18 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
 #define BITLINEAR_LAUNCH_PF(MT_, NT_, KS_)                                                                          \
     BL_LAUNCH((gemm_i2_prefill_kernel<MT_, NT_, KS_>), grid, block, KS_ * 2 * 32 * MT_ * kPfRowBytes, stream, \
                        act, wq, M, N, K, units, cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual)
-    if (tile == 4) {
+#define BITLINEAR_LAUNCH_PFX(MT_, CK_)                                                                                   \
+    BL_LAUNCH((gemm_i2_prefill_dma_kernel<MT_, 2, CK_>), grid, block, 3 * 32 * MT_ * CK_, stream, act, wq, M, N, K, units, \
+              cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual)
+    if (dma && dma_fits && ks == 1 && (tile == 8 || (tile == 1 && dma_mt == 4))) {
+        g_last_kernel = "gemm_i2_prefill_dma_kernel";
+        if (tile == 8) {
+            if (K % 256 == 0) BITLINEAR_LAUNCH_PFX(1, 256);
+            else BITLINEAR_LAUNCH_PFX(1, 128);
+        } else {
+            BITLINEAR_LAUNCH_PFX(4, 128);
+        }
+    } else if (tile == 4) {
         if (ks == 4) {
             BITLINEAR_LAUNCH_PF(1, 1, 4);
         } else if (ks == 2) {
@@ -2930,12 +2955,8 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
             BITLINEAR_LAUNCH_PF(2, 2, 2);
         } else if (dma && dma_fits) {
             g_last_kernel = "gemm_i2_prefill_dma_kernel";
-            if (K % 256 == 0)
-                BL_LAUNCH((gemm_i2_prefill_dma_kernel<2, 2, 256>), grid, block, 3 * 64 * 256, stream, act, wq, M, N, K, units,
-                          cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual);
-            else
-                BL_LAUNCH((gemm_i2_prefill_dma_kernel<2, 2, 128>), grid, block, 3 * 64 * 128, stream, act, wq, M, N, K, units,
-                          cseg_shift | (out ? 256 : 0), band, seg_cols, s, out, acc_out, ws, smap, residual);
+            if (K % 256 == 0) BITLINEAR_LAUNCH_PFX(2, 256);
+            else BITLINEAR_LAUNCH_PFX(2, 128);
         } else {
             BITLINEAR_LAUNCH_PF(2, 2, 1);
         }
@@ -2945,6 +2966,7 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
         BITLINEAR_LAUNCH_PF(2, 1, 1);
     }
 #undef BITLINEAR_LAUNCH_PF
+#undef BITLINEAR_LAUNCH_PFX
     return launch_status();
 }
 
@@ -3323,7 +3345,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
-        if (a < 0 || a > 5 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 0 || a > 7 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
         g.path = 5;
         g.prefill_big = a;
         g.prefill_band = b;
