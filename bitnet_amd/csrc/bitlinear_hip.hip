@@ -21,6 +21,7 @@
 // epilogue (gpu/bitnet_kernels/bitnet_kernels.h:79-82) is applied.
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <type_traits>
@@ -2179,6 +2180,157 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_i2_solo_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// BitLinearKernel.forward for up to eight tokens in one launch: every lane quantizes for its own token
+// ---------------------------------------------------------------------------
+// gemv_i2_solo_kernel's decomposition (a workgroup owns RPW 16-row blocks, S waves split K, UPW k-steps per
+// wave) with the quantizer in front of the products inside the wave.  The activation operand of a k-step is
+// 16 int8 of token p = lane % 16 for the 16 k of chunk g = lane / 16, and that is also how the bf16 rows are
+// read: lanes p and p + 8 share token p % 8 and load 8 of the 16 values behind that operand each, swapped with
+// one rotation inside the 16-lane row per register.  The tokens are quantized side by side, so a call with
+// eight tokens runs about the instructions of a call with one, and nothing passes through LDS in front of
+// the products but a token's slice maxima, exchanged between the waves behind one barrier.  Arithmetic,
+// rounding points and the +2 of the codes as in bitlinear_solo_kernel and gemv_i2_solo_kernel.
+// Measured per call against the quantizer kernel + gemv_i2_solo_kernel (HIP graph of dependent launches, distinct
+// weights): 3840 x 2560 at 5 / 8 tokens 4.80 -> 4.21 / 5.51 -> 4.59 us, 2560 x 2560 4.49 -> 4.15 / 5.39 -> 4.55,
+// 13824 x 2560 5.83 -> 5.56 / 6.61 -> 5.91.  Variants measured and left out: sixteen values per lane for nine to
+// sixteen tokens (twice the quantizer instructions per wave: 5.74 -> 5.79 at 12 tokens, 5.90 -> 6.64 at 16), rows
+// of 6912 values (16 waves of 7 k-steps: 7.42 -> 8.65 at 8 tokens), and the RMSNorm / gate prologues in front
+// (fp64 sums of squares per lane and a second exchange: 5.79 -> 5.72 at 8 tokens, level with the two launches).
+constexpr int kTokMaxTokens = 8;
+
+__device__ __forceinline__ uint32_t token_max_u32(uint32_t v) {
+    v = max(v, (uint32_t)__shfl_xor((int)v, 16));
+    v = max(v, (uint32_t)__shfl_xor((int)v, 32));
+    return max(v, (uint32_t)dpp_move<0x128>((int)v));  // row_ror:8: the lane with the token's other half
+}
+
+template <int UPW, int RPW>
+__global__ __launch_bounds__(kMaxWaves * 64) void bitlinear_solo_tok_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, int M, int N, int K, int rb_map, int S, int slot_rows,
+    const uint16_t* __restrict__ ws, uint16_t* __restrict__ out, int8_t* __restrict__ q_out, uint16_t* __restrict__ s_out,
+    int32_t* __restrict__ acc_out) {
+    __shared__ __attribute__((aligned(16))) int red[kSoloRedSlots][256];  // partial 16 x 16 tiles, [row block * S + k slice]
+    __shared__ uint32_t wmax[kMaxWaves][kTokMaxTokens];                   // a wave's slice maximum per token
+    const uint32_t slot_map = (uint32_t)rb_map >> 8;  // run j of slot_rows output rows reads ws[(slot_map >> 3 j) & 7]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int ks = __builtin_amdgcn_readfirstlane(tid >> 6);  // one group of waves per workgroup: the wave is the k slice
+    const int rb = blockIdx.x * RPW;                          // the wave's first row block
+    const int g = lane >> 4;
+    const int p = lane & 15;
+    const int tk = p & 7;     // the token this lane prepares
+    const int half = p >> 3;  // which 8 of the chunk's 16 values
+
+    // requests, all at once: the lane's vectors of its token's row (a token past M, or a k-step past the end of
+    // K, asks past the end of the descriptor: zeros, no access), then the weight words
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00020000);
+    const int slice_k0 = ks * (UPW * 64);
+    const int lane_k = slice_k0 + g * 16 + half * 8;
+    uint4 sv[UPW];
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) {
+        const int k = lane_k + j * 64;
+        const bool live = tk < M && k < K;  // K % 64 == 0: a k-step is inside K or outside
+        sv[j] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, live ? (tk * K + k) * 2 : 0x7ffffff0, 0, 0));
+    }
+    const int lane_word = (g >> 1) * 32 + (p >> 3) * 16 + (g & 1) * 8 + (p & 7);
+    const int w_voff = lane_word * 4 + ks * (UPW * 256);
+    uint32_t w[RPW][UPW];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+        // one descriptor per row block, spanning exactly its K * 4 bytes: a k-step past the end of K reads as zero
+        const bool rows_ok = rb + i < (N >> 4);
+        const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)((const char*)wq + (size_t)(rows_ok ? rb + i : 0) * K * 4), 0, rows_ok ? K * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) w[i][j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(w_rsrc, w_voff + j * 256, 0, 2 /* nt */);
+    }
+    const int n_first = blockIdx.x * RPW * 16;
+    const int n_last = (n_first + RPW * 16 - 1) < N ? (n_first + RPW * 16 - 1) : N - 1;
+    int slot_first = 0, slot_last = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSeg; ++j) {
+        slot_first += n_first >= j * slot_rows ? 1 : 0;
+        slot_last += n_last >= j * slot_rows ? 1 : 0;
+    }
+    const uint16_t wsb_first = ws[(slot_map >> (3 * slot_first)) & 7u];
+    const int nthreads = 64 * S;
+    __builtin_amdgcn_sched_barrier(0);  // every request above is on its way before anything below is looked at
+
+    // row maxima -> scales: the S waves cover all of K between them
+    uint32_t am = 0;
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) am = absmax_bits8(sv[j], am);
+    am = token_max_u32(am);
+    if (lane < kTokMaxTokens) wmax[ks][lane] = am;
+    lds_barrier();
+    am = 0;
+    for (int k = 0; k < S; ++k) am = max(am, wmax[k][tk]);
+    const float sf = quant_scale<0>(am);
+
+    // the lane's values -> int8 -> the MFMA's activation operands, in registers: lanes p < 8 hold values 0..7 of
+    // the chunk and fetch 8..15 from lane p + 8; the columns p >= 8 of the product belong to no token and are
+    // never read
+    v4i b[UPW];
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) {
+        const uint2 qv = quant_vec8<0>(sv[j], sf);
+        const int k = lane_k + j * 64;
+        if (blockIdx.x == 0 && q_out && tk < M && k < K) *(uint2*)(q_out + (size_t)tk * K + k) = qv;
+        b[j] = v4i{(int)qv.x, (int)qv.y, dpp_move<0x128>((int)qv.x), dpp_move<0x128>((int)qv.y)};
+    }
+    if (blockIdx.x == 0 && s_out && ks == 0 && lane < kTokMaxTokens && tk < M) s_out[tk] = f32_to_bf16_rne(sf);
+
+    // sum_k a[p, k] over the slice, in the accumulator layout (every row of the tile holds it)
+    const int ones_w = 0x01010101;
+    const v4i ones = {ones_w, ones_w, ones_w, ones_w};
+    v4i asum = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, b[j], asum, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < UPW; ++j) {
+            const uint32_t wj = w[i][j];  // zero past the end of K
+            v4i e;
+            e.x = (int)(wj & 0x03030303u);
+            e.y = (int)((wj >> 2) & 0x03030303u);
+            e.z = (int)((wj >> 4) & 0x03030303u);
+            e.w = (int)((wj >> 6) & 0x03030303u);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(e, b[j], acc, 0, 0, 0);
+        }
+        // lane holds token p, rows 4 g + i in register i
+        int* dst = &red[i * S + ks][lane];
+        dst[0] = acc.x - 2 * asum.x;
+        dst[64] = acc.y - 2 * asum.y;
+        dst[128] = acc.z - 2 * asum.z;
+        dst[192] = acc.w - 2 * asum.w;
+    }
+    lds_barrier();
+
+    // every thread finishes the output slots t = tid, tid + nthreads, ... of the workgroup: [row block][reg][lane];
+    // a slot's token is t % 16 = p, and for every token there is (p < 8) that is the token whose scale the lane holds
+#pragma unroll
+    for (int r = 0; r < kFusedMaxRB; ++r) {
+        const int t = tid + r * nthreads;
+        if (t >= RPW * 256) break;
+        const int l = t & 63;
+        const int m = l & 15;
+        const int tb = t >> 8;  // row block of the slot
+        const int n = (blockIdx.x * RPW + tb) * 16 + 4 * (l >> 4) + ((t >> 6) & 3);
+        if (m < M && n < N) {
+            int sum = 0;
+            for (int k = 0; k < S; ++k) sum += red[tb * S + k][t & 255];
+            if (acc_out) acc_out[(size_t)m * N + n] = sum;  // uniform: parity tests only
+            uint16_t wsb = wsb_first;
+            if (slot_first != slot_last) wsb = ws[(slot_map >> (3 * (n / slot_rows))) & 7u];  // uniform branch, rare
+            if (out) out[(size_t)m * N + n] = f32_to_bf16_rne((float)sum / sf * bf16_to_f32(wsb));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 thread_local int g_status = BITLINEAR_OK;
@@ -2207,6 +2359,7 @@ struct Tuning {
     int solo_rpw = 0;              // row blocks per wave: 0 = built-in choice, 1, 2, 4
     int prod_solo = 0;             // the drop-in product through gemv_i2_solo_kernel: 0 = built-in choice, 1 = always (prod_s waves of prod_upw k-steps), 2 = never
     int prod_s = 0, prod_upw = 0;
+    int tok = 0;  // forward for up to 8 tokens through bitlinear_solo_tok_kernel: 0 = built-in choice (from 5 tokens), 1 = wherever an instance exists, 2 = never
 };
 std::mutex g_tuning_mutex;
 Tuning g_tuning_shared;
@@ -2229,6 +2382,16 @@ namespace dispatch {
 // tokens above which the product is the MFMA GEMM instead of a GEMV kernel (the GEMV kernels hold at most 16
 // tokens: one MFMA column block)
 constexpr int kPrefillMinTokens = 16;
+// bitlinear_forward_bf16 from this many tokens up to eight (rows of up to 3200 values) in one launch through
+// bitlinear_solo_tok_kernel; below, the kernels for one to four tokens are ahead (3840 x 2560 at 4 tokens 4.14 us
+// against 4.24; at 5 tokens 4.80 against 4.21)
+constexpr int kTokMinTokens = 5;
+// ... and rows of up to this many values (waves of five k-steps, at most ten of them; 2560 x 6912 with 16 waves of
+// seven k-steps measured 7.42 us against 8.65 through this kernel at 8 tokens)
+constexpr int kTokMaxK = 3200;
+// ... and at most one workgroup per CU (3200 x 3200, 200 workgroups, at 8 tokens 6.03 -> 5.46 us; 4800 x 3200, 300
+// workgroups, 6.88 -> 7.35; 20480 x 3200, 640 workgroups, 10.04 -> 10.50)
+constexpr int kTokMaxWorkgroups = 256;
 // 16 < M <= this: GEMM or split-K GEMV by the estimate in launch_gemv (fitted to the 2B shapes; above it the
 // GEMM is always ahead)
 constexpr int kSplitKMaxTokens = 256;
@@ -2807,6 +2970,35 @@ int launch_prod_solo(const int8_t* act, const int8_t* packed, uint16_t* out, int
     return launch_status();
 }
 
+// bitlinear_solo_tok_kernel: launch shape as plan_prod_solo (S waves of UPW k-steps, RPW row blocks per wave);
+// instances exist for five k-steps per wave, which the plan chooses for rows of up to 3200 values, and one or
+// four row blocks per wave (two, the plan's choice from 432 row blocks on, measured behind the other kernels:
+// 8192 x 2048 at 5 tokens 4.70 us against 5.12).
+bool tok_plan_ok(int M, const ProdPlan& pl) {
+    return pl.ok && pl.upw == 5 && (pl.rpw == 1 || pl.rpw == 4) && M >= 1 && M <= kTokMaxTokens;
+}
+
+int launch_solo_tok(const uint16_t* x, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* ws,
+                    const ScaleMap& smap, int8_t* q_out, uint16_t* s_out, int M, int N, int K, const ProdPlan& pl,
+                    hipStream_t stream) {
+    const int blocks16 = N / 16;
+    const dim3 grid((blocks16 + pl.rpw - 1) / pl.rpw, 1, 1);
+    const dim3 block(64 * pl.s, 1, 1);
+    const uint32_t* wq = (const uint32_t*)packed;
+    const SlotRule rule = slot_rule(smap, N);
+    if (!rule.ok || !tok_plan_ok(M, pl)) return BITLINEAR_ERR_ARG;
+    const int slot_rows = rule.slot_rows;
+    const int rb_map = 1 | (int)(rule.map << 8);
+    g_last_kernel = "bitlinear_solo_tok_kernel";
+#define BITLINEAR_LAUNCH_TOK(W)                                                                                        \
+    BL_LAUNCH((bitlinear_solo_tok_kernel<5, W>), grid, block, 0, stream, x, wq, M, N, K, rb_map, pl.s, slot_rows, ws, \
+              out, q_out, s_out, acc_out)
+    if (pl.rpw == 1) BITLINEAR_LAUNCH_TOK(1);
+    else BITLINEAR_LAUNCH_TOK(4);
+#undef BITLINEAR_LAUNCH_TOK
+    return launch_status();
+}
+
 int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32_t* acc_out, const uint16_t* s,
                    const uint16_t* ws, const ScaleMap& smap, int M, int N, int K, hipStream_t stream,
                    const uint16_t* residual = nullptr) {
@@ -3258,6 +3450,8 @@ const char* bitlinear_status_string(int status) {
         case BITLINEAR_ERR_ARG: return "invalid argument";
         case BITLINEAR_ERR_SCRATCH:
             return "activation block beyond the static scratch (need M <= 16384 and M * K <= 16744448)";
+        case BITLINEAR_ERR_CAPTURE:
+            return "bitlinear_forward_bf16_static: the first call on a device must come from outside a stream capture";
         default: return "unknown status";
     }
 }
@@ -3272,7 +3466,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);
     Tuning& g = g_tuning_shared;
     if (kernel == 0) {
-        g.path = g.waves = g.upw = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = g.prod_solo = 0;
+        g.path = g.waves = g.upw = g.staged = g.stream = g.stream_depth = g.stream_waves = g.solo = g.solo_coop = g.solo_rpw = g.prod_solo = g.tok = 0;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 6) {
@@ -3292,6 +3486,11 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         if (a < 0 || a > 2 || b < 0 || b > 4) return set_status(BITLINEAR_ERR_ARG);
         g.solo_coop = a;
         g.solo_rpw = b;
+        return set_status(BITLINEAR_OK);
+    }
+    if (kernel == 11) {
+        if (a < 0 || a > 2) return set_status(BITLINEAR_ERR_ARG);
+        g.tok = a;
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 10) {
@@ -3533,6 +3732,13 @@ static int forward_impl(const uint16_t* x, const int8_t* packed, uint16_t* outpu
         if (sp.ok && (t_tune.solo >= 1 || solo_wanted(M, N, K)))
             return set_status(launch_solo(x, packed, output0, acc_out, ws, sm, q_ws, s_ws, M, N, K, sp, (hipStream_t)stream));
     }
+    // five to eight tokens, rows of up to 3200 values: the kernel whose lanes quantize for their own token
+    if (mode == 0 && t_tune.path == 0 && t_tune.tok != 2 && M <= kTokMaxTokens && (t_tune.tok == 1 || (M >= kTokMinTokens && K <= kTokMaxK)) &&
+        (long long)M * K * 2 < 0x7ffffff0ll && slot_rule(sm, N).ok) {
+        const ProdPlan tp = plan_prod_solo(M, N, K);
+        if (tok_plan_ok(M, tp) && (t_tune.tok == 1 || (N / 16 + tp.rpw - 1) / tp.rpw <= kTokMaxWorkgroups))
+            return set_status(launch_solo_tok(x, packed, output0, acc_out, ws, sm, q_ws, s_ws, M, N, K, tp, (hipStream_t)stream));
+    }
     const FusedPlan pl = plan_fused(M, N, K);
     // one kernel while the activation block is small enough for every workgroup to quantize it
     // again (or when the caller gave no workspaces for the two-kernel path)
@@ -3562,10 +3768,11 @@ int bitlinear_forward_bf16_seg(const uint16_t* x, const int8_t* packed, uint16_t
 
 // The array's name is only a handle on the host: its device address is looked up once per device
 // (each GPU has its own copy) and kept.
-static unsigned char* static_scratch_ptr(hipError_t* err) {
+static unsigned char* static_scratch_ptr(hipError_t* err, hipStream_t stream, bool* refused_under_capture) {
     static std::once_flag flags[bitnet_host::kMaxDevices];
     static unsigned char* ptrs[bitnet_host::kMaxDevices];
     static hipError_t results[bitnet_host::kMaxDevices];
+    static std::atomic<bool> known[bitnet_host::kMaxDevices];
     int dev = 0;
     *err = hipGetDevice(&dev);
     if (*err != hipSuccess) return nullptr;
@@ -3573,10 +3780,20 @@ static unsigned char* static_scratch_ptr(hipError_t* err) {
         *err = hipErrorInvalidDevice;
         return nullptr;
     }
+    if (!known[dev].load()) {
+        // the look-up below is a host call that a stream capture in progress may refuse: the first call on a
+        // device has to come from outside a capture, and says so instead of failing in some other way
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+            *refused_under_capture = true;
+            return nullptr;
+        }
+    }
     std::call_once(flags[dev], [dev] {
         void* p = nullptr;
         results[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         ptrs[dev] = results[dev] == hipSuccess ? (unsigned char*)p : nullptr;
+        known[dev].store(results[dev] == hipSuccess);
     });
     *err = results[dev];
     return ptrs[dev];
@@ -3588,7 +3805,9 @@ int bitlinear_forward_bf16_static(const uint16_t* x, const int8_t* packed, uint1
     if (M > kStaticMaxTokens || (size_t)M * (size_t)K > kStaticMaxElems) return set_status(BITLINEAR_ERR_SCRATCH);
     if (!x || !packed || !output0 || !ws) return set_status(BITLINEAR_ERR_NULL);
     hipError_t err = hipSuccess;
-    unsigned char* base = static_scratch_ptr(&err);
+    bool under_capture = false;
+    unsigned char* base = static_scratch_ptr(&err, (hipStream_t)stream, &under_capture);
+    if (under_capture) return set_status(BITLINEAR_ERR_CAPTURE);
     if (err != hipSuccess || !base) return set_status(BITLINEAR_ERR_LAUNCH);
     return forward_impl(x, packed, output0, nullptr, ws, (int8_t*)(base + kStaticScaleBytes), (uint16_t*)base, M, N, K, mode,
                         stream);

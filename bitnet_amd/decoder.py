@@ -95,8 +95,17 @@ class AttnWorkspace:
         output (bitnet_attn_decode_error_index)."""
         return int(self.partials[self.error_index : self.error_index + 1].view(torch.int32).item())
 
+    def reset(self) -> None:
+        """Back to the state of a fresh workspace (zero records, epochs and error word).  Not inside a graph
+        capture; graphs captured on this workspace keep working, since they hold its buffers, not their contents."""
+        self.partials.zero_()
+        self.counters.zero_()
+
     def check(self) -> None:
+        """Raises if a merge gave up since the last check, and clears the condition: one failed call is reported
+        once and does not poison the object (later calls compute healthy results again)."""
         if self.error():
+            self.reset()
             raise _lib.BitLinearLibraryError(
                 "attention decode: a merge of the split records gave up (workspace not zeroed before its first use, "
                 "or shared between overlapping calls); the affected output rows are NaN"
@@ -541,7 +550,12 @@ class Generator:
         with torch.cuda.graph(self.graph):
             self._step()
 
-    kMaxPrefillGraphs = 12  # distinct (prompt length, logits) pairs kept captured; further ones run launch by launch
+    kMaxPrefillGraphs = 12  # captured prompt passes kept; the least recently replayed one makes room for a new one
+    kPrefillBucket = 32  # prompts are padded to a multiple of this many tokens, so that lengths share captured passes
+
+    def _bucket(self, P: int) -> int:
+        b = self.kPrefillBucket
+        return min(self.max_seq, (P + b - 1) // b * b)
 
     def _prefill_fused(self, prompt, lens, tok_out, logits):
         """The prompt through the library's kernels; only each sequence's last real token goes through the LM head."""
@@ -550,17 +564,24 @@ class Generator:
         return lm_head_greedy(last, self.model.norm, self.model.output.weight, self.lm_ws, token_out=tok_out, logits_out=logits)
 
     def _prefill_replay(self, prompt: torch.Tensor, lens: Optional[torch.Tensor], want_logits: bool):
-        """prompt [B, P] (padded) through the captured pass for this length: (first token [B], logits or None)."""
+        """prompt [B, P] (padded) through the captured pass of P's bucket: (first token [B], logits or None).
+        The pass runs on the prompt padded further, with token 0, to the bucket's length; every sequence's real
+        length travels in `lens` (attention is causal, so the pads change no real token's result, and the cache rows
+        they write are overwritten before a decode step reads them).  The captured passes are therefore at most
+        two per bucket, and beyond kMaxPrefillGraphs the least recently replayed one is dropped."""
         B, P = prompt.shape
-        key = (P, want_logits)
-        entry = self._pf_graphs.get(key)
+        Pb = self._bucket(P)
+        key = (Pb, want_logits)
+        entry = self._pf_graphs.pop(key, None)
         if entry is None:
+            while len(self._pf_graphs) >= self.kMaxPrefillGraphs:
+                self._pf_graphs.pop(next(iter(self._pf_graphs)))  # dicts keep insertion order: the oldest entry
             dev = self.tok.device
-            bufs = {"prompt": torch.zeros(B, P, dtype=torch.int64, device=dev),
+            bufs = {"prompt": torch.zeros(B, Pb, dtype=torch.int64, device=dev),
                     "lens": torch.full((B,), P, dtype=torch.int64, device=dev),
                     "tok": torch.zeros(B, dtype=torch.int64, device=dev),
                     "logits": torch.empty(B, self.model.args.vocab_size, dtype=torch.float32, device=dev) if want_logits else None}
-            bufs["prompt"].copy_(prompt)
+            bufs["prompt"][:, :P].copy_(prompt)
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -570,9 +591,12 @@ class Generator:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 self._prefill_fused(bufs["prompt"], bufs["lens"], bufs["tok"], bufs["logits"])
-            entry = self._pf_graphs[key] = (graph, bufs)
+            entry = (graph, bufs)
+        self._pf_graphs[key] = entry  # (re-)inserted last: most recently used
         graph, bufs = entry
-        bufs["prompt"].copy_(prompt)
+        bufs["prompt"][:, :P].copy_(prompt)
+        if P < Pb:
+            bufs["prompt"][:, P:].zero_()
         if lens is None:
             bufs["lens"].fill_(P)
         else:
@@ -585,7 +609,7 @@ class Generator:
         """prompt [B, P] int64 -> first generated token [B]."""
         B, P = prompt.shape
         if self.lm_head:
-            if self.use_graph and B == self.batch and ((P, False) in self._pf_graphs or len(self._pf_graphs) < self.kMaxPrefillGraphs):
+            if self.use_graph and B == self.batch:
                 return self._prefill_replay(prompt, None, False)[0]
             lens = torch.full((B,), P, dtype=torch.int64, device=prompt.device)
             rows = self._rows if B == self.batch else torch.arange(B, device=prompt.device)
@@ -658,7 +682,7 @@ class Generator:
         rows = self._rows
         V = self.model.args.vocab_size
         if self.lm_head:
-            if self.use_graph and ((P, want_logits) in self._pf_graphs or len(self._pf_graphs) < self.kMaxPrefillGraphs):
+            if self.use_graph:
                 tok, logits = self._prefill_replay(prompt, lens, want_logits)
                 return tok, logits, lens
             logits = torch.empty(self.batch, V, dtype=torch.float32, device=dev) if want_logits else None
@@ -711,8 +735,9 @@ class Generator:
             torch.cuda.synchronize()
             t_prefill = time.perf_counter()
         out = [first.view(1, -1)]
-        stop = eos_id is not None and bool((first == eos_id).any())
-        if gen_length > 1 and not stop:
+        # (an end token that comes out of the prompt pass does not end the batch: the reference tests for it only
+        # inside its decode loop, gpu/generate.py:262-284; the answers are trimmed per sequence below)
+        if gen_length > 1:
             if not use_sampling:
                 out.append(self.decode(first, lens, gen_length - 1, eos_id=eos_id))
             else:

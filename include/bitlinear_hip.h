@@ -33,6 +33,8 @@ extern "C" {
                                    an operand not 16-byte aligned           */
 #define BITLINEAR_ERR_SCRATCH 5 /* bitlinear_forward_bf16_static: the
                                    activation block exceeds the static scratch */
+#define BITLINEAR_ERR_CAPTURE 6 /* bitlinear_forward_bf16_static: first call on a
+                                   device made under a stream capture        */
 
 /*
  * Drop-in replacement for the reference's only exported symbol
@@ -191,10 +193,14 @@ int bitlinear_forward_bf16(const uint16_t* x, const int8_t* packed,
  * the library's device image (one copy per GPU, held until the process ends).
  * Limits: M <= 16384 tokens and M * K <= 16744448 activation elements (the
  * largest prompt block of the 2B shapes, 2048 x 6912, fits); beyond them the
- * call launches nothing and returns BITLINEAR_ERR_SCRATCH.  Same kernels and
+ * call launches nothing and returns BITLINEAR_ERR_SCRATCH.  The array costs its
+ * 16 MiB of device memory in every process that loads the library, on every GPU
+ * it uses, whether or not this entry is ever called.  Same kernels and
  * the same bits as bitlinear_forward_bf16.  Allocates nothing and frees
  * nothing; the first call on a device looks the array's address up (a host
- * call, not stream work).  All calls on one GPU share the array: two of them
+ * call, not stream work, which a stream capture in progress may refuse: made
+ * under a capture, that first call launches nothing and returns
+ * BITLINEAR_ERR_CAPTURE; every later call may be captured).  All calls on one GPU share the array: two of them
  * must not overlap in time (same stream, or ordered by events), or they race
  * on the quantized rows.  Nothing in the array needs clearing between calls:
  * every element the product reads was written by the same call's quantizer.
@@ -329,6 +335,13 @@ int bitlinear_plan_name(int entry, int M, int N, int K, char* buf, int buflen);
  *             and c (4, 5, 7 or 8) k-steps per wave (b * c * 64 must cover K,
  *             else the built-in kernels run; row blocks per wave from kernel 9's
  *             b), a = 2 never.  Applies with kernel 0 only; kernel 0 resets it.
+ *   kernel 11: bitlinear_forward_bf16 (mode 0, M <= 8) in one launch through the
+ *             kernel whose lanes quantize for their own token: a = 0 built-in
+ *             choice (5 to 8 tokens, K <= 3200, at most 256 workgroups), 1 wherever
+ *             its launch shape exists (waves of five k-steps cover K, one or four
+ *             row blocks per wave; the kernel 8 setting a = 5
+ *             keeps the one-to-four-token kernel out of the way), 2 never.
+ *             Applies with kernel 0 only; kernel 0 resets it.
  */
 int bitlinear_set_tuning(int kernel, int a, int b, int c);
 

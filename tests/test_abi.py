@@ -76,7 +76,8 @@ def test_host_only_entry_points():
     assert lib.bitlinear_set_tuning(9, 1, 4, 0) == 0 and lib.bitlinear_set_tuning(9, 1, 5, 0) != 0
     assert lib.bitlinear_set_tuning(10, 1, 8, 5) == 0 and lib.bitlinear_set_tuning(10, 2, 0, 0) == 0
     assert lib.bitlinear_set_tuning(10, 1, 8, 6) != 0 and lib.bitlinear_set_tuning(10, 3, 0, 0) != 0
-    assert lib.bitlinear_set_tuning(11, 0, 0, 0) != 0
+    assert lib.bitlinear_set_tuning(11, 1, 0, 0) == 0 and lib.bitlinear_set_tuning(11, 2, 0, 0) == 0
+    assert lib.bitlinear_set_tuning(11, 3, 0, 0) != 0 and lib.bitlinear_set_tuning(12, 0, 0, 0) != 0
     assert lib.bitlinear_set_tuning(0, 0, 0, 0) == 0
 
 

@@ -23,13 +23,14 @@ def test_dispatch_matches_the_committed_table():
 
 def test_plan_rows_say_what_the_design_says():
     """A few rows spelled out, so that the table cannot drift as a whole: one token goes through the kernel whose
-    waves prepare their own slices, five to sixteen tokens through a quantizer kernel plus the product without
-    staging, more than sixteen through the MFMA GEMM, the largest matrix through the streaming kernel."""
+    waves prepare their own slices, five to eight tokens (short rows) through the kernel whose lanes quantize for their
+    own token, up to sixteen through a quantizer kernel plus the product without staging, more than sixteen through the MFMA GEMM, the largest matrix through the streaming kernel."""
     p = _lib.plan_name
     assert p(1, 1, 2560, 2560).startswith("bitlinear_solo_kernel<5, 5, 1, false, 0, false, 1> grid=(160,1,1) block=512")
     assert p(1, 1, 13824, 2560).startswith("bitlinear_solo_kernel<5, 5, 1, false, 0, false, 4> grid=(216,1,1)")
     assert p(2, 1, 3840, 2560).startswith("bitlinear_solo_kernel<5, 1, 1, true, 1, false, 1>")
-    two = p(1, 8, 3840, 2560).split(" + ")
+    assert p(1, 8, 3840, 2560).startswith("bitlinear_solo_tok_kernel<5, 1> grid=(240,1,1) block=512")
+    two = p(1, 16, 3840, 2560).split(" + ")
     assert len(two) == 2 and two[0].startswith("quant_absmax_rows_kernel<0, 5>") and two[1].startswith("gemv_i2_solo_kernel<5, 1, false>")
     assert "gemm_i2_prefill_kernel" in p(0, 17, 13824, 2560) and "gemm_i2_prefill_dma_kernel<2, 2, 256>" in p(0, 2048, 13824, 2560)
     assert p(0, 1, 55296, 5120).startswith("gemv_i2_stream_kernel<5, true>")

@@ -1122,6 +1122,65 @@ def test_forward_kernel_whose_waves_quantize_their_own_slices(n, k, m, shape, co
     _assert_bits_equal(host_bits(out4), want1, "mode 1")
 
 
+TOK_SHAPES = [(2560, 2560), (3840, 2560), (13824, 2560), (7008, 2560), (1040, 3200), (48, 192), (176, 4480), (64, 5120),
+              (2560, 6912)]
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 7, 8, 9])
+@pytest.mark.parametrize("n,k", TOK_SHAPES)
+def test_forward_kernel_whose_lanes_quantize_for_their_own_token(n, k, m):
+    """bitlinear_solo_tok_kernel (one launch for up to eight tokens; the library's choice from five tokens on for
+    rows of up to 3200 values): int32 accumulators, bf16 outputs and the q / s workspaces bit for bit against the
+    oracle chain, with and without workspaces, over 1 and 4 row blocks per wave, one to sixteen waves, K that
+    the waves do not divide, three scale slots; where the kernel has no launch shape (nine tokens, K = 6912, 7008
+    rows) the other kernels give the same."""
+    lib = _lib.load_library()
+    rng = np.random.default_rng(n + 3 * k + m)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    x = rng.standard_normal((m, k)).astype(np.float32) * rng.choice([0.05, 1.0, 30.0], size=(m, 1)).astype(np.float32)
+    x[m // 2, ::5] *= 20.0
+    x[m - 1, k - 1] = 97.0  # the last token's maximum sits in the last wave's slice
+    xb = o.f32_to_bf16_bits(x)
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    q, s_bits = o.quant_input(xb, 0)
+    acc_want, want = o.bitlinear_int8xint2(q, w, s_bits, ws_bits)
+    pk = _packed_dev(w)
+    # the launch plan's row blocks per wave: two from 432 row blocks on (four from 864 on with more than four
+    # tokens), and for two there is no instance
+    rpw = 1 if n // 16 < 432 else (4 if n // 16 >= 864 and m > 4 else 2)
+    applies = m <= 8 and k != 6912 and rpw != 2
+    try:
+        if 5 <= m <= 8 and k <= 3200 and applies:  # the library's own choice
+            st, out0, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
+            assert st == 0 and bitlinear.last_kernel() == "bitlinear_solo_tok_kernel"
+            _assert_bits_equal(host_bits(out0), want, "built-in choice")
+        assert lib.bitlinear_set_tuning(8, 5, 0, 0) == 0  # not the one-to-four-token kernel
+        assert lib.bitlinear_set_tuning(11, 1, 0, 0) == 0
+        out, acc = bitlinear.bitlinear_forward_acc(dev_bf16(xb), pk, dev_bf16(ws_bits))
+        assert (bitlinear.last_kernel() == "bitlinear_solo_tok_kernel") == applies
+        st, out2, qd, sd = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
+        assert st == 0 and (bitlinear.last_kernel() == "bitlinear_solo_tok_kernel") == applies
+        st, out3, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0, with_ws=False)
+        if not applies and st == 2:  # a block that only the two-kernel path takes needs the workspaces
+            out3 = out2
+        assert st == 0 or not applies
+        st, out4, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 1)  # quantizer mode 1: the other kernels
+        assert st == 0 and bitlinear.last_kernel() != "bitlinear_solo_tok_kernel"
+        assert lib.bitlinear_set_tuning(11, 2, 0, 0) == 0
+        st, out5, _, _ = _forward_raw(lib, xb, pk, ws_bits, m, n, k, 0)
+        assert st == 0 and bitlinear.last_kernel() != "bitlinear_solo_tok_kernel"
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    for t, what in ((out, "forward + acc"), (out2, "forward"), (out3, "forward without workspaces"), (out5, "switched off")):
+        _assert_bits_equal(host_bits(t), want, what)
+    assert np.array_equal(qd.cpu().numpy(), q)
+    assert np.array_equal(host_bits(sd), s_bits)
+    q1, s1 = o.quant_input(xb, 1)
+    _, want1 = o.bitlinear_int8xint2(q1, w, s1, ws_bits)
+    _assert_bits_equal(host_bits(out4), want1, "mode 1")
+
+
 @pytest.mark.parametrize("norm", [0, 1])
 @pytest.mark.parametrize("coop", [1, 2])
 @pytest.mark.parametrize("rpw", [0, 2, 3, 4])

@@ -444,11 +444,16 @@ def test_attention_merge_that_gives_up_is_reported():
     assert torch.isnan(bad[0].float()).all()           # every head of the sequence whose splits had to be merged
     assert torch.equal(bad[1], good[1])                # the single-split sequence is not affected
     assert ws.error() == 1
-    with pytest.raises(_lib.BitLinearLibraryError):
-        ws.check()
     again = decoder.attn_decode(xqkv, ck.clone(), cv.clone(), pos, cos, sin, nh, nkv, ws)
     torch.cuda.synchronize()
-    assert torch.equal(again, good) and ws.error() == 1  # results recover, the word is sticky
+    assert torch.equal(again, good) and ws.error() == 1  # results recover; the word stays until someone looks
+    with pytest.raises(_lib.BitLinearLibraryError):
+        ws.check()
+    assert ws.error() == 0                              # reported once: check() put the workspace back to its fresh state
+    ws.check()
+    once_more = decoder.attn_decode(xqkv, ck.clone(), cv.clone(), pos, cos, sin, nh, nkv, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(once_more, good) and ws.error() == 0
     ws2 = decoder.AttnWorkspace(B, nh, nkv, n_splits, dev)
     fresh = decoder.attn_decode(xqkv, ck.clone(), cv.clone(), pos, cos, sin, nh, nkv, ws2)
     assert torch.equal(fresh, good) and ws2.error() == 0
@@ -747,7 +752,9 @@ def test_generate_all_stops_at_the_end_token_and_trims_the_answers():
     full = gen.generate_all(prompts, 16)
     # take a token that sequence 1 produces at step 5 as the end token
     eos = full[1][5]
-    first_hit = min(min(a.index(eos) for a in full if eos in a), 15)
+    # the loop ends after the first DECODE step (index >= 1) in which any sequence produced it: a hit in the
+    # prompt pass's own token does not end the batch (gpu/generate.py:262-284)
+    first_hit = min([a.index(eos, 1) for a in full if eos in a[1:]] + [15])
     timings = {}
     cut = gen.generate_all(prompts, 16, eos_id=eos, timings=timings)
     assert timings["decode_tokens"] == 2 * (len(max(cut, key=len)) - 1) or timings["decode_tokens"] == 2 * first_hit
@@ -778,9 +785,10 @@ def test_generate_all_sampling_is_reproducible_and_greedy_for_a_tiny_nucleus():
 
 
 def test_captured_prompt_pass_equals_the_launch_by_launch_one():
-    """Generator.prefill replays one captured graph per prompt length; every replay, with other work of the
-    program in between (decode steps, prompts of other lengths), gives the tokens, and leaves the cache rows,
-    of the same pass issued launch by launch."""
+    """Generator.prefill replays one captured graph per bucket of prompt lengths (multiples of 32 tokens, the
+    prompt padded up to the bucket); every replay, with other work of the program in between (decode steps,
+    prompts of other lengths), gives the tokens, and leaves the cache rows, of the unpadded pass issued launch by
+    launch.  Beyond kMaxPrefillGraphs captured passes the least recently used one is dropped."""
     model = _build(BIG_HEADS, seed=8)
     dev = torch.device("cuda")
     g = torch.Generator(device="cuda").manual_seed(21)
@@ -798,7 +806,16 @@ def test_captured_prompt_pass_equals_the_launch_by_launch_one():
         d1 = graphed.decode(t1, P, 5)
         d2 = eager.decode(t2, P, 5)
         assert torch.equal(d1, d2)
-    assert sorted(k[0] for k in graphed._pf_graphs) == [7, 24, 40]
+    assert sorted(k[0] for k in graphed._pf_graphs) == [32, 64]  # 7 and 24 share a pass, 40 has the other
+    # a bucket cut short by the cache's capacity, and the bound on the passes kept
+    graphed.kMaxPrefillGraphs = 2
+    prompt = torch.randint(0, BIG_HEADS.vocab_size, (2, 70), generator=g, device=dev)
+    assert torch.equal(graphed.prefill(prompt), eager.prefill(prompt))
+    assert [k[0] for k in graphed._pf_graphs] == [64, 96]  # 32, replayed longest ago, made room
+    prompt = torch.randint(0, BIG_HEADS.vocab_size, (2, 9), generator=g, device=dev)
+    assert torch.equal(graphed.prefill(prompt), eager.prefill(prompt))
+    assert [k[0] for k in graphed._pf_graphs] == [96, 32]
+    graphed.kMaxPrefillGraphs = 12
     # ragged prompts go through the same captured pass with their own lengths
     prompts = [torch.randint(2, BIG_HEADS.vocab_size, (n,), generator=torch.Generator().manual_seed(n)).tolist() for n in (40, 13)]
     assert graphed.generate_all(prompts, 6) == eager.generate_all(prompts, 6)

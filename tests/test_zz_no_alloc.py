@@ -81,3 +81,59 @@ def test_static_scratch_forward_in_a_graph_and_size_limit():
     assert lib.bitlinear_forward_bf16_static(_P(x), _P(pk), _P(out_g), _P(ws), 16385, n, 64, 0, None) == 5
     assert lib.bitlinear_forward_bf16_static(_P(x), _P(pk), _P(out_g), _P(ws), 4096, n, 4160, 0, None) == 5
     assert b"static scratch" in lib.bitlinear_status_string(5)
+    assert b"capture" in lib.bitlinear_status_string(6)
+
+
+def test_static_scratch_forward_at_the_exact_limit():
+    """M * K = 16 MiB - 32 KiB = 16744448 elements (511 rows of 32768) is the largest block the scratch holds: it
+    runs, bit-equal to the workspace entry; one row more is refused before anything is launched."""
+    lib = _lib.load_library()
+    m, n, k = 511, 16, 32768
+    assert m * k == (16 << 20) - 2 * 16384
+    rng = np.random.default_rng(9)
+    w = rng.integers(-1, 2, size=(n, k), dtype=np.int8)
+    pk = pack_weight.convert_weight_int8_to_int2(torch.from_numpy(w)).cuda()
+    ws = dev_bf16(o.f32_to_bf16_bits(np.array([0.02, 0, 0, 0], dtype=np.float32)))
+    x = dev_bf16(o.f32_to_bf16_bits(rng.standard_normal((m + 1, k)).astype(np.float32)))
+    out_s, out_w = _both(lib, x, pk, ws, m, n, k)
+    assert torch.equal(out_s.view(torch.int16), out_w.view(torch.int16))
+    assert not torch.isnan(out_s.float()).any()
+    out = torch.zeros(m + 1, n, dtype=torch.bfloat16, device="cuda")
+    assert lib.bitlinear_forward_bf16_static(_P(x), _P(pk), _P(out), _P(ws), m + 1, n, k, 0, None) == 5
+
+
+def test_first_static_call_on_a_device_under_capture_says_so():
+    """In a fresh process whose first call of the entry sits inside a stream capture, the call launches nothing and
+    returns the status of its own (6); after one call outside a capture, the captured call works."""
+    import subprocess
+    import sys
+    code = r"""
+import ctypes, torch
+from bitnet_amd import _lib
+lib = _lib.load_library()
+P = lambda t: ctypes.c_void_p(t.data_ptr())
+m, n, k = 4, 16, 256
+x = torch.randn(m, k, device="cuda").bfloat16()
+pk = torch.zeros(n // 4, k, dtype=torch.int8, device="cuda")
+ws = torch.ones(4, device="cuda").bfloat16()
+out = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+torch.cuda.synchronize()
+g = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g):
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    first = lib.bitlinear_forward_bf16_static(P(x), P(pk), P(out), P(ws), m, n, k, 0, sp)
+    torch.zeros(1, device="cuda")
+torch.cuda.synchronize()
+eager = lib.bitlinear_forward_bf16_static(P(x), P(pk), P(out), P(ws), m, n, k, 0, None)
+torch.cuda.synchronize()
+g2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g2):
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    later = lib.bitlinear_forward_bf16_static(P(x), P(pk), P(out), P(ws), m, n, k, 0, sp)
+g2.replay()
+torch.cuda.synchronize()
+print("STATUS", first, eager, later)
+"""
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "STATUS 6 0 0" in r.stdout, r.stdout + r.stderr[-2000:]
