@@ -354,15 +354,51 @@ def batched_and_prefill(lib, shapes, layers, scales, dev, decode_ms=(2, 4, 8, 16
             tot_us += res[1]
             tot_fwd_us += res[0]
         tops = tot_ops / (tot_us * 1e-6) / 1e12
+        vendor = vendor_int8_gemm(shapes, M, dev) if M >= 512 else None
         out["prefill"][f"M{M}"] = {
+            **({"vendor_int8_gemm": vendor} if vendor else {}),
             "per_shape": per,
             "layer_gemm_TOPS": round(tops, 1),
             "layer_forward_TOPS": round(tot_ops / (tot_fwd_us * 1e-6) / 1e12, 1),
             "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": round(tops / INT8_MFMA_PEAK_TOPS, 4), "kernel": "gemm_i2_prefill_kernel, the four 2B shapes of one layer"},
+                         "frac": round(tops / INT8_MFMA_PEAK_TOPS, 4), "kernel": "gemm_i2_prefill_dma_kernel (gemm_i2_prefill_kernel where K % 128 != 0), the four 2B shapes of one layer"},
             "prefill_tokens_per_s_bitlinear_only": round(M / (tot_fwd_us * 1e-6 * len(layers)), 1),
         }
     return out
+
+
+def vendor_int8_gemm(shapes, M, dev, reps=20):
+    """For scale, not part of the product: the platform library's int8 x int8 -> int32 GEMM (torch._int_mm) on
+    the same four shapes, with the ternary weights already expanded to one byte each (four times the weight
+    bytes of the packed form, no 2-bit decode, no scaling epilogue, int32 outputs), the faster of its two
+    operand layouts per shape.  Not fatal when the library refuses a shape."""
+    import torch
+
+    per, tot_us, tot_ops = {}, 0.0, 0.0
+    try:
+        for sh in shapes:
+            a = torch.randint(-127, 128, (M, sh.K), dtype=torch.int8, device=dev)
+            best = None
+            for b in (torch.randint(-1, 2, (sh.K, sh.N), dtype=torch.int8, device=dev),
+                      torch.randint(-1, 2, (sh.N, sh.K), dtype=torch.int8, device=dev).t()):
+                for _ in range(3):
+                    torch._int_mm(a, b)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(reps):
+                    torch._int_mm(a, b)
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / reps
+                best = us if best is None else min(best, us)
+            per[sh.name] = round(best, 2)
+            tot_us += best
+            tot_ops += 2.0 * M * sh.N * sh.K
+    except Exception as e:  # a measurement for comparison only
+        return {"error": f"{type(e).__name__}: {str(e)[:160]}"}
+    return {"what": "torch._int_mm (int8 weights, int32 out), us per call, eager launches back to back", "per_shape_us": per,
+            "layer_TOPS": round(tot_ops / (tot_us * 1e-6) / 1e12, 1)}
 
 
 def mfma_ceiling(lib, dev, iters=20000):
@@ -647,9 +683,23 @@ def end_to_end_decode(batches=(1, 8), prompt_len=512, gen_len=128):
         toks = gen.decode(first, prompt_len, gen_len - 1)
         torch.cuda.synchronize()
         t3 = time.perf_counter()
+        a = model.args
+        hd = a.dim // a.n_heads
+        # bytes a decode step must move at least: every packed weight matrix once, the bf16 LM head (the tied
+        # embedding) once, and the cache rows 0 .. position of every layer (k and v) for every sequence
+        w_bytes = a.n_layers * ((a.dim + 2 * a.n_kv_heads * hd) * a.dim + a.dim * a.dim + 2 * a.ffn_dim * a.dim + a.dim * a.ffn_dim) // 4
+        lm_bytes = a.vocab_size * a.dim * 2
+        mean_pos = prompt_len + (gen_len - 1) / 2.0
+        kv_bytes = int(B * a.n_layers * 2 * a.n_kv_heads * hd * 2 * mean_pos)
+        step_s = (t3 - t2) / (gen_len - 1)
+        step_gbps = (w_bytes + lm_bytes + kv_bytes) / step_s / 1e9
         out[f"batch{B}"] = {
             "decode_tokens_per_s": round(B * (gen_len - 1) / (t3 - t2), 1),
             "ms_per_decode_step": round((t3 - t2) * 1e3 / (gen_len - 1), 4),
+            "roofline": {"bound": "hbm", "achieved": round(step_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(step_gbps / HBM_PEAK_GBPS, 4),
+                         "bytes_per_step": {"packed_weights": w_bytes, "lm_head_bf16": lm_bytes, "kv_cache_mean": kv_bytes},
+                         "what": "one whole decode step (all launches of the captured graph), wall clock over the decode phase"},
             "prefill_tokens_per_s": round(B * prompt_len / (t1 - t0), 1),
             "prompt_len": prompt_len,
             "generated": gen_len,

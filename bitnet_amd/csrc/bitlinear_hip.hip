@@ -138,10 +138,15 @@ constexpr int kDecodeMaxTokens = 4;
 // entries sit in lanes 20*G + m (G = sigma), register q, and the four G parts are added at the end; the
 // off-diagonal entries are never read.  The problem's int8
 // activation rows are copied into LDS once per workgroup (requested before the weights, so that they
-// are not queued behind them: loads return in the order of their requests), with sum(a) per token
-// taken on the way (it removes the +2 of the stored codes); after that single barrier no wave waits
-// for another, and the only other LDS traffic is each wave's own 1 KB transposition of its diagonal
-// results.  Several problems of one shape (a grouped launch) are the grid's second dimension.
+// are not queued behind them: loads return in the order of their requests); after that single barrier
+// no wave waits for another, and the only other LDS traffic is each wave's own 1 KB transposition of
+// its diagonal results.  What stands between the arrival of the first weight words and their use is
+// time in which the wave's ring is not refilled, so the copy is all there is in front of the loop
+// (only the 16-byte pieces that exist are requested; measured per launch of 30 problems against a
+// prologue that also summed the rows: 3840 x 2560 14.9 -> 14.3 us, 2560 x 2560 11.3 -> 10.8): sum(a)
+// per token, which removes the +2 of the stored codes, is taken by every wave from the rows in LDS
+// behind the products of its first row block, when the ring is full again.
+// Several problems of one shape (a grouped launch) are the grid's second dimension.
 constexpr int kStreamMaxProblems = 48;  // the operands of a grouped launch travel as kernel arguments
 constexpr int kStreamMaxTokens = 4;
 constexpr int kStreamMaxActBytes = 32768;  // M * K: at most 8 16-byte pieces per thread of the staging pass
@@ -169,7 +174,6 @@ template <int D, bool COMPUTE>
 __global__ __launch_bounds__(256) void gemv_i2_stream_kernel(const StreamArgs a, uint32_t* __restrict__ sink) {
     extern __shared__ __attribute__((aligned(16))) int8_t lds_act[];  // [M][K + pad] + tail
     __shared__ __attribute__((aligned(16))) int red[4][256];         // per wave: [G][token][row]
-    __shared__ int wave_part[4][kStreamMaxTokens];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -210,7 +214,9 @@ __global__ __launch_bounds__(256) void gemv_i2_stream_kernel(const StreamArgs a,
             const int row = (pc >= kp16 ? 1 : 0) + (pc >= 2 * kp16 ? 1 : 0) + (pc >= 3 * kp16 ? 1 : 0);
             prow[i] = pc < a.M * kp16 ? row : -1;
             pdst[i] = row * kp + (pc - row * kp16) * 16;
-            piece[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, pc * 16, 0, 0));  // past the end: zeros
+            // a wave whose 64 pieces of this pass all lie past the block requests nothing (wave-uniform)
+            if ((wave * 64 + i * 256) < a.M * kp16)
+                piece[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, pc * 16, 0, 0));  // past the end: zeros
         }
         // (unconditional: a call without output hands in addresses that exist; a load under a branch would
         // be waited for inside the branch, in front of the weight requests)
@@ -229,29 +235,15 @@ __global__ __launch_bounds__(256) void gemv_i2_stream_kernel(const StreamArgs a,
     float e_sf = 1.0f;    // that token's activation scale
     uint32_t e_wsv = 0;   // lane j < nseg: weight scale of slot j, as fp32 bits
     if (COMPUTE) {
-        int part[kStreamMaxTokens] = {0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < kPieces; ++i) {
+        for (int i = 0; i < kPieces; ++i)
             if (prow[i] >= 0) *(v4i*)(lds_act + pdst[i]) = piece[i];
-            const int ones = 0x01010101;
-            int d = __builtin_amdgcn_sdot4(piece[i].x, ones, 0, false);
-            d = __builtin_amdgcn_sdot4(piece[i].y, ones, d, false);
-            d = __builtin_amdgcn_sdot4(piece[i].z, ones, d, false);
-            d = __builtin_amdgcn_sdot4(piece[i].w, ones, d, false);
-#pragma unroll
-            for (int m = 0; m < kStreamMaxTokens; ++m) part[m] += prow[i] == m ? d : 0;
-        }
-#pragma unroll
-        for (int m = 0; m < kStreamMaxTokens; ++m) {
-            const int tot = wave_sum_i32(part[m]);
-            if (lane == 0) wave_part[wave][m] = tot;
-        }
         e_sf = bf16_to_f32(e_sb);
         e_wsv = ((uint32_t)e_wb) << 16;
         lds_barrier();  // LDS only: the weight words stay in flight
-        rowsum2_tok = 2 * (wave_part[0][q] + wave_part[1][q] + wave_part[2][q] + wave_part[3][q]);
     }
     if (!have_items) return;  // behind the only barrier
+    bool rowsum_due = COMPUTE;
 
     const int8_t* bp = lds_act + tokB * kp + chunk * 16;
     uint32_t x_acc = 0;  // load-only variant: something that depends on every byte
@@ -299,6 +291,26 @@ __global__ __launch_bounds__(256) void gemv_i2_stream_kernel(const StreamArgs a,
             }
         }
         if (COMPUTE) {
+            if (rowsum_due) {
+                // once per wave: the sum of the lane's token's row, from the chunks the lane multiplies (chunk
+                // `chunk` of every 256-k step that lies inside K), added up over the 16 lanes of the token
+                rowsum_due = false;
+                const int ones = 0x01010101;
+                int rs = 0;
+                for (int st = 0; st < a.steps; ++st) {
+                    const v4i v = *(const v4i*)(bp + st * 256);
+                    int d = __builtin_amdgcn_sdot4(v.x, ones, 0, false);
+                    d = __builtin_amdgcn_sdot4(v.y, ones, d, false);
+                    d = __builtin_amdgcn_sdot4(v.z, ones, d, false);
+                    d = __builtin_amdgcn_sdot4(v.w, ones, d, false);
+                    rs += (st * 256 + chunk * 16) < a.K ? d : 0;
+                }
+                rs += dpp_move<0x124>(rs);  // row_ror:4 and :8: the four lanes of the 16-lane row with this token
+                rs += dpp_move<0x128>(rs);
+                rs += __shfl_xor(rs, 16);
+                rs += __shfl_xor(rs, 32);
+                rowsum2_tok = 2 * rs;
+            }
             // result lane 16 G + p' holds A-rows 4 G + r (r = register); the diagonal blocks (sigma' == G) sit in
             // the lanes with g == sg, token q; register r of MFMA i is weight row 4 r + i
             int* my = red[wave];
