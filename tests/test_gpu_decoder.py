@@ -546,10 +546,10 @@ def _rel_l2(a, b):
 
 @pytest.mark.parametrize("B", [1, 8])
 def test_full_size_decoder_graph_loop_equals_eager_loop(model_2b, B):
-    """512-token prompt, then 16 greedy steps: the graph-replayed loop and the
-    eager loop run the same kernels on the same data, so the tokens must be
-    identical; so must a second generation from the same prompt."""
-    P, G = 512, 16
+    """512-token prompt, then 128 generated tokens as the end-to-end workload names them (the first from the
+    prompt pass, 127 greedy steps): the graph-replayed loop and the eager loop run the same kernels on the same
+    data, so the tokens must be identical; so must a second generation from the same prompt."""
+    P, G = 512, 127
     dev = torch.device("cuda")
     g = torch.Generator(device="cuda").manual_seed(1234 + B)
     prompt = torch.randint(0, model_2b.args.vocab_size, (B, P), generator=g, device=dev)
