@@ -169,7 +169,9 @@ int bitlinear_repack(const int8_t* packed_ref, void* packed_out, int N, int K,
  * as above), product and epilogue.  While the activation block is small
  * (M * K <= 16384 elements) this is ONE kernel: every workgroup (or every wave
  * its own slice of k) quantizes x itself, keeps the int8 rows in LDS and never
- * reads s from memory.  Larger
+ * reads s from memory; five to eight tokens on rows of up to 3200 values
+ * (mode 0, at most 256 workgroups) are one kernel too: every lane quantizes
+ * for its own token, in registers.  Larger
  * blocks run the quantizer once, in a kernel of its own, and then the product
  * kernel (M <= 16: int8 rows staged in LDS per workgroup; M > 16: MFMA GEMM).
  *   q_ws (int8 [M, K], 16-byte aligned) and s_ws (bf16 [M]) receive the
