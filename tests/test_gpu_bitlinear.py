@@ -1122,8 +1122,8 @@ def test_forward_kernel_whose_waves_quantize_their_own_slices(n, k, m, shape, co
     _assert_bits_equal(host_bits(out4), want1, "mode 1")
 
 
-TOK_SHAPES = [(2560, 2560), (3840, 2560), (13824, 2560), (7008, 2560), (1040, 3200), (48, 192), (176, 4480), (64, 5120),
-              (2560, 6912)]
+TOK_SHAPES = [(2560, 2560), (3840, 2560), (13824, 2560), (13840, 2560), (7008, 2560), (1040, 3200), (48, 192), (176, 4480),
+              (64, 5120), (2560, 6912)]
 
 
 @pytest.mark.parametrize("m", [1, 2, 5, 7, 8, 9])
@@ -1131,8 +1131,8 @@ TOK_SHAPES = [(2560, 2560), (3840, 2560), (13824, 2560), (7008, 2560), (1040, 32
 def test_forward_kernel_whose_lanes_quantize_for_their_own_token(n, k, m):
     """bitlinear_solo_tok_kernel (one launch for up to eight tokens; the library's choice from five tokens on for
     rows of up to 3200 values): int32 accumulators, bf16 outputs and the q / s workspaces bit for bit against the
-    oracle chain, with and without workspaces, over 1 and 4 row blocks per wave, one to sixteen waves, K that
-    the waves do not divide, three scale slots; where the kernel has no launch shape (nine tokens, K = 6912, 7008
+    oracle chain, with and without workspaces, over 1 and 4 row blocks per wave (13840 rows: a last workgroup with
+    one row block of its four), one to sixteen waves, K that the waves do not divide, three scale slots; where the kernel has no launch shape (nine tokens, K = 6912, 7008
     rows) the other kernels give the same."""
     lib = _lib.load_library()
     rng = np.random.default_rng(n + 3 * k + m)
