@@ -926,7 +926,6 @@ void gemm_i2_prefill_kernel(
 //  * with the interleaved column tiles a lane's accumulators of one register quad are 4 * NT consecutive output
 //    columns: 16-byte (NT = 2) or 32-byte stores per token instead of 8.
 // K must be a multiple of CK.
-constexpr int kPfxWaves = 4;
 template <int NT>
 struct PfxWords;
 template <>
@@ -942,12 +941,14 @@ __device__ __forceinline__ void load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, int8_
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)ldsp, 16, voff, soff, 0, 0);
 }
 
-template <int MT, int NT, int CK>
-__global__ __launch_bounds__(kPfxWaves * 64) __attribute__((amdgpu_waves_per_eu(MT * NT <= 4 ? 3 : 2)))
-void gemm_i2_prefill_dma_kernel(
-    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int nunits, int cseg_shift,
-    int band, int seg_cols, const uint16_t* __restrict__ s, uint16_t* __restrict__ out, int32_t* __restrict__ acc_out,
-    const uint16_t* __restrict__ ws, ScaleMap smap, const uint16_t* __restrict__ residual) {
+// One output tile of (32 MT) rows x (WAVES x 32 NT) columns at (row_tile, column n_base) by the WAVES waves of the
+// calling workgroup (further waves of the workgroup must not enter).
+template <int MT, int NT, int CK, int WAVES>
+__device__ __forceinline__ void pfx_tile(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int row_tile, int n_base, bool has_out,
+    const uint16_t* __restrict__ s, uint16_t* __restrict__ out, int32_t* __restrict__ acc_out,
+    const uint16_t* __restrict__ ws, const ScaleMap& smap, const uint16_t* __restrict__ residual) {
+    constexpr int kPfxWaves = WAVES;
     constexpr int TM = MT * 32;
     constexpr int KSTEPS = CK / 32;
     constexpr int PPR = CK / 16;             // 16-byte pieces per row and chunk
@@ -962,18 +963,8 @@ void gemm_i2_prefill_dma_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // workgroup -> tile: as gemm_i2_prefill_kernel (bands of row tiles per XCD, column segments)
-    const int row_tiles = (M + TM - 1) / TM;
-    const int col_tiles = (N + kPfxWaves * NT * 32 - 1) / (kPfxWaves * NT * 32);
-    const int unit = (blockIdx.x & 7) + 8 * blockIdx.z;
-    if (unit >= nunits) return;
-    const bool has_out = (cseg_shift >> 8) != 0;
-    cseg_shift &= 0xff;
-    const int col_tile = (unit & ((1 << cseg_shift) - 1)) * seg_cols + blockIdx.y;
-    const int row_tile = (unit >> cseg_shift) * band + (blockIdx.x >> 3);
-    if (row_tile >= row_tiles || col_tile >= col_tiles) return;
     const int m0 = row_tile * TM;
-    const int n0 = (col_tile * kPfxWaves + wave) * NT * 32;
+    const int n0 = n_base + wave * NT * 32;
     const int nl = lane & 31;
     const int kc = lane >> 5;
     const int nchunks = K / CK;
@@ -1162,6 +1153,62 @@ void gemm_i2_prefill_dma_kernel(
                 }
             }
         }
+    }
+}
+
+constexpr int kPfxWaves = 4;
+template <int MT, int NT, int CK>
+__global__ __launch_bounds__(kPfxWaves * 64) __attribute__((amdgpu_waves_per_eu(MT * NT <= 4 ? 3 : 2)))
+void gemm_i2_prefill_dma_kernel(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int nunits, int cseg_shift,
+    int band, int seg_cols, const uint16_t* __restrict__ s, uint16_t* __restrict__ out, int32_t* __restrict__ acc_out,
+    const uint16_t* __restrict__ ws, ScaleMap smap, const uint16_t* __restrict__ residual) {
+    // workgroup -> tile: as gemm_i2_prefill_kernel (bands of row tiles per XCD, column segments)
+    const int row_tiles = (M + MT * 32 - 1) / (MT * 32);
+    const int col_tiles = (N + kPfxWaves * NT * 32 - 1) / (kPfxWaves * NT * 32);
+    const int unit = (blockIdx.x & 7) + 8 * blockIdx.z;
+    if (unit >= nunits) return;
+    const bool has_out = (cseg_shift >> 8) != 0;
+    cseg_shift &= 0xff;
+    const int col_tile = (unit & ((1 << cseg_shift) - 1)) * seg_cols + blockIdx.y;
+    const int row_tile = (unit >> cseg_shift) * band + (blockIdx.x >> 3);
+    if (row_tile >= row_tiles || col_tile >= col_tiles) return;
+    pfx_tile<MT, NT, CK, kPfxWaves>(act, wq, M, N, K, row_tile, col_tile * (kPfxWaves * NT * 32), has_out, s, out, acc_out, ws, smap,
+                                    residual);
+}
+
+// The same tiles in two sizes from one launch, for output shapes that leave a little more than one 64 x 256 tile per CU
+// (2048 x 2560: 320 tiles on 256 CUs -- a quarter of the CUs with two tiles, or three half-height tiles on half of them):
+// the first big_cols column tiles of 256 go to workgroups that take a 64 x 256 tile each, the columns behind them to
+// workgroups of which two waves take a 32 x 128 tile (a quarter of the work; the other two waves leave at once), so that
+// a CU holds one tile of each kind.  Workgroup w of a kind -> XCD w % 8 -> a band of row tiles of its own.
+template <int CK>
+__global__ __launch_bounds__(kPfxWaves * 64) __attribute__((amdgpu_waves_per_eu(3)))
+void gemm_i2_prefill_mix_kernel(
+    const int8_t* __restrict__ act, const uint32_t* __restrict__ wq, int M, int N, int K, int nbig, int big_cols, int flags,
+    int small_cols, const uint16_t* __restrict__ s, uint16_t* __restrict__ out, int32_t* __restrict__ acc_out,
+    const uint16_t* __restrict__ ws, ScaleMap smap, const uint16_t* __restrict__ residual) {
+    const bool has_out = (flags & 1) != 0;
+    const int w = blockIdx.x;
+    if (w < nbig) {
+        // 64-row tiles: XCD x takes a band of row tiles x * band .. and walks the columns (nbig = 8 * band * big_cols)
+        const int rt = (M + 63) >> 6;
+        const int band = (rt + 7) >> 3;
+        const int j = w >> 3;
+        const int row_tile = (w & 7) * band + j % band;
+        const int col_tile = j / band;
+        if (row_tile >= rt) return;  // a ragged last band
+        pfx_tile<2, 2, CK, 4>(act, wq, M, N, K, row_tile, col_tile * 256, has_out, s, out, acc_out, ws, smap, residual);
+    } else {
+        if (threadIdx.x >= 128) return;
+        const int v = w - nbig;
+        const int rt = (M + 31) >> 5;
+        const int band = (rt + 7) >> 3;  // 32-row tiles per XCD
+        const int j = v >> 3;
+        const int row_tile = (v & 7) * band + j % band;
+        const int col_tile = j / band;
+        if (row_tile >= rt || col_tile >= small_cols) return;
+        pfx_tile<1, 2, CK, 2>(act, wq, M, N, K, row_tile, big_cols * 256 + col_tile * 128, has_out, s, out, acc_out, ws, smap, residual);
     }
 }
 
@@ -2458,6 +2505,10 @@ constexpr int kPrefillOnePerCuMin = 128, kPrefillOnePerCuMax = 256;
 // a little more than one round of 64 x 256 tiles (three per CU): one round of 128 x 256 tiles (two per CU) instead
 // (13824 x 2560 at M = 1024: 864 tiles, 46.5 -> 42.3 us)
 constexpr int kPrefillRound64 = 768, kPrefillRound128 = 1024;
+// gemm_i2_prefill_mix_kernel: CUs a round of 64 x 256 tiles is sized for, and the most 32 x 128 tiles behind the whole
+// rounds for which the launch with two tile sizes is taken (about 1.4 per CU; figures at launch_prefill)
+constexpr int kPrefillMixCus = 256;
+constexpr int kPrefillMixMaxQuarters = 360;
 }  // namespace dispatch
 using namespace dispatch;
 
@@ -3058,6 +3109,36 @@ int launch_prefill(const int8_t* act, const int8_t* packed, uint16_t* out, int32
     // weight words of two column tiles with one request (a layer's four GEMMs at M = 2048: 1.72 -> 1.92 POP/s on
     // uniform random int8; 13824 x 2560 73.3 -> 64.8 us, 2560 x 6912 46.3 -> 42.2, at M = 4096 1.97 -> 2.20),
     // given 128-k chunks that divide K and 16-byte aligned rows
+    // one launch with tiles of two sizes (see gemm_i2_prefill_mix_kernel): whole rounds of one 64 x 256 tile per CU over the
+    // first columns, the columns behind them as 32 x 128 tiles.  Taken when those quarter tiles are at most about 1.4
+    // per CU (measured, 64 x 256 tiles or half-height ones -> this: 2560 x 2560 at M = 2048 19.0 -> 17.3 us, at M = 3584
+    // 28.5 -> 25.9, at 5120 39.4 -> 36.1; 2560 x 6912 41.0 -> 36.5 / 62.7 -> 57.3 / 91.4 -> 82.0; 3200 x 3200 at M = 1536
+    // 22.4 -> 20.1, 2560 33.0 -> 28.5, 5120 58.0 -> 49.9; with more of them the even tiles are ahead: 2560 x 2560 at
+    // M = 2560 21.3 against 26.5, 3840 x 2560 at M = 2048 22.8 against 28.0)
+    if (dma_fits && (t_tune.path == 0 || (t_tune.path == 5 && t_tune.prefill_big == 8))) {
+        const int rt64 = (M + 63) / 64, rt32 = (M + 31) / 32;
+        const int band64 = (rt64 + 7) / 8, band32 = (rt32 + 7) / 8;
+        const long long wide = (long long)((N + 255) / 256) * rt64;
+        const int rounds = wide / kPrefillMixCus > 1 ? (int)(wide / kPrefillMixCus) : 1;
+        int big_cols = (int)((long long)kPrefillMixCus * rounds / rt64);
+        if (big_cols > N / 256) big_cols = N / 256;
+        const int small_cols = (N - big_cols * 256 + 127) / 128;
+        const long long quarters = (long long)rt32 * small_cols;
+        const bool wanted = t_tune.path == 5 || (wide > kPrefillMixCus && big_cols >= 1 && quarters > 0 && quarters <= kPrefillMixMaxQuarters);
+        const long long groups = 8ll * band64 * big_cols + 8ll * band32 * small_cols;
+        if (wanted && rt64 <= 4096 && groups < (1ll << 30)) {
+            const int nbig = 8 * band64 * big_cols;
+            const dim3 mgrid((unsigned)groups, 1, 1), mblock(256, 1, 1);
+            g_last_kernel = "gemm_i2_prefill_mix_kernel";
+            if (K % 256 == 0)
+                BL_LAUNCH((gemm_i2_prefill_mix_kernel<256>), mgrid, mblock, 3 * 64 * 256, stream, act, wq, M, N, K, nbig, big_cols,
+                          out ? 1 : 0, small_cols, s, out, acc_out, ws, smap, residual);
+            else
+                BL_LAUNCH((gemm_i2_prefill_mix_kernel<128>), mgrid, mblock, 3 * 64 * 128, stream, act, wq, M, N, K, nbig, big_cols,
+                          out ? 1 : 0, small_cols, s, out, acc_out, ws, smap, residual);
+            return launch_status();
+        }
+    }
     bool dma = true;
     int dma_mt = 2;  // row tiles of 32 tokens per workgroup of that kernel: 64 x 256, or 32 x 256 / 128 x 256 when forced
     if (t_tune.path == 5) {
@@ -3556,7 +3637,7 @@ int bitlinear_set_tuning(int kernel, int a, int b, int c) {
         return set_status(BITLINEAR_OK);
     }
     if (kernel == 5) {
-        if (a < 0 || a > 7 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
+        if (a < 0 || a > 8 || b < 0 || b > 64 || (c != 0 && c != 1 && c != 2 && c != 4)) return set_status(BITLINEAR_ERR_ARG);
         g.path = 5;
         g.prefill_big = a;
         g.prefill_band = b;

@@ -302,7 +302,10 @@ int bitlinear_plan_name(int entry, int M, int N, int K, char* buf, int buflen);
  *             chunks straight into LDS (the built-in choice for that tile when
  *             K % 128 == 0; a = 2 forces the other kernel), 6 = 32 x 256 and
  *             7 = 128 x 256 through that kernel (without K % 128 == 0: 32 x 128 and
- *             128 x 256 through the other); b = row tiles per band of the tile order (0 = the
+ *             128 x 256 through the other), 8 = whole rounds of 64 x 256 tiles over
+ *             the first columns and 32 x 128 tiles behind them in one launch (the
+ *             built-in choice when those are at most about 1.4 per CU; needs
+ *             K % 128 == 0); b = row tiles per band of the tile order (0 = the
  *             library's choice, up to 64); c = groups of four waves that split a
  *             tile's K between them (0 = the library's choice, 1, 2 (tiles 0 and 4)
  *             or 4 (tile 4))

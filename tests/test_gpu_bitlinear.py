@@ -576,6 +576,38 @@ def test_prefill_gemm_through_the_direct_to_lds_kernel(m, n, k):
     _assert_bits_equal(host_bits(out_seg), want_seg, f"direct-to-LDS GEMM, segments {ends}")
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 2560, 256), (1000, 4368, 384), (500, 8448, 1280), (2017, 2560, 512), (1024, 4112, 2560),
+                                   (2100, 2560, 384), (40, 272, 128)])
+def test_prefill_gemm_with_tiles_of_two_sizes_in_one_launch(m, n, k):
+    """gemm_i2_prefill_mix_kernel: 64 x 256 tiles on the first columns and 32 x 128 tiles (two waves of a workgroup)
+    behind them, one launch: all columns in big tiles; a ragged rest of 272 and of 16 columns; ragged M; row tile
+    counts that the eight bands do not divide; fewer row tiles than bands; one to ten chunks of 128 or 256 k.
+    Accumulators and outputs (equal slots, and segments cutting through a register quad) equal to the oracle's bit
+    for bit; M = 2048 at N = 2560 is where the library takes it by itself."""
+    assert _lib.plan_name(0, 2048, 2560, 2560).startswith("gemm_i2_prefill_mix_kernel<256> grid=(512,1,1)")
+    lib = _lib.load_library()
+    w, a = _rand_case(n, k, m, seed=m + n + k)
+    s_bits = o.f32_to_bf16_bits(np.linspace(3.0, 90.0, m).astype(np.float32))
+    ws_bits = o.f32_to_bf16_bits(np.array([0.0161, 0.0247, 0.0093, 0.0], dtype=np.float32))
+    acc_want, want = o.bitlinear_int8xint2(a, w, s_bits, ws_bits)
+    ends = [20, n // 2 + 4, n]
+    _, want_seg = o.bitlinear_int8xint2_seg(a, w, s_bits, ws_bits, ends)
+    ad, pk, sd, wsd = dev_i8(a), _packed_dev(w), dev_bf16(s_bits), dev_bf16(ws_bits)
+    try:
+        assert lib.bitlinear_set_tuning(5, 8, 0, 0) == 0
+        acc = bitlinear.bitnet_int8xint2_acc(ad, pk)
+        name = bitlinear.last_kernel()
+        out = bitlinear.bitnet_int8xint2_linear(ad, pk, sd, wsd)
+        out_seg = bitlinear.bitnet_int8xint2_linear_seg(ad, pk, sd, wsd, ends)
+        torch.cuda.synchronize()
+    finally:
+        lib.bitlinear_set_tuning(0, 0, 0, 0)
+    assert name == "gemm_i2_prefill_mix_kernel"
+    assert np.array_equal(acc.cpu().numpy(), acc_want)
+    _assert_bits_equal(host_bits(out), want, "tiles of two sizes")
+    _assert_bits_equal(host_bits(out_seg), want_seg, f"tiles of two sizes, segments {ends}")
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("m,n,k", [(17, 48, 192), (64, 128, 64), (100, 272, 320), (128, 2560, 2560), (129, 3840, 2560),
                                    (300, 1040, 3200), (512, 2560, 6912)])
@@ -652,7 +684,7 @@ def test_prefill_scaled_output_with_outliers(shape_id, m):
     mod.weight.data = _packed_dev(w)
     mod.weight_scale.data = dev_bf16(ws_bits)
     out = mod(dev_bf16(xb))
-    assert bitlinear.last_kernel() in ("gemm_i2_prefill_kernel", "gemm_i2_prefill_dma_kernel")
+    assert bitlinear.last_kernel() in ("gemm_i2_prefill_kernel", "gemm_i2_prefill_dma_kernel", "gemm_i2_prefill_mix_kernel")
     _assert_bits_equal(host_bits(out), want, f"{sh.name} prefill M={m}")
     qd, sd = mod.quant_input(dev_bf16(xb))
     assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(host_bits(sd).reshape(-1), s_bits)
@@ -861,15 +893,15 @@ def test_norm_forward_without_workspaces_and_beyond_decode_sizes():
     assert st != 0
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4, 5, 8])
 @pytest.mark.parametrize("m,n,k,glu", [(40, 2560, 2560, 0), (130, 3840, 2560, 0), (300, 2560, 6912, 1), (77, 48, 192, 1),
                                        (513, 1040, 640, 0), (1030, 64, 2560, 0), (1025, 272, 640, 0), (1024, 48, 4096, 0),
                                        (1026, 32, 6912, 1)])  # from 1024 rows on without the gate: a wave per row
 def test_norm_forward_with_residual_beyond_decode_sizes(m, n, k, glu, tile):
     """Prompt-sized blocks: gate / norm / quantizer kernel, then the product with
     the residual added in its epilogue -- through the library's own choice of
-    product kernel (tile -1: split-K or GEMM) and through every GEMM tile --
-    against the oracle chain, bit for bit."""
+    product kernel (tile -1: split-K or GEMM), through every GEMM tile and through the launch with tiles of two
+    sizes (8) -- against the oracle chain, bit for bit."""
     import ctypes
 
     lib = _lib.load_library()
