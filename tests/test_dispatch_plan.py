@@ -33,6 +33,10 @@ def test_plan_rows_say_what_the_design_says():
     two = p(1, 16, 3840, 2560).split(" + ")
     assert len(two) == 2 and two[0].startswith("quant_absmax_rows_kernel<0, 5>") and two[1].startswith("gemv_i2_solo_kernel<5, 1, false>")
     assert "gemm_i2_prefill_kernel" in p(0, 17, 13824, 2560) and "gemm_i2_prefill_dma_kernel<2, 2, 256>" in p(0, 2048, 13824, 2560)
+    # 2048 x 2560 outputs are 320 tiles of 64 x 256: one round of the machine plus a quarter -> tiles of two sizes in one
+    # launch (256 + 256 workgroups); 2560 x 2560 outputs (400 tiles) leave too large a rest for that
+    assert p(0, 2048, 2560, 6912).startswith("gemm_i2_prefill_mix_kernel<256> grid=(512,1,1) block=256")
+    assert "gemm_i2_prefill_mix_kernel" not in p(0, 2560, 2560, 2560) and "gemm_i2_prefill_mix_kernel" not in p(0, 2048, 3840, 2560)
     assert p(0, 1, 55296, 5120).startswith("gemv_i2_stream_kernel<5, true>")
     assert p(0, 1, 20480, 3200).startswith("bitlinear_fused_kernel<")
 
