@@ -66,7 +66,7 @@ int bitnet_decode_step_begin(const int64_t* tokens, const int64_t* positions, co
  * bitnet_attn_decode with the rotation values of every sequence's position handed over as ready
  * rows (rope_rows float [B, head_dim], as bitnet_decode_step_begin writes them; they must be the
  * tables' rows at positions[b]): results are identical, the kernel saves the memory round trip of
- * the table lookup behind the position.  With kernel 1 selected the rows are ignored.
+ * the table lookup behind the position.
  */
 int bitnet_attn_decode_rows(const uint16_t* qkv, uint16_t* cache_k, uint16_t* cache_v,
                             const int64_t* positions, const float* cos_table,
