@@ -765,6 +765,16 @@ def test_generate_all_stops_at_the_end_token_and_trims_the_answers():
             want = want[: want.index(eos) + 1]
         assert a == want
     assert cut[1][-1] == eos or eos in cut[0]
+    # the end token as the very first token of sequence 0 (out of the prompt pass): that sequence's answer is the end
+    # token alone, the other sequence goes on as if nothing had happened, until a decode step produces the token
+    eos0 = full[0][0]
+    cut0 = gen.generate_all(prompts, 16, eos_id=eos0)
+    assert cut0[0] == [eos0]
+    hit = min([a.index(eos0, 1) for a in full if eos0 in a[1:]] + [15])
+    want1 = full[1][: hit + 1]
+    if eos0 in want1:
+        want1 = want1[: want1.index(eos0) + 1]
+    assert cut0[1] == want1 and len(cut0[1]) > 1
 
 
 def test_generate_all_sampling_is_reproducible_and_greedy_for_a_tiny_nucleus():
