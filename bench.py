@@ -361,7 +361,7 @@ def batched_and_prefill(lib, shapes, layers, scales, dev, decode_ms=(2, 4, 8, 16
             "layer_gemm_TOPS": round(tops, 1),
             "layer_forward_TOPS": round(tot_ops / (tot_fwd_us * 1e-6) / 1e12, 1),
             "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": round(tops / INT8_MFMA_PEAK_TOPS, 4), "kernel": "gemm_i2_prefill_dma_kernel (gemm_i2_prefill_kernel where K % 128 != 0), the four 2B shapes of one layer"},
+                         "frac": round(tops / INT8_MFMA_PEAK_TOPS, 4), "kernel": "gemm_i2_prefill_dma_kernel and gemm_i2_prefill_mix_kernel (gemm_i2_prefill_kernel for the small tiles with k-groups), the four 2B shapes of one layer"},
             "prefill_tokens_per_s_bitlinear_only": round(M / (tot_fwd_us * 1e-6 * len(layers)), 1),
         }
     return out
